@@ -1,0 +1,164 @@
+/*
+ * C ABI of libvkllama_hip.so: the HIP/gfx950 layer that replaces the
+ * reference's Vulkan device, command-buffer, pipeline and shader layer
+ * (src/core/gpu_device.*, src/core/command.h, src/core/pipeline.*,
+ * every compute shader under src/shaders/).  The C++ operator classes in vkllama_amd/src/ops call
+ * nothing else.
+ *
+ * Conventions
+ *  - every function returns 0 on success or a hipError_t value;
+ *    vkl_error_string() turns it into text.  Shape violations return
+ *    hipErrorInvalidValue (1) before anything is launched.
+ *  - pointers are device pointers unless the name ends in _h.
+ *  - `stream` is a hipStream_t passed as void*; launches are asynchronous.
+ *  - fp16 data is IEEE binary16 (uint16_t bit patterns on the host side).
+ *  - strides are in ELEMENTS, not bytes.
+ *  - Q8_0 tensors live on the device in the PLANAR layout: for a matrix of
+ *    `rows` rows and K columns, nb = ceil(K/32):
+ *        int8  q[rows][nb*32]   at byte offset 0
+ *        fp16  d[rows][nb]      at byte offset rows*nb*32
+ *    (34*nb bytes per row in total, the same count as the GGUF block layout
+ *    { fp16 d; int8 q[32]; } of src/shaders/common.h:8-10).  vkl_q8_0_pack /
+ *    vkl_q8_0_unpack convert between the two on the device.
+ */
+#ifndef VKL_HIP_H
+#define VKL_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- device, streams, memory: replaces src/core/gpu_device.h:13-37 and the
+ * submit/wait/upload/download half of src/core/command.h:26-483 ---------- */
+typedef struct
+{
+  int device;
+  int compute_units;
+  int wavefront_size;
+  int max_lds_bytes;
+  size_t total_mem;
+  char name[128];
+  char arch[64];
+} vkl_device_info;
+
+int vkl_device_count (int *n);
+int vkl_device_open (int dev, vkl_device_info *info);
+const char *vkl_error_string (int err);
+int vkl_stream_create (void **stream);
+int vkl_stream_destroy (void *stream);
+int vkl_stream_sync (void *stream);
+int vkl_device_sync (void);
+int vkl_malloc (void **p, size_t bytes);
+int vkl_free (void *p);
+int vkl_host_malloc_h (void **p, size_t bytes); /* pinned */
+int vkl_host_free_h (void *p);
+int vkl_memcpy_h2d (void *dst, const void *src_h, size_t bytes, void *stream);
+int vkl_memcpy_d2h (void *dst_h, const void *src, size_t bytes, void *stream);
+int vkl_memcpy_d2d (void *dst, const void *src, size_t bytes, void *stream);
+int vkl_memset (void *dst, int value, size_t bytes, void *stream);
+/* timing: replaces the timestamp queries of src/core/pipeline.cpp:425-445 */
+int vkl_event_create (void **ev);
+int vkl_event_destroy (void *ev);
+int vkl_event_record (void *ev, void *stream);
+int vkl_event_sync (void *ev);
+int vkl_event_elapsed_ms (void *start, void *stop, float *ms);
+
+/* ---- Q8_0: src/core/quants.h:35-139 ------------------------------------ */
+/* host quantiser, 34-byte blocks, fp16 (RNE) scale */
+void vkl_quantize_q8_0_h (const float *src_h, size_t n, uint8_t *dst_h);
+void vkl_dequantize_q8_0_h (const uint8_t *src_h, size_t n, float *dst_h);
+size_t vkl_q8_0_row_bytes (size_t K);
+/* GGUF 34-byte blocks (device) <-> planar (device) */
+int vkl_q8_0_pack (const void *raw, void *planar, size_t rows, size_t K,
+                   void *stream);
+int vkl_q8_0_unpack (const void *planar, void *raw, size_t rows, size_t K,
+                     void *stream);
+
+/* ---- operators -------------------------------------------------------- */
+/* src/ops/embedding.cpp:58-114, src/shaders/embedding_q8_0.comp,
+ * embedding_fp16.comp.  toks: device uint32 [n]; out fp16 [n, VW]. */
+int vkl_embed_q8_0 (const void *table_planar, uint32_t VH, uint32_t VW,
+                    const uint32_t *toks, uint32_t n, uint32_t unk, void *out,
+                    void *stream);
+int vkl_embed_f16 (const void *table, uint32_t VH, uint32_t VW,
+                   const uint32_t *toks, uint32_t n, uint32_t unk, void *out,
+                   void *stream);
+/* src/ops/rms_norm.cpp:60-91, src/shaders/rms_norm_fp16.comp */
+int vkl_rmsnorm_f16 (const void *x, const float *w, int rows, int W,
+                     float eps, void *out, void *stream);
+/* src/ops/mat_mul.cpp:159-228 with FP16 x Q8_0, transpose_b:
+ * src/shaders/matmul_b0_fp16_x_q8_0.comp.  y[m,n] = act(scale * sum_k
+ * x[m,k] W[n,k] + bias), act 1 = SiLU.  x [M,K] row stride xs; y [M,N] row
+ * stride ys.  If residual != NULL: y = fp16(fp32(fp16(v)) + residual[m,n])
+ * (the ElementWise add of models/llama2.h:193-196,209 folded in); residual may
+ * alias y.  If y32 != NULL the fp16 result is also widened to fp32 there
+ * (the Cast of models/llama2.h:294). */
+int vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N,
+                     int K, size_t xs, size_t ys, float scale, float bias,
+                     int act, const void *residual, void *y, float *y32,
+                     void *stream);
+/* src/ops/multiheadattention_v2.cpp:190-202, src/shaders/kqv_fp16_x_q8_0.comp */
+int vkl_kqv_q8_0 (const void *x, const void *wk, const void *wq,
+                  const void *wv, int M, int N, int K, void *k, void *q,
+                  void *v, void *stream);
+/* src/ops/feed_forward.cpp:106-120, src/shaders/ffn_up_and_gate_q8_0.comp:
+ * out = fp16(silu(x Wgate^T) * (x Wup^T)) */
+int vkl_ffn_upgate_q8_0 (const void *x, const void *wup, const void *wgate,
+                         int M, int N, int K, void *out, void *stream);
+/* src/shaders/matmul_b0_tb_fp16_v2.comp: Y[c,m,n] = act(scale * sum_k
+ * A[c,m,k] B[c,n,k] + bias); A strides (acs, ahs), B (bcs, bhs), Y (ycs, yhs).
+ * residual / y32 as for vkl_matmul_q8_0 (dense [C*M, N]). */
+int vkl_matmul_f16_tb (const void *a, const void *b, int C, int M, int N,
+                       int K, size_t acs, size_t ahs, size_t bcs, size_t bhs,
+                       size_t ycs, size_t yhs, float scale, float bias,
+                       int act, const void *residual, void *y, float *y32,
+                       void *stream);
+/* src/shaders/matmul_broadcast0_fp16_v2.comp, transpose_b = 0:
+ * Y[c,m,n] = act(scale * sum_k A[c,m,k] B[c,k,n] + bias) */
+int vkl_matmul_f16_nn (const void *a, const void *b, int C, int M, int N,
+                       int K, size_t acs, size_t ahs, size_t bcs, size_t bhs,
+                       size_t ycs, size_t yhs, float scale, float bias,
+                       int act, void *y, void *stream);
+/* src/shaders/ffn_up_and_gate_fp16.comp */
+int vkl_ffn_upgate_f16 (const void *x, const void *wup, const void *wgate,
+                        int M, int N, int K, void *out, void *stream);
+/* src/ops/rope.cpp:112-150, src/shaders/rope_fp16.comp: in place on x
+ * [C,H,W]; tables fp32 [rows, W/2]; row y uses table row y + offset. */
+int vkl_rope_f16 (void *x, int C, int H, int W, const float *freqc,
+                  const float *freqs, uint32_t offset, void *stream);
+/* src/ops/update_kv_cache.cpp:36-76, src/shaders/update_kvcache_fp16.comp:
+ * cache[c, (offset+y) % HO, :] = kv[c, y, :] */
+int vkl_kv_update_f16 (void *cache, const void *kv, int C, int HO, int H,
+                       int W, uint32_t offset, void *stream);
+/* src/ops/softmax.cpp:52-92, src/shaders/softmax_fp16.comp */
+int vkl_softmax_f16 (const void *x, int C, int H, int W, int seq_mask,
+                     uint32_t offset, void *out, void *stream);
+/* src/ops/elementwise.cpp:60-101, src/shaders/element_wise_fp16.comp:
+ * y = fp16(x op y), in place into y; op 0..3 = add, sub, mul, div */
+int vkl_elementwise_f16 (const void *x, void *y, size_t n, int op,
+                         void *stream);
+/* src/ops/elementwise.cpp:104-133, element_wise_constant_fp16.comp:
+ * out = fp16(x op alpha) */
+int vkl_elementwise_const_f16 (const void *x, float alpha, size_t n, int op,
+                               void *out, void *stream);
+/* src/ops/cast.cpp:40-77 */
+int vkl_cast_f16_f32 (const void *x, float *out, size_t n, void *stream);
+int vkl_cast_f32_f16 (const float *x, void *out, size_t n, void *stream);
+/* src/ops/argop.h:72-140, argmax_stage0_fp16.comp + argmax_stage1.comp:
+ * first index of the maximum (op 0) / minimum (op 1) of each row */
+int vkl_argop_f16 (const void *x, int rows, int W, int op, uint32_t *out,
+                   void *stream);
+/* src/ops/slice.cpp:30-77, src/shaders/slice_fp16.comp */
+int vkl_slice_f16 (const void *x, int C, int H, int W, int c0, int h0, int w0,
+                   int CE, int HE, int WE, void *out, void *stream);
+/* src/ops/transpose.cpp:36-80 type 0, transpose_type0_fp16.comp:
+ * [C,H,W] -> [H,C,W] */
+int vkl_transpose102_f16 (const void *x, int C, int H, int W, void *out,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,26 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "slow: long-running case")
+
+
+@pytest.fixture(scope="session")
+def dev():
+    """One opened GPU + stream for the whole session (GPU tests only)."""
+    from vkllama_amd import capi
+    return capi.Device(0)
+
+
+@pytest.fixture
+def rng():
+    return np.random.default_rng(1234)

@@ -1,0 +1,301 @@
+"""Parity of every HIP operator kernel with the CPU oracle, through the C ABI.
+
+Bars (BASELINE north star): bit-exact for Q8_0 repacking, embedding gather,
+KV-cache writes, arg-max ids and plain copies; fp16 outputs within 1e-2
+relative of the oracle (measured against max(|ref|, 1e-2 max|ref|)).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from util import q8_weights, rel_err, ulp_diff_f16
+from vkllama_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+F16_REL_TOL = 1e-2
+
+
+def L():
+    return capi.lib()
+
+
+def f16(buf, shape):
+    return buf.read(np.uint16, shape).view(np.float16)
+
+
+# ------------------------------------------------------------------ Q8_0 ----
+@pytest.mark.parametrize("rows,K", [(5, 32), (64, 1376), (33, 4096), (7, 100)])
+def test_q8_pack_unpack_roundtrip_bit_exact(dev, rng, rows, K):
+    raw, _ = q8_weights(rng, rows, K)
+    nb = (K + 31) // 32
+    staging = dev.upload(raw)
+    planar = dev.alloc(raw.nbytes)
+    back = dev.alloc(raw.nbytes)
+    capi.check(L().vkl_q8_0_pack(staging.ptr, planar.ptr, rows, K, dev.stream))
+    capi.check(L().vkl_q8_0_unpack(planar.ptr, back.ptr, rows, K, dev.stream))
+    p = planar.read(np.uint8, raw.nbytes)
+    blocks = raw.reshape(rows * nb, 34)
+    assert np.array_equal(p[:rows * nb * 32].reshape(-1, 32), blocks[:, 2:])      # int8 plane
+    assert np.array_equal(p[rows * nb * 32:].reshape(-1, 2), blocks[:, :2])       # scale plane
+    assert np.array_equal(back.read(np.uint8, raw.shape), raw)
+
+
+# -------------------------------------------------------------- embedding ---
+def test_embedding_q8_bit_exact(dev, rng):
+    V, W = 300, 512
+    raw, _ = q8_weights(rng, V, W)
+    toks = np.array([0, 299, 7, 300, 2 ** 31 + 5, 7, 128], np.uint32)
+    table = dev.upload_q8_0(raw, V, W)
+    dt = dev.upload(toks)
+    out = dev.alloc(toks.size * W * 2)
+    capi.check(L().vkl_embed_q8_0(table.ptr, V, W, dt.ptr, toks.size, 0, out.ptr, dev.stream))
+    want = O.embedding_q8_0(raw, W, toks, 0)
+    assert np.array_equal(f16(out, want.shape).view(np.uint16), want.view(np.uint16))
+
+
+def test_embedding_f16_bit_exact(dev, rng):
+    V, W = 100, 200
+    table = rng.standard_normal((V, W)).astype(np.float16)
+    toks = np.array([3, 99, 100, 0], np.uint32)
+    dtab, dt = dev.upload(table), dev.upload(toks)
+    out = dev.alloc(toks.size * W * 2)
+    capi.check(L().vkl_embed_f16(dtab.ptr, V, W, dt.ptr, toks.size, 5, out.ptr, dev.stream))
+    assert np.array_equal(f16(out, (4, W)), O.embedding_f16(table, toks, 5))
+
+
+# ----------------------------------------------------------------- RMSNorm --
+@pytest.mark.parametrize("rows,W", [(1, 4096), (16, 512), (3, 1000), (2, 5120)])
+def test_rmsnorm(dev, rng, rows, W):
+    x = (rng.standard_normal((rows, W)) * 2).astype(np.float16)
+    w = rng.uniform(0.5, 1.5, W).astype(np.float32)
+    dx, dw = dev.upload(x), dev.upload(w)
+    out = dev.alloc(x.nbytes)
+    capi.check(L().vkl_rmsnorm_f16(dx.ptr, dw.ptr, rows, W, 1e-5, out.ptr, dev.stream))
+    got, want = f16(out, x.shape), O.rmsnorm(x, w, 1e-5)
+    assert ulp_diff_f16(got, want).max() <= 1
+    assert rel_err(got, want) < F16_REL_TOL
+
+
+# ------------------------------------------------------------ Q8_0 matmul ---
+def _run_matmul_q8(dev, x, raw, N, K, scale=1.0, bias=0.0, act=0, residual=None, want32=False):
+    M = x.shape[0]
+    dx = dev.upload(x)
+    dw = dev.upload_q8_0(raw, N, K)
+    dy = dev.alloc(M * N * 2)
+    dres = dev.upload(residual) if residual is not None else None
+    d32 = dev.alloc(M * N * 4) if want32 else None
+    capi.check(L().vkl_matmul_q8_0(dx.ptr, dw.ptr, M, N, K, K, N, scale, bias, act,
+                                   dres.ptr if dres else None, dy.ptr, d32.ptr if d32 else None, dev.stream))
+    y = f16(dy, (M, N))
+    return (y, d32.read(np.float32, (M, N))) if want32 else y
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 37, 256), (1, 512, 1376), (1, 1376, 512), (3, 64, 1376),
+                                   (16, 130, 512), (1, 6, 11008), (5, 9, 100)])
+def test_matmul_q8_0(dev, rng, M, N, K):
+    raw, deq = q8_weights(rng, N, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    got = _run_matmul_q8(dev, x, raw, N, K)
+    want = O.matmul_q8_0(x, raw, K)
+    assert rel_err(got, want) < F16_REL_TOL
+    assert ulp_diff_f16(got, want).max() <= 1             # same products, fp32 sums in another order
+    exact = x.astype(np.float64) @ deq[:, :K].T
+    assert rel_err(got, exact) < F16_REL_TOL
+
+
+def test_matmul_q8_0_one_hot_exact_and_subnormal_activations(dev, rng):
+    N, K = 40, 256
+    raw, deq = q8_weights(rng, N, K)
+    for k in (0, 15, 16, 31, 32, 255):
+        x = np.zeros((1, K), np.float16)
+        x[0, k] = 1.0
+        got = _run_matmul_q8(dev, x, raw, N, K)
+        assert np.array_equal(got[0], deq[:, k].astype(np.float16))
+    # activations in the fp16 subnormal range must still contribute
+    x = (rng.standard_normal((1, K)) * 2e-5).astype(np.float16)
+    raw2, _ = q8_weights(rng, N, K, 0.5, 1.0)
+    got = _run_matmul_q8(dev, x, raw2, N, K)
+    want = O.matmul_q8_0(x, raw2, K)
+    assert rel_err(got, want) < F16_REL_TOL
+
+
+def test_matmul_q8_0_epilogue(dev, rng):
+    M, N, K = 2, 96, 512
+    raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    got = _run_matmul_q8(dev, x, raw, N, K, scale=0.5, bias=0.25, act=1)
+    want = O.matmul_q8_0(x, raw, K, 0.5, 0.25, 1)
+    assert rel_err(got, want) < F16_REL_TOL
+    got, got32 = _run_matmul_q8(dev, x, raw, N, K, residual=res, want32=True)
+    want = O.elementwise(O.matmul_q8_0(x, raw, K), res, 0)
+    assert rel_err(got, want) < F16_REL_TOL
+    assert np.array_equal(got32, got.astype(np.float32))  # the widening cast is exact
+
+
+def test_kqv_q8_0(dev, rng):
+    M, N, K = 3, 512, 512
+    ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dx = dev.upload(x)
+    dws = [dev.upload_q8_0(w, N, K) for w in ws]
+    outs = [dev.alloc(M * N * 2) for _ in range(3)]
+    capi.check(L().vkl_kqv_q8_0(dx.ptr, dws[0].ptr, dws[1].ptr, dws[2].ptr, M, N, K, outs[0].ptr, outs[1].ptr,
+                                outs[2].ptr, dev.stream))
+    want = O.kqv_q8_0(x, ws[0], ws[1], ws[2], K)
+    for o, w in zip(outs, want):
+        assert rel_err(f16(o, (M, N)), w) < F16_REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1376, 512), (4, 300, 256), (1, 11008, 4096)])
+def test_ffn_upgate_q8_0(dev, rng, M, N, K):
+    up, _ = q8_weights(rng, N, K, 0.005, 0.02)
+    gate, _ = q8_weights(rng, N, K, 0.005, 0.02)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dx, dup, dg = dev.upload(x), dev.upload_q8_0(up, N, K), dev.upload_q8_0(gate, N, K)
+    out = dev.alloc(M * N * 2)
+    capi.check(L().vkl_ffn_upgate_q8_0(dx.ptr, dup.ptr, dg.ptr, M, N, K, out.ptr, dev.stream))
+    assert rel_err(f16(out, (M, N)), O.ffn_upgate_q8_0(x, up, gate, K)) < F16_REL_TOL
+
+
+# ------------------------------------------------------------ fp16 matmul ---
+@pytest.mark.parametrize("C,M,N,K", [(1, 9, 9, 128), (8, 1, 300, 64), (4, 7, 50, 128), (1, 1, 512, 4096),
+                                     (2, 3, 5, 100), (1, 2, 9, 36)])
+def test_matmul_f16_tb(dev, rng, C, M, N, K):
+    a = rng.standard_normal((C, M, K)).astype(np.float16)
+    b = rng.standard_normal((C, N, K)).astype(np.float16)
+    da, db = dev.upload(a), dev.upload(b)
+    dy = dev.alloc(C * M * N * 2)
+    capi.check(L().vkl_matmul_f16_tb(da.ptr, db.ptr, C, M, N, K, M * K, K, N * K, K, M * N, N, 0.125, 0.0, 0,
+                                     None, dy.ptr, None, dev.stream))
+    assert rel_err(f16(dy, (C, M, N)), O.matmul_f16_tb(a, b, scale=0.125)) < F16_REL_TOL
+
+
+def test_matmul_f16_tb_reads_cache_view(dev, rng):
+    """scores = Q K^T over the first L rows of a [H, maxlen, hd] cache."""
+    H, maxlen, hd, Lk, S = 4, 64, 64, 37, 3
+    q = rng.standard_normal((H, S, hd)).astype(np.float16)
+    cache = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    dq, dc = dev.upload(q), dev.upload(cache)
+    dy = dev.alloc(H * S * Lk * 2)
+    capi.check(L().vkl_matmul_f16_tb(dq.ptr, dc.ptr, H, S, Lk, hd, S * hd, hd, maxlen * hd, hd, S * Lk, Lk,
+                                     1 / 8.0, 0.0, 0, None, dy.ptr, None, dev.stream))
+    want = O.matmul_f16_tb(q, np.ascontiguousarray(cache[:, :Lk]), scale=1 / 8.0)
+    assert rel_err(f16(dy, (H, S, Lk)), want) < F16_REL_TOL
+
+
+@pytest.mark.parametrize("C,M,N,K", [(4, 3, 64, 37), (2, 1, 128, 300), (1, 2, 20, 17)])
+def test_matmul_f16_nn(dev, rng, C, M, N, K):
+    a = rng.uniform(0, 0.1, (C, M, K)).astype(np.float16)
+    b = rng.standard_normal((C, K, N)).astype(np.float16)
+    da, db = dev.upload(a), dev.upload(b)
+    dy = dev.alloc(C * M * N * 2)
+    capi.check(L().vkl_matmul_f16_nn(da.ptr, db.ptr, C, M, N, K, M * K, K, K * N, N, M * N, N, 1.0, 0.0, 0, dy.ptr,
+                                     dev.stream))
+    assert rel_err(f16(dy, (C, M, N)), O.matmul_f16_nn(a, b)) < F16_REL_TOL
+
+
+def test_ffn_upgate_f16(dev, rng):
+    M, N, K = 2, 300, 512
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    up = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    gate = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    dx, du, dg = dev.upload(x), dev.upload(up), dev.upload(gate)
+    out = dev.alloc(M * N * 2)
+    capi.check(L().vkl_ffn_upgate_f16(dx.ptr, du.ptr, dg.ptr, M, N, K, out.ptr, dev.stream))
+    assert rel_err(f16(out, (M, N)), O.ffn_upgate_f16(x, up, gate)) < F16_REL_TOL
+
+
+# ------------------------------------------------- RoPE / KV / softmax ------
+@pytest.mark.parametrize("C,H,W,off", [(8, 16, 64, 0), (32, 1, 128, 100), (3, 5, 64, 1019)])
+def test_rope_bit_exact(dev, rng, C, H, W, off):
+    # tests/test_rope.cpp:211-217 uses offsets 0 / 100 / 1020
+    fc, fs = O.rope_tables(1024, W)
+    x = rng.standard_normal((C, H, W)).astype(np.float16)
+    dx, dfc, dfs = dev.upload(x), dev.upload(fc), dev.upload(fs)
+    capi.check(L().vkl_rope_f16(dx.ptr, C, H, W, dfc.ptr, dfs.ptr, off, dev.stream))
+    want = O.rope(x, fc, fs, off)
+    assert np.array_equal(f16(dx, x.shape).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("off", [0, 1022, 500])
+def test_kv_update_bit_exact(dev, rng, off):
+    C, HO, H, W = 8, 1024, 5, 64
+    cache = rng.standard_normal((C, HO, W)).astype(np.float16)
+    kv = rng.standard_normal((C, H, W)).astype(np.float16)
+    dc, dk = dev.upload(cache), dev.upload(kv)
+    capi.check(L().vkl_kv_update_f16(dc.ptr, dk.ptr, C, HO, H, W, off, dev.stream))
+    assert np.array_equal(f16(dc, cache.shape), O.update_kvcache(cache, kv, off))
+
+
+@pytest.mark.parametrize("C,H,W,off,mask", [(8, 16, 16, 0, 1), (32, 1, 289, 288, 1), (2, 5, 70, 64, 1),
+                                            (3, 4, 1000, 0, 0)])
+def test_softmax(dev, rng, C, H, W, off, mask):
+    x = (rng.standard_normal((C, H, W)) * 2).astype(np.float16)
+    dx = dev.upload(x)
+    out = dev.alloc(x.nbytes)
+    capi.check(L().vkl_softmax_f16(dx.ptr, C, H, W, mask, off, out.ptr, dev.stream))
+    got, want = f16(out, x.shape), O.softmax(x, mask, off)
+    assert np.array_equal(got == 0, want == 0)            # masked entries are exactly zero
+    assert rel_err(got, want) < F16_REL_TOL
+    assert ulp_diff_f16(got, want).max() <= 1
+
+
+# ------------------------------------------- element-wise, casts, arg, ... --
+def test_elementwise_and_casts_bit_exact(dev, rng):
+    n = 5000
+    a = rng.standard_normal(n).astype(np.float16)
+    b = (rng.standard_normal(n) + 3).astype(np.float16)
+    for op in range(4):
+        da, db = dev.upload(a), dev.upload(b)
+        capi.check(L().vkl_elementwise_f16(da.ptr, db.ptr, n, op, dev.stream))
+        assert np.array_equal(f16(db, n).view(np.uint16), O.elementwise(a, b, op).view(np.uint16))
+    da = dev.upload(a)
+    out = dev.alloc(n * 2)
+    capi.check(L().vkl_elementwise_const_f16(da.ptr, 0.5, n, 2, out.ptr, dev.stream))
+    assert np.array_equal(f16(out, n), (a.astype(np.float32) * np.float32(0.5)).astype(np.float16))
+    o32 = dev.alloc(n * 4)
+    capi.check(L().vkl_cast_f16_f32(da.ptr, o32.ptr, n, dev.stream))
+    assert np.array_equal(o32.read(np.float32, n), a.astype(np.float32))
+    f = rng.standard_normal(n).astype(np.float32)
+    df = dev.upload(f)
+    capi.check(L().vkl_cast_f32_f16(df.ptr, out.ptr, n, dev.stream))
+    assert np.array_equal(f16(out, n), f.astype(np.float16))
+
+
+def test_argop_bit_exact(dev, rng):
+    rows, W = 7, 32000
+    x = rng.standard_normal((rows, W)).astype(np.float16)
+    x[2, 17] = x[2, 25000] = 30.0
+    x[4, :] = -1.0
+    x[5, 31999] = 50.0
+    dx = dev.upload(x)
+    out = dev.alloc(rows * 4)
+    capi.check(L().vkl_argop_f16(dx.ptr, rows, W, 0, out.ptr, dev.stream))
+    assert list(out.read(np.uint32, rows)) == list(O.argmax_f16(x))
+    capi.check(L().vkl_argop_f16(dx.ptr, rows, W, 1, out.ptr, dev.stream))
+    assert list(out.read(np.uint32, rows)) == list(np.argmin(x.astype(np.float32), axis=1))
+
+
+def test_slice_and_transpose_bit_exact(dev, rng):
+    C, H, W = 5, 9, 40
+    x = rng.standard_normal((C, H, W)).astype(np.float16)
+    dx = dev.upload(x)
+    out = dev.alloc(x.nbytes)
+    capi.check(L().vkl_slice_f16(dx.ptr, C, H, W, 1, 2, 3, 3, 4, 30, out.ptr, dev.stream))
+    assert np.array_equal(f16(out, (3, 4, 30)), x[1:4, 2:6, 3:33])
+    capi.check(L().vkl_transpose102_f16(dx.ptr, C, H, W, out.ptr, dev.stream))
+    assert np.array_equal(f16(out, (H, C, W)), O.transpose102(x))
+
+
+def test_invalid_arguments_are_rejected_before_launch(dev):
+    buf = dev.alloc(1024)
+    assert L().vkl_slice_f16(buf.ptr, 2, 2, 2, 1, 0, 0, 2, 1, 1, buf.ptr, dev.stream) == 1   # c0+CE > C
+    assert L().vkl_rope_f16(buf.ptr, 1, 1, 3, buf.ptr, buf.ptr, 0, dev.stream) == 1          # odd width
+    assert L().vkl_kv_update_f16(buf.ptr, buf.ptr, 1, 2, 3, 4, 0, dev.stream) == 1           # kv longer than cache
+    assert L().vkl_matmul_q8_0(buf.ptr, buf.ptr, 1, 4, 32, 16, 4, 1.0, 0.0, 0, None, buf.ptr, None,
+                               dev.stream) == 1                                              # row stride < K
+    dev.sync()

@@ -1,0 +1,125 @@
+// Device-side helpers shared by the gfx950 kernels (wave64).
+#ifndef VKL_COMMON_H
+#define VKL_COMMON_H
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define VKL_WAVE 64
+
+#define VKL_CHECK_ARG(cond)                                                   \
+  do                                                                          \
+    {                                                                         \
+      if (!(cond))                                                            \
+        return (int)hipErrorInvalidValue;                                     \
+    }                                                                         \
+  while (0)
+
+#define VKL_HIP(expr)                                                         \
+  do                                                                          \
+    {                                                                         \
+      hipError_t e__ = (expr);                                                \
+      if (e__ != hipSuccess)                                                  \
+        return (int)e__;                                                      \
+    }                                                                         \
+  while (0)
+
+static inline int
+vkl_launch_status ()
+{
+  return (int)hipGetLastError ();
+}
+
+typedef _Float16 h16;
+typedef _Float16 h16x2 __attribute__ ((ext_vector_type (2)));
+
+namespace vkl
+{
+// sum over the 64 lanes of a wave; every lane gets the total.
+__device__ __forceinline__ float
+wave_sum (float v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    v += __shfl_xor (v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float
+wave_max (float v)
+{
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    v = fmaxf (v, __shfl_xor (v, o, 64));
+  return v;
+}
+
+__device__ __forceinline__ float
+h2f (uint16_t bits)
+{
+  return (float)__builtin_bit_cast (h16, bits);
+}
+
+__device__ __forceinline__ uint16_t
+f2h (float f)
+{
+  return __builtin_bit_cast (uint16_t, (h16)f); // v_cvt_f16_f32: RNE
+}
+
+__device__ __forceinline__ float
+silu (float v)
+{
+  return v / (1.0f + expf (-v));
+}
+
+// Four int8 packed in a dword -> two half2 holding the exact integer values.
+// (b ^ 0x80) is the byte biased by 128; 0x6400 | byte is the fp16 number
+// 1024 + byte, and subtracting 1152 gives the signed value exactly.
+__device__ __forceinline__ void
+i8x4_to_h2x2 (uint32_t w, h16x2 &lo, h16x2 &hi)
+{
+  const uint32_t u = w ^ 0x80808080u;
+  const uint32_t l = __builtin_amdgcn_perm (0x64646464u, u, 0x04010400u);
+  const uint32_t h = __builtin_amdgcn_perm (0x64646464u, u, 0x04030402u);
+  const h16x2 bias = { (h16)1152.0f, (h16)1152.0f };
+  lo = __builtin_bit_cast (h16x2, l) - bias;
+  hi = __builtin_bit_cast (h16x2, h) - bias;
+}
+
+// sum_{i<16} x[i] * q[i] with fp32 accumulation (v_dot2_f32_f16: products of
+// two fp16 numbers are exact in fp32).  w: 16 int8, x: 16 fp16 as 8 half2.
+__device__ __forceinline__ float
+dot16_q8 (const uint4 w, const h16x2 *x, float acc)
+{
+  h16x2 lo, hi;
+  i8x4_to_h2x2 (w.x, lo, hi);
+  acc = __builtin_amdgcn_fdot2 (lo, x[0], acc, false);
+  acc = __builtin_amdgcn_fdot2 (hi, x[1], acc, false);
+  i8x4_to_h2x2 (w.y, lo, hi);
+  acc = __builtin_amdgcn_fdot2 (lo, x[2], acc, false);
+  acc = __builtin_amdgcn_fdot2 (hi, x[3], acc, false);
+  i8x4_to_h2x2 (w.z, lo, hi);
+  acc = __builtin_amdgcn_fdot2 (lo, x[4], acc, false);
+  acc = __builtin_amdgcn_fdot2 (hi, x[5], acc, false);
+  i8x4_to_h2x2 (w.w, lo, hi);
+  acc = __builtin_amdgcn_fdot2 (lo, x[6], acc, false);
+  acc = __builtin_amdgcn_fdot2 (hi, x[7], acc, false);
+  return acc;
+}
+
+// sum_{i<8} a[i]*b[i], both fp16 (one dwordx4 each)
+__device__ __forceinline__ float
+dot8_f16 (const uint4 a, const uint4 b, float acc)
+{
+  acc = __builtin_amdgcn_fdot2 (__builtin_bit_cast (h16x2, a.x),
+                                __builtin_bit_cast (h16x2, b.x), acc, false);
+  acc = __builtin_amdgcn_fdot2 (__builtin_bit_cast (h16x2, a.y),
+                                __builtin_bit_cast (h16x2, b.y), acc, false);
+  acc = __builtin_amdgcn_fdot2 (__builtin_bit_cast (h16x2, a.z),
+                                __builtin_bit_cast (h16x2, b.z), acc, false);
+  acc = __builtin_amdgcn_fdot2 (__builtin_bit_cast (h16x2, a.w),
+                                __builtin_bit_cast (h16x2, b.w), acc, false);
+  return acc;
+}
+} // namespace vkl
+#endif
