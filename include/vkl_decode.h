@@ -1,0 +1,69 @@
+/*
+ * C ABI of the fused one-token decode step (libvkllama_hip.so).  It replaces,
+ * for a forward pass over ONE token, the chain of about 19 dispatches per
+ * block that the reference records in models/llama2.h:160-213 +
+ * src/ops/multiheadattention_v2.cpp:190-324 + src/ops/feed_forward.cpp:106-128
+ * and the output layer of models/llama2.h:283-298, with five phases per block:
+ *   1. RMSNorm + fused K/Q/V projection
+ *   2. RoPE + KV-cache write + attention over the cache (fp16 scores and
+ *      probabilities, as the reference materialises them)
+ *   3. Wo projection + residual add
+ *   4. RMSNorm + fused up/gate projection with SiLU
+ *   5. down projection + residual add
+ * then RMSNorm(eps 1e-6) + lm_head + fp32 widening + arg-max.  Every fp16
+ * rounding point of the operator chain is kept.
+ */
+#ifndef VKL_DECODE_H
+#define VKL_DECODE_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct
+{
+  /* matrices [out, in]: planar Q8_0 (see vkl_hip.h) or dense fp16 */
+  const void *wk, *wq, *wv, *wo, *w_gate, *w_up, *w_down;
+  const float *attn_norm, *ffn_norm; /* [dim] fp32 */
+  void *kcache, *vcache;             /* [heads, maxlen, head_dim] fp16 */
+} vkl_layer_weights;
+
+typedef struct
+{
+  int dim, n_layers, n_heads, head_dim, ffn, vocab, maxlen;
+  int wtype; /* GGML type of the matrices: 8 = Q8_0, 1 = FP16 */
+  float eps;       /* block RMSNorm eps */
+  float final_eps; /* output RMSNorm eps (1e-6 in the reference) */
+  const vkl_layer_weights *layers; /* DEVICE array [n_layers] */
+  const void *tok_embd;            /* [vocab, dim] */
+  const void *output;              /* [vocab, dim] */
+  const float *output_norm;        /* [dim] */
+  const float *freqc, *freqs;      /* RoPE tables fp32 [maxlen, head_dim/2] */
+  void *scratch; /* device, vkl_decode_scratch_bytes() bytes, zeroed once */
+} vkl_decode_model;
+
+/* bytes of device scratch a model of these dimensions needs */
+size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
+
+/* One token at KV position `pos` (context length becomes pos + 1).
+ *  tok      device-visible uint32: the input token id (ids >= vocab -> 0)
+ *  mode     0 = one launch per phase, 1 = one persistent launch per step
+ *  logits32 optional device fp32 [vocab]: widened fp16 logits
+ *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
+ * Returns 0 or a hipError_t; hipErrorInvalidValue for shapes the kernels do
+ * not cover (dim % 32, head_dim not 64/128, ffn % 32, pos >= maxlen, ...). */
+int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
+                     uint32_t pos, int mode, float *logits32,
+                     uint32_t *next_tok, void *stream);
+
+/* device pointer to the fp16 logits [vocab] of the last step inside scratch */
+const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
+/* arg-max over fp32 values (first maximum); out is device-visible */
+int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

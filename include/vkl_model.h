@@ -1,0 +1,84 @@
+/*
+ * C ABI of libvkllama_host.so around the C++ drop-in classes
+ * (vkllama_amd/src/ops, vkllama_amd/models/llama2.h): what a binding in
+ * another language needs to drive the llama2 token loop of the reference's
+ * app/llama2_infer.cpp:120-218 (model.init, model(toks, offset), greedy
+ * sampling) without touching C++ types.
+ *
+ * All functions return 0 on success, otherwise an absl::StatusCode value
+ * (3 = invalid argument, 11 = out of range, 13 = internal, ...);
+ * vkl_model_last_error() gives the message.
+ */
+#ifndef VKL_MODEL_H
+#define VKL_MODEL_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct vkl_model vkl_model;
+
+/* one GGUF tensor as models/llama2.h:401-431,486-646 reads it:
+ * type 0 = F32, 1 = F16, 8 = Q8_0 (34-byte blocks); dim0 = columns (input
+ * features), dim1 = rows; data/bsize = the raw GGUF bytes. */
+typedef struct
+{
+  const char *name;
+  uint32_t type;
+  uint64_t dim0, dim1;
+  const void *data;
+  uint64_t bsize;
+} vkl_tensor_desc;
+
+/* GGUF hyper-parameters models/llama2.h:367-370 reads */
+typedef struct
+{
+  uint32_t head_count;    /* llama.attention.head_count */
+  uint32_t block_count;   /* llama.block_count */
+  uint32_t context_length; /* llama.context_length */
+  float rms_eps;          /* llama.attention.layer_norm_rms_epsilon */
+} vkl_model_hparams;
+
+/* Model::Model(dev) + Model::init(kv, tensors) */
+int vkl_model_create (int dev, const vkl_model_hparams *hp,
+                      const vkl_tensor_desc *tensors, size_t n_tensors,
+                      vkl_model **out);
+void vkl_model_destroy (vkl_model *m);
+const char *vkl_model_last_error (const vkl_model *m);
+size_t vkl_model_vocab (const vkl_model *m);
+
+/* Model::operator()(toks, offset): fp32 logits of the last row -> logits_h
+ * (vocab floats) */
+int vkl_model_forward (vkl_model *m, const uint32_t *toks_h, size_t n_toks,
+                       size_t offset, float *logits_h);
+/* the greedy loop of app/llama2_infer.cpp:140-218; times in milliseconds */
+int vkl_model_generate_greedy (vkl_model *m, const uint32_t *prompt_h,
+                               size_t n_prompt, size_t n_gen,
+                               uint32_t *out_ids_h, double *prefill_ms,
+                               double *decode_ms);
+/* options: fused one-token decode on/off, decode launch mode (0 = one launch
+ * per phase, 1 = persistent), the reference's last-block RoPE position quirk */
+int vkl_model_set_option (vkl_model *m, const char *name, int value);
+/* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */
+int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,
+                             uint16_t *out_h, size_t n);
+/* algorithmic bytes of one decode step at context length L */
+size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
+
+/* ---- synthetic weights (seeded, host) ----------------------------------
+ * N(0, std) values from a counter-based generator: element i of stream
+ * `seed` is a pure function of (seed, i), so tensors can be produced in
+ * parallel and in any order. */
+void vkl_synth_normal_f32 (uint64_t seed, size_t n, float std, float *out_h);
+void vkl_synth_normal_f16 (uint64_t seed, size_t n, float std,
+                           uint16_t *out_h);
+/* rows x K matrix of N(0, std) quantised to Q8_0 GGUF blocks */
+void vkl_synth_normal_q8_0 (uint64_t seed, size_t rows, size_t K, float std,
+                            uint8_t *out_h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

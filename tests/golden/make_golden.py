@@ -1,0 +1,82 @@
+"""Writes the committed fixtures under tests/golden/ from the CPU oracle.
+
+Run from the repository root: python tests/golden/make_golden.py
+The reference ships no golden vectors for this path (its tests draw unseeded
+random inputs), so the fixtures hold the oracle's outputs on seeded synthetic
+inputs; tests/test_golden.py checks both the oracle (CPU) and the HIP kernels
+(GPU) against them.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from oracle import oracle as O  # noqa: E402
+from util import q8_weights  # noqa: E402
+from vkllama_amd import model as M  # noqa: E402
+
+TINY = dict(dim=512, n_layers=8, n_heads=8, ffn=1376, vocab=32000, maxlen=512, eps=1e-5, wtype=8)
+
+
+def tiny_llama():
+    w = M.synth_weights(TINY, seed=1234)
+    rng = np.random.default_rng(1234)
+    prompt = rng.integers(3, 32000, 16).astype(np.uint32)
+    om = O.OracleModel(TINY, w)
+    ids, first = om.generate_greedy(prompt, 128)
+    top = np.argsort(-first, kind="stable")[:8]
+    out = {
+        "config": TINY, "weight_seed": 1234, "prompt": [int(t) for t in prompt],
+        "oracle_ids": [int(t) for t in ids],
+        "first_logits_top8_idx": [int(i) for i in top],
+        "first_logits_top8_val": [float(first[i]) for i in top],
+    }
+    with open(os.path.join(HERE, "tiny_llama_c2_greedy.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("tiny llama ids:", out["oracle_ids"][:16], "...")
+
+
+def ops():
+    rng = np.random.default_rng(2024)
+    d = {}
+    N, K, M_ = 48, 256, 2
+    raw, _ = q8_weights(rng, N, K)
+    x = rng.standard_normal((M_, K)).astype(np.float16)
+    d["q8_w"], d["q8_x"] = raw, x
+    d["q8_y"] = O.matmul_q8_0(x, raw, K)
+    raw2, _ = q8_weights(rng, N, K)
+    raw3, _ = q8_weights(rng, N, K)
+    d["q8_w2"], d["q8_w3"] = raw2, raw3
+    k, q, v = O.kqv_q8_0(x, raw, raw2, raw3, K)
+    d["kqv_k"], d["kqv_q"], d["kqv_v"] = k, q, v
+    d["upgate"] = O.ffn_upgate_q8_0(x, raw, raw2, K)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    d["norm_w"] = w
+    d["norm_y"] = O.rmsnorm(x, w, 1e-5)
+    fc, fs = O.rope_tables(64, 64)
+    r = rng.standard_normal((4, 3, 64)).astype(np.float16)
+    d["rope_x"], d["rope_y"] = r, O.rope(r, fc, fs, 17)
+    s = (rng.standard_normal((4, 3, 20)) * 2).astype(np.float16)
+    d["softmax_x"], d["softmax_y"] = s, O.softmax(s, True, 17)
+    a = rng.standard_normal((4, 3, 64)).astype(np.float16)
+    b = rng.standard_normal((4, 20, 64)).astype(np.float16)
+    d["tb_a"], d["tb_b"], d["tb_y"] = a, b, O.matmul_f16_tb(a, b, scale=0.125)
+    p = rng.uniform(0, 0.2, (4, 3, 20)).astype(np.float16)
+    d["nn_a"], d["nn_y"] = p, O.matmul_f16_nn(p, b)
+    xq = rng.uniform(-5, 5, (3, 95)).astype(np.float32)
+    d["quant_x"], d["quant_y"] = xq, O.quantize_q8_0(xq, 2)
+    toks = np.array([0, 47, 7, 48, 2 ** 31], np.uint32)
+    d["embed_toks"], d["embed_y"] = toks, O.embedding_q8_0(raw, K, toks, 0)
+    np.savez_compressed(os.path.join(HERE, "ops_golden.npz"), **d)
+    print("ops fixture:", sum(v.nbytes for v in d.values()), "bytes raw")
+
+
+if __name__ == "__main__":
+    ops()
+    tiny_llama()

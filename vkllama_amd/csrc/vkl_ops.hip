@@ -124,8 +124,8 @@ elementwise_kernel (const uint16_t *__restrict__ x, uint16_t *y, size_t n,
 }
 
 __global__ void
-elementwise_const_kernel (const uint16_t *__restrict__ x, float alpha,
-                          size_t n, int op, uint16_t *__restrict__ out)
+elementwise_const_kernel (const uint16_t *x, float alpha, size_t n, int op,
+                          uint16_t *out)
 {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n)

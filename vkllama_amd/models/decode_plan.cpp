@@ -1,0 +1,163 @@
+#include "models/decode_plan.h"
+#include "models/llama2.h"
+#include "vkl_hip.h"
+#include <string.h>
+
+namespace vkllama
+{
+static absl::Status
+hip_status (const char *what, int e)
+{
+  if (!e)
+    return absl::OkStatus ();
+  if (e == 1)
+    return absl::InvalidArgumentError (
+        absl::StrFormat ("%s: rejected by the HIP layer", what));
+  return absl::InternalError (
+      absl::StrFormat ("%s: %s", what, vkl_error_string (e)));
+}
+
+DecodePlan::DecodePlan ()
+    : gpu_ (nullptr), usable_ (false), mode_ (0), adopted_valid_ (false),
+      vocab_ (0)
+{
+  memset (&desc_, 0, sizeof (desc_));
+}
+
+DecodePlan::~DecodePlan () {}
+
+absl::Status
+DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
+                   std::vector<Llama2Block *> &blocks, OutputLayer *out,
+                   float eps)
+{
+  gpu_ = gpu;
+  vocab_ = model.vocab_size ();
+  tok_slot_ = Tensor (1, 1, 1, gpu, UINT32, true);
+  VKLLAMA_STATUS_OK (tok_slot_.create ());
+  logits32_ = Tensor (1, 1, (int)vocab_, gpu, FP32, false);
+  VKLLAMA_STATUS_OK (logits32_.create ());
+
+  Tensor &emb = in->embedding ()->vocab ();
+  auto *attn0 = blocks[0]->attention ();
+  const size_t dim = emb.width ();
+  const size_t hd = attn0->kcache ().width ();
+  const size_t heads = attn0->kcache ().channels ();
+  const size_t ffn = blocks[0]->feed_forward ()->w1 ().height ();
+  const bool q8 = emb.dtype () == Q8_0 && out->weight ().dtype () == Q8_0
+                  && attn0->wk ().dtype () == Q8_0
+                  && attn0->wo ().dtype () == Q8_0
+                  && blocks[0]->feed_forward ()->w1 ().dtype () == Q8_0;
+  if (!q8 || (hd != 64 && hd != 128) || heads * hd != dim || dim % 32
+      || ffn % 32 || vocab_ % 2)
+    {
+      usable_ = false; // the operator chain serves these models
+      return absl::OkStatus ();
+    }
+
+  std::vector<vkl_layer_weights> lw (blocks.size ());
+  for (size_t i = 0; i < blocks.size (); ++i)
+    {
+      auto *a = blocks[i]->attention ();
+      auto *f = blocks[i]->feed_forward ();
+      lw[i].wk = a->wk ().data ();
+      lw[i].wq = a->wq ().data ();
+      lw[i].wv = a->wv ().data ();
+      lw[i].wo = a->wo ().data ();
+      lw[i].w_gate = f->w1 ().data ();
+      lw[i].w_down = f->w2 ().data ();
+      lw[i].w_up = f->w3 ().data ();
+      lw[i].attn_norm = (const float *)blocks[i]->attn_norm ()->weight ().data ();
+      lw[i].ffn_norm = (const float *)blocks[i]->ffn_norm ()->weight ().data ();
+      lw[i].kcache = a->kcache ().data ();
+      lw[i].vcache = a->vcache ().data ();
+    }
+  const size_t lbytes = lw.size () * sizeof (vkl_layer_weights);
+  layers_ = Tensor (1, 1, (int)lbytes, gpu, INT8, false);
+  VKLLAMA_STATUS_OK (layers_.create ());
+  VKLLAMA_STATUS_OK (hip_status (
+      "uploading layer table",
+      vkl_memcpy_h2d (layers_.data (), lw.data (), lbytes, gpu->stream ())));
+  VKLLAMA_STATUS_OK (
+      hip_status ("uploading layer table", vkl_stream_sync (gpu->stream ())));
+
+  desc_.dim = (int)dim;
+  desc_.n_layers = (int)blocks.size ();
+  desc_.n_heads = (int)heads;
+  desc_.head_dim = (int)hd;
+  desc_.ffn = (int)ffn;
+  desc_.vocab = (int)vocab_;
+  desc_.maxlen = (int)attn0->kcache ().height ();
+  desc_.wtype = 8;
+  desc_.eps = eps;
+  desc_.final_eps = out->norm ()->eps ();
+  desc_.layers = (const vkl_layer_weights *)layers_.data ();
+  desc_.tok_embd = emb.data ();
+  desc_.output = out->weight ().data ();
+  desc_.output_norm = (const float *)out->norm ()->weight ().data ();
+  desc_.freqc = (const float *)attn0->rope ()->freqc ().data ();
+  desc_.freqs = (const float *)attn0->rope ()->freqs ().data ();
+  const size_t sbytes = vkl_decode_scratch_bytes (&desc_);
+  scratch_ = Tensor (1, 1, (int)sbytes, gpu, INT8, false);
+  VKLLAMA_STATUS_OK (scratch_.create ());
+  VKLLAMA_STATUS_OK (hip_status (
+      "clearing decode scratch",
+      vkl_memset (scratch_.data (), 0, sbytes, gpu->stream ())));
+  desc_.scratch = scratch_.data ();
+  usable_ = true;
+  return absl::OkStatus ();
+}
+
+absl::Status
+DecodePlan::step_host_token (uint32_t tok, size_t offset)
+{
+  // the slot may still be read by a queued step
+  VKLLAMA_STATUS_OK (
+      hip_status ("waiting for the stream", vkl_stream_sync (gpu_->stream ())));
+  *(uint32_t *)tok_slot_.host () = tok;
+  return step_device_token ((const uint32_t *)tok_slot_.data (), offset);
+}
+
+absl::Status
+DecodePlan::step_device_token (const uint32_t *tok, size_t offset)
+{
+  if (!usable_)
+    return absl::FailedPreconditionError (
+        "fused decode does not cover this model");
+  adopted_valid_ = false;
+  return hip_status ("decode step",
+                     vkl_decode_step (&desc_, tok, (uint32_t)offset, mode_,
+                                      (float *)logits32_.data (), nullptr,
+                                      gpu_->stream ()));
+}
+
+absl::Status
+DecodePlan::adopt_logits (Tensor logits32)
+{
+  if (logits32.dtype () != FP32 || logits32.size () < vocab_)
+    return absl::InvalidArgumentError ("logits tensor has the wrong type");
+  adopted_ = logits32;
+  adopted_valid_ = true;
+  return absl::OkStatus ();
+}
+
+absl::Status
+DecodePlan::read_logits (float *dst)
+{
+  const Tensor &src = adopted_valid_ ? adopted_ : logits32_;
+  const float *p = (const float *)src.data () + (src.size () - vocab_);
+  VKLLAMA_STATUS_OK (hip_status (
+      "downloading logits",
+      vkl_memcpy_d2h (dst, p, vocab_ * sizeof (float), gpu_->stream ())));
+  return hip_status ("downloading logits", vkl_stream_sync (gpu_->stream ()));
+}
+
+absl::Status
+DecodePlan::argmax_logits (uint32_t *dst)
+{
+  const Tensor &src = adopted_valid_ ? adopted_ : logits32_;
+  const float *p = (const float *)src.data () + (src.size () - vocab_);
+  return hip_status ("argmax", vkl_argmax_f32 (p, (int)vocab_, dst,
+                                               gpu_->stream ()));
+}
+}

@@ -1,0 +1,53 @@
+// DecodePlan: the device-pointer view of a loaded model that the fused
+// one-token decode step (include/vkl_decode.h) consumes, plus the small state
+// the greedy loop keeps on the device (current logits, token slot).
+#ifndef __VKLLAMA_MODELS_DECODE_PLAN_H__
+#define __VKLLAMA_MODELS_DECODE_PLAN_H__
+#include "absl/status/status.h"
+#include "src/core/tensor.h"
+#include "vkl_decode.h"
+#include <vector>
+
+namespace vkllama
+{
+class GPUDevice;
+class InputLayer;
+class OutputLayer;
+class Llama2Block;
+class Model;
+
+struct DecodePlan
+{
+  DecodePlan ();
+  ~DecodePlan ();
+  absl::Status build (Model &model, GPUDevice *gpu, InputLayer *in,
+                      std::vector<Llama2Block *> &blocks, OutputLayer *out,
+                      float eps);
+  // true when the fused kernels cover this model (Q8_0, head width 64/128)
+  bool usable () const { return usable_; }
+  void set_mode (int mode) { mode_ = mode; }
+  // token id given by the host / read from device-visible memory
+  absl::Status step_host_token (uint32_t tok, size_t offset);
+  absl::Status step_device_token (const uint32_t *tok, size_t offset);
+  // copies the fp32 logits of the last step (fused or adopted) to the host
+  absl::Status read_logits (float *dst);
+  // remember the fp32 logits tensor of an operator-chain pass
+  absl::Status adopt_logits (Tensor logits32);
+  // arg-max of the current logits into device-visible memory
+  absl::Status argmax_logits (uint32_t *dst);
+
+private:
+  GPUDevice *gpu_;
+  bool usable_;
+  int mode_;
+  vkl_decode_model desc_;
+  Tensor layers_;   // device array of vkl_layer_weights
+  Tensor scratch_;
+  Tensor logits32_; // fp32 [vocab] written by the fused step
+  Tensor tok_slot_; // pinned uint32
+  Tensor adopted_;  // logits of the operator chain, if newer
+  bool adopted_valid_;
+  size_t vocab_;
+};
+}
+#endif
