@@ -1,0 +1,143 @@
+#!/usr/bin/env python3
+"""Benchmark of the llama2 token loop on one MI355X.
+
+A step is one batch-1 greedy decode token.  The default workload is BASELINE
+config 3: Llama-2-7B shape (dim 4096, 32 layers, 32 heads, FFN 11008, vocab
+32000, context 4096), random-init N(0, 0.02) weights quantised to Q8_0, fp16
+activations and KV cache, a 32-token random-id prompt, then K greedy decode
+tokens (K = 256 by default, contexts 33 .. 32+K).
+
+Prints ONE JSON line.  `value` is decode tokens per second with weights and
+KV cache resident in HBM, timed across the K steps between device
+synchronisations, including the on-device arg-max and the token hand-over.
+`roofline` prices the decode step against the 8 TB/s HBM peak with the
+algorithmic bytes per token; `cpu_baseline` is the CPU oracle timed on this
+box's host cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # BASELINE configs 2, 3, 5 (config 4, FP16 weights, runs on the operator chain)
+    "llama2-tiny-q8_0": dict(dim=512, n_layers=8, n_heads=8, ffn=1376, vocab=32000, maxlen=512, eps=1e-5, wtype=8,
+                             prompt=16, prefill_kv=0),
+    "llama2-7b-q8_0": dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5,
+                           wtype=8, prompt=32, prefill_kv=0),
+    "llama2-13b-q8_0-ctx3968": dict(dim=5120, n_layers=40, n_heads=40, ffn=13824, vocab=32000, maxlen=4096,
+                                    eps=1e-5, wtype=8, prompt=3968, prefill_kv=1),
+}
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(cfg, weights, n_tokens):
+    """The CPU oracle (a plain-C restatement of the reference's arithmetic,
+    OpenMP over output rows) decoding n_tokens after a 4-token prompt."""
+    from oracle import oracle as O
+    om = O.OracleModel(cfg, weights)
+    om.forward(np.array([5, 17, 99, 3], np.uint32), 0)
+    tok, pos = 7, 4
+    t0 = time.perf_counter()
+    for _ in range(n_tokens):
+        logits = om.forward([tok], pos)
+        tok = int(np.argmax(logits))
+        pos += 1
+    dt = time.perf_counter() - t0
+    om.close()
+    return n_tokens / dt, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS))
+    ap.add_argument("--decode-mode", type=int, default=0)
+    ap.add_argument("--cpu-tokens", type=int, default=-1, help="decode tokens of the CPU baseline (0 = skip)")
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (batch-1 decode is a single dependency chain; "
+                 "see DESIGN.md for how it would shard); got --gpus %d" % args.gpus)
+
+    from vkllama_amd import capi, model as M
+
+    wl = dict(WORKLOADS[args.workload])
+    n_prompt, prefill_kv = wl.pop("prompt"), wl.pop("prefill_kv")
+    cfg = wl
+    steps, warmup = args.steps, args.warmup
+    if n_prompt + steps + 1 > cfg["maxlen"]:
+        sys.exit("prompt %d + %d steps exceed the context length %d" % (n_prompt, steps, cfg["maxlen"]))
+
+    t0 = time.perf_counter()
+    weights = M.synth_weights(cfg, seed=args.seed)
+    t_synth = time.perf_counter() - t0
+    rng = np.random.default_rng(args.seed)
+    prompt = rng.integers(3, cfg["vocab"], n_prompt).astype(np.uint32)
+
+    t0 = time.perf_counter()
+    m = M.Llama2(cfg, weights)
+    m.set_option("decode_mode", args.decode_mode)
+    t_load = time.perf_counter() - t0
+
+    # warm-up: prompt pass + W decode steps, untimed
+    m.generate_greedy(prompt, warmup + 1)
+    # timed: prompt pass (reported as prefill), then exactly `steps` decode steps
+    ids, prefill_ms, decode_ms = m.generate_greedy(prompt, steps + 1)
+    tok_s = steps / (decode_ms * 1e-3)
+    ms_per_step = decode_ms / steps
+
+    # algorithmic bytes per decode step, averaged over the contexts of the timed steps
+    ctx = np.arange(n_prompt + 1, n_prompt + steps + 1)
+    step_bytes = float(np.mean([m.decode_step_bytes(int(L)) for L in (ctx[0], ctx[-1])]))
+    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "decode_tokens_per_second_bs1",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "q8_0 weights x f16 activations, f32 accumulate",
+        "data": "synthetic: random-init N(0,0.02) weights quantised to Q8_0, random prompt ids",
+        "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
+                   "decode_mode": "persistent" if args.decode_mode else "launch-per-phase",
+                   "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
+        "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "decode step (all phases of one token)",
+                     "bytes_per_step": int(step_bytes)},
+        "load_seconds": {"synthesize": round(t_synth, 1), "upload": round(t_load, 1)},
+        "first_ids": [int(t) for t in ids[:8]],
+    }
+    m.close()
+
+    cpu_tokens = args.cpu_tokens
+    if cpu_tokens < 0:
+        cpu_tokens = 8 if cfg["dim"] >= 4096 else 64
+    if cpu_tokens > 0:
+        v, dt = cpu_baseline(cfg, weights, cpu_tokens)
+        result["cpu_baseline"] = {
+            "value": round(v, 3), "unit": "tok/s", "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count())),
+            "kind": "port",
+            "sample": "%d greedy decode tokens at context 5..%d after a 4-token prompt, same weights (%.1f s)"
+                      % (cpu_tokens, 4 + cpu_tokens, dt)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -255,8 +255,16 @@ vkl_synth_normal_q8_0 (uint64_t seed, size_t rows, size_t K, float std,
 #pragma omp for schedule(static)
     for (size_t r = 0; r < rows; ++r)
       {
-        for (size_t k = 0; k < K; ++k)
-          row[k] = normal_at (seed, r * K + k, std);
+        // element i of the stream comes from pair i/2; rows start on an even
+        // index when K is even, then one pair fills two neighbours
+        const size_t base = r * K;
+        size_t k = 0;
+        if (base & 1)
+          row[k] = normal_at (seed, base, std), ++k;
+        for (; k + 1 < K; k += 2)
+          normal_pair (seed, (base + k) >> 1, std, row[k], row[k + 1]);
+        if (k < K)
+          row[k] = normal_at (seed, base + k, std);
         vkl_quantize_q8_0_h (row.data (), K, out + r * rb);
       }
   }
