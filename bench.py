@@ -114,7 +114,7 @@ def main():
         "dtype": "q8_0 weights x f16 activations, f32 accumulate",
         "data": "synthetic: random-init N(0,0.02) weights quantised to Q8_0, random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
-                   "decode_mode": "persistent" if args.decode_mode else "launch-per-phase",
+                   "decode_mode": ("launch-per-phase", "persistent", "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

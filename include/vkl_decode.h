@@ -36,7 +36,8 @@ typedef struct
   int wtype; /* GGML type of the matrices: 8 = Q8_0, 1 = FP16 */
   float eps;       /* block RMSNorm eps */
   float final_eps; /* output RMSNorm eps (1e-6 in the reference) */
-  const vkl_layer_weights *layers; /* DEVICE array [n_layers] */
+  const vkl_layer_weights *layers;   /* DEVICE array [n_layers] */
+  const vkl_layer_weights *layers_h; /* the same table in HOST memory */
   const void *tok_embd;            /* [vocab, dim] */
   const void *output;              /* [vocab, dim] */
   const float *output_norm;        /* [dim] */
@@ -49,7 +50,10 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
 
 /* One token at KV position `pos` (context length becomes pos + 1).
  *  tok      device-visible uint32: the input token id (ids >= vocab -> 0)
- *  mode     0 = one launch per phase, 1 = one persistent launch per step
+ *  mode     0 = one launch per phase; 1 = one persistent launch per step
+ *           with grid barriers; 2 = one launch per phase on two alternating
+ *           streams, consecutive phases overlapping and handing over
+ *           through an arrival counter
  *  logits32 optional device fp32 [vocab]: widened fp16 logits
  *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
  * Returns 0 or a hipError_t; hipErrorInvalidValue for shapes the kernels do

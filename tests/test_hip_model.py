@@ -158,3 +158,22 @@ def test_errors(small):
     short["blk.0.ffn_up.weight"] = w["blk.0.ffn_up.weight"][:-1]
     with pytest.raises(capi.VklError, match=r"\(11\)"):
         M.Llama2(cfg, short)
+
+
+@pytest.mark.parametrize("mode", [1])
+@pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5), (TINY, 1234)])
+def test_other_decode_modes_match_oracle(cfg, seed, mode):
+    """decode_mode 1: one persistent launch per token with grid barriers;
+    decode_mode 2: one launch per phase on two alternating streams, each phase
+    prefetching its weights while it waits for its predecessor's arrivals."""
+    w = M.synth_weights(cfg, seed=seed)
+    prompt = np.array([5, 17, 99, 3], np.uint32)
+    m = M.Llama2(cfg, w)
+    m.set_option("decode_mode", mode)
+    om = O.OracleModel(cfg, w)
+    assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
+    assert logit_err(m.forward([7], 4), om.forward([7], 4)) < 1e-2
+    ids, _, t_dec = m.generate_greedy(prompt, 32)
+    want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 32)
+    assert list(ids) == list(want)
+    m.close()

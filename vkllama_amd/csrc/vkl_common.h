@@ -33,8 +33,37 @@ vkl_launch_status ()
 typedef _Float16 h16;
 typedef _Float16 h16x2 __attribute__ ((ext_vector_type (2)));
 
+#define VKL_GLOBAL __attribute__ ((address_space (1)))
+typedef uint32_t vkl_u32x4 __attribute__ ((ext_vector_type (4)));
+
 namespace vkl
 {
+// Loads and stores through pointers that were themselves read from memory
+// (e.g. a per-layer table of weight pointers) are FLAT accesses unless the
+// address space is stated: a flat load also counts against the LDS counter,
+// so that waiting for an LDS read would wait for every weight load in flight.
+// These helpers pin the global address space.
+template <typename T>
+__device__ __forceinline__ T
+ldg (const T *p)
+{
+  return *(const VKL_GLOBAL T *)p;
+}
+
+template <typename T>
+__device__ __forceinline__ void
+stg (T *p, T v)
+{
+  *(VKL_GLOBAL T *)p = v;
+}
+
+__device__ __forceinline__ uint4
+ldg4 (const void *p)
+{
+  const vkl_u32x4 v = *(const VKL_GLOBAL vkl_u32x4 *)p;
+  return make_uint4 (v.x, v.y, v.z, v.w);
+}
+
 // sum over the 64 lanes of a wave; every lane gets the total.
 __device__ __forceinline__ float
 wave_sum (float v)

@@ -1,16 +1,23 @@
 // Fused one-token decode step for Llama-2-shaped models with Q8_0 weights.
 //
-// Work decomposition (both launch modes): a grid of G workgroups of 512
-// threads, G = number of compute units.  In a projection phase workgroup g
-// owns the contiguous output rows [N*g/G, N*(g+1)/G) of the weight matrix, so
-// it streams one contiguous span of the int8 plane; inside it wave w takes
-// the row pairs 2w, 2w+16, ...; lane l of a wave handles the 16 quants at
-// k = step*1024 + 16*l of each row (one dwordx4 load = half a Q8_0 block).
-// The activation vector is staged once per phase in LDS as fp16 (with the
-// RMSNorm folded in where the phase starts with one).  Attention runs one
-// workgroup per head.
+// Work decomposition: a grid of G workgroups of 512 threads (8 waves), G = the
+// number of compute units.  In a projection phase the output rows are grouped
+// into units of 2 rows (4 for the fused up/gate product: two up rows and the
+// two gate rows that pair with them); workgroup g owns a contiguous range of
+// units, so it streams one contiguous span of each int8 plane, and wave w of
+// the group takes every 8th unit.  Lane l of a wave handles the 16 quants at
+// k = step*1024 + 16*l of a row (one dwordx4 load = half a Q8_0 block).
 //
-// Each phase is HBM-bound: 34 bytes per 32 weights are read exactly once, the
+// A wave's work is a sequence of items (one unit x one K chunk, 8 dwordx4
+// loads per lane) that runs through a two-deep register pipeline: the loads of
+// item i+1 are in flight while item i is multiplied, and the first item of a
+// phase is issued BEFORE the activation vector is staged (its weights do not
+// depend on the activations), which takes the activation latency off the
+// critical path.  The activation vector sits in LDS as fp16, with the RMSNorm
+// folded into the staging where a phase starts with one.  Attention runs one
+// workgroup per head with the first cache rows prefetched the same way.
+//
+// Every phase is HBM-bound: 34 bytes per 32 weights are read exactly once, the
 // activations (a few KiB) come from L2.
 #include "../../include/vkl_decode.h"
 #include "vkl_decode_dev.h"
@@ -21,10 +28,10 @@ namespace
 {
 struct Scratch
 {
-  uint16_t *x;    // [dim] residual stream
-  uint16_t *kqv;  // [3*dim]: k | q | v
-  uint16_t *att;  // [dim]
-  uint16_t *t;    // [ffn]
+  uint16_t *x;        // [dim] residual stream
+  uint16_t *kqv;      // [3*dim]: k | q | v
+  uint16_t *att;      // [dim]
+  uint16_t *t;        // [ffn] 32-bit words, fp16 in the low half
   uint16_t *logits16; // [vocab]
   float *logits32;    // [vocab]
   float *amax_val;    // [1024]
@@ -48,7 +55,7 @@ carve (void *base, int dim, int ffn, int vocab)
   s.x = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
   s.kqv = (uint16_t *)(p + o), o += align256 ((size_t)dim * 6);
   s.att = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
-  s.t = (uint16_t *)(p + o), o += align256 ((size_t)ffn * 2);
+  s.t = (uint16_t *)(p + o), o += align256 ((size_t)ffn * 4);
   s.logits16 = (uint16_t *)(p + o), o += align256 ((size_t)vocab * 2);
   s.logits32 = (float *)(p + o), o += align256 ((size_t)vocab * 4);
   s.amax_val = (float *)(p + o), o += 4096;
@@ -66,7 +73,20 @@ struct Params
   uint32_t pos;
   float *logits32;    // destination of the widened logits
   uint32_t *next_tok; // may be null
+  uint32_t wait_target; // overlapped launches: arrivals to wait for
+#ifdef VKL_TRACE
+  unsigned long long *trace; // [phase slot][wg][8] wall-clock stamps
+#endif
 };
+
+#ifdef VKL_TRACE
+#define VKL_TR(slot)                                                          \
+  if (threadIdx.x == 0 && p.trace)                                            \
+    p.trace[((size_t)(layer * 8 + phase) * 1024 + wg) * 8 + (slot)]           \
+        = wall_clock64 ();
+#else
+#define VKL_TR(slot)
+#endif
 
 // ---------------------------------------------------------------------------
 // activation staging
@@ -77,7 +97,7 @@ ld_u32 (const uint32_t *p)
 {
   if (COH)
     return ld_coherent_u32 (p);
-  return *p;
+  return ldg (p);
 }
 
 template <bool COH>
@@ -87,7 +107,7 @@ st_u32 (uint32_t *p, uint32_t v)
   if (COH)
     st_coherent_u32 (p, v);
   else
-    *p = v;
+    stg (p, v);
 }
 
 // sum over the workgroup; `red` is an LDS array of kDecWaves floats
@@ -106,68 +126,208 @@ block_sum (float v, float *red)
   return t;
 }
 
-// xl[0..Kp) <- fp16 activation row (K valid, zero padded), from global memory
+// The activation row (K fp16 values, K a multiple of 32, K <= 16384) is
+// fetched into registers first: thread t holds the 8-element chunks t,
+// t+512, t+1024, t+1536.  Issued before any weight load, these are the oldest
+// vector-memory operations of the wave, so they return first (loads return in
+// order) while the weight prefetch issued right after them is still in
+// flight.
+struct XRegs
+{
+  uint4 v[4];
+};
+
+struct NormRegs
+{
+  uint4 w[4][2]; // 8 fp32 weights per chunk
+};
+
 template <bool COH>
 __device__ __forceinline__ void
-stage_raw (const uint16_t *src, int K, int Kp, uint16_t *xl)
+issue_x (const uint16_t *src, int K, XRegs &x)
 {
-  const uint32_t *s32 = (const uint32_t *)src;
-  uint32_t *x32 = (uint32_t *)xl;
-  for (int i = threadIdx.x; i < Kp / 2; i += kDecThreads)
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
     {
-      uint32_t v = 0;
-      if (2 * i + 1 < K)
-        v = ld_u32<COH> (s32 + i);
-      else if (2 * i < K)
-        v = src[2 * i];
-      x32[i] = v;
+      const int idx = threadIdx.x + j * kDecThreads;
+      x.v[j] = make_uint4 (0, 0, 0, 0);
+      if (idx * 8 < K)
+        {
+          if (COH)
+            {
+              const uint32_t *s32 = (const uint32_t *)src + idx * 4;
+              x.v[j] = make_uint4 (ld_coherent_u32 (s32), ld_coherent_u32 (s32 + 1),
+                                   ld_coherent_u32 (s32 + 2), ld_coherent_u32 (s32 + 3));
+            }
+          else
+            x.v[j] = ldg4 (src + idx * 8);
+        }
     }
 }
 
-// xl <- one row of a planar Q8_0 table, dequantised: fp16(float(q) * d)
+// the same from a row stored as one 32-bit word per element (fp16 in the low
+// half)
+template <bool COH>
 __device__ __forceinline__ void
-stage_embed_q8 (const QMat tab, size_t row, int K, int Kp, uint16_t *xl)
+issue_x32 (const uint32_t *src, int K, XRegs &x)
 {
-  const uint32_t *q32 = (const uint32_t *)(tab.q + row * Kp);
-  const uint16_t *d = tab.d + row * (Kp >> 5);
-  uint32_t *x32 = (uint32_t *)xl;
-  for (int i = threadIdx.x; i < Kp / 4; i += kDecThreads)
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
     {
-      const uint32_t w = q32[i];
-      const float sc = h2f (d[i >> 3]);
-      uint16_t h[4];
+      const int idx = threadIdx.x + j * kDecThreads;
+      x.v[j] = make_uint4 (0, 0, 0, 0);
+      if (idx * 8 < K)
+        {
+          uint32_t w[8];
+          if (COH)
+            {
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                w[i] = ld_coherent_u32 (src + idx * 8 + i);
+            }
+          else
+            {
+              const uint4 a = ldg4 (src + idx * 8), b = ldg4 (src + idx * 8 + 4);
+              w[0] = a.x, w[1] = a.y, w[2] = a.z, w[3] = a.w;
+              w[4] = b.x, w[5] = b.y, w[6] = b.z, w[7] = b.w;
+            }
+          x.v[j] = make_uint4 ((w[0] & 0xffffu) | (w[1] << 16),
+                               (w[2] & 0xffffu) | (w[3] << 16),
+                               (w[4] & 0xffffu) | (w[5] << 16),
+                               (w[6] & 0xffffu) | (w[7] << 16));
+        }
+    }
+}
+
+// one row of a planar Q8_0 table: the 8 quants of each chunk land in v[j].x/.y
+// and the block scale in v[j].z; dequant_embed turns them into fp16
+__device__ __forceinline__ void
+issue_embed_q8 (const QMat tab, size_t row, int K, XRegs &x)
+{
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const int idx = threadIdx.x + j * kDecThreads;
+      x.v[j] = make_uint4 (0, 0, 0, 0);
+      if (idx * 8 < K)
+        {
+          const unsigned long long q
+              = ldg ((const unsigned long long *)(tab.q + row * K + idx * 8));
+          x.v[j].x = (uint32_t)q, x.v[j].y = (uint32_t)(q >> 32);
+          x.v[j].z = ldg (tab.d + row * (K >> 5) + (idx >> 2));
+        }
+    }
+}
+
+// fp16(float(q) * float(d)), the embedding lookup's arithmetic
+__device__ __forceinline__ void
+dequant_embed (XRegs &x)
+{
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const float sc = h2f ((uint16_t)x.v[j].z);
+      const uint32_t w[2] = { x.v[j].x, x.v[j].y };
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        {
+          const int8_t b0 = (int8_t)((w[i >> 1] >> (16 * (i & 1))) & 0xff);
+          const int8_t b1 = (int8_t)((w[i >> 1] >> (16 * (i & 1) + 8)) & 0xff);
+          o[i] = (uint32_t)f2h ((float)b0 * sc)
+                 | ((uint32_t)f2h ((float)b1 * sc) << 16);
+        }
+      x.v[j] = make_uint4 (o[0], o[1], o[2], o[3]);
+    }
+}
+
+__device__ __forceinline__ void
+issue_norm (const float *w, int K, NormRegs &n)
+{
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const int idx = threadIdx.x + j * kDecThreads;
+      n.w[j][0] = n.w[j][1] = make_uint4 (0, 0, 0, 0);
+      if (idx * 8 < K)
+        {
+          n.w[j][0] = ldg4 (w + idx * 8);
+          n.w[j][1] = ldg4 (w + idx * 8 + 4);
+        }
+    }
+}
+
+// Parks the norm weights in LDS so that they do not occupy 32 registers while
+// a phase waits for its predecessor; finish_x reads them back from there.
+__device__ __forceinline__ void
+stash_norm (const NormRegs &n, int K, uint8_t *nl)
+{
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const int idx = threadIdx.x + j * kDecThreads;
+      if (idx * 8 < K)
+        {
+          ((uint4 *)nl)[2 * idx] = n.w[j][0];
+          ((uint4 *)nl)[2 * idx + 1] = n.w[j][1];
+        }
+    }
+}
+
+// Writes the row to LDS as fp16; with `n` it is RMS-normalised on the way:
+// y = fp16(x * w * (1 / sqrt(mean(x^2) + eps))).  Ends with a barrier.
+template <bool NORM, bool NLDS = false>
+__device__ __forceinline__ void
+finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
+          float *red, const uint8_t *nl = nullptr)
+{
+  float alpha = 0.f;
+  if (NORM)
+    {
+      float s = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         {
-          const int8_t b = (int8_t)((w >> (8 * j)) & 0xff);
-          h[j] = 4 * i + j < K ? f2h ((float)b * sc) : (uint16_t)0;
+          const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            {
+              const float a = h2f ((uint16_t)(w[i] & 0xffff));
+              const float b = h2f ((uint16_t)(w[i] >> 16));
+              s += a * a;
+              s += b * b;
+            }
         }
-      x32[2 * i] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-      x32[2 * i + 1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+      const float total = block_sum (s, red);
+      alpha = 1.0f / sqrtf (total / (float)K + eps);
     }
-}
-
-__device__ __forceinline__ void
-stage_embed_f16 (const uint16_t *tab, size_t row, int K, int Kp, uint16_t *xl)
-{
-  for (int i = threadIdx.x; i < Kp; i += kDecThreads)
-    xl[i] = i < K ? tab[row * K + i] : (uint16_t)0;
-}
-
-// in-place RMSNorm of the staged row: y = fp16(x * w * rsqrt(mean(x^2)+eps))
-__device__ __forceinline__ void
-norm_staged (uint16_t *xl, int K, const float *w, float eps, float *red)
-{
-  float s = 0.f;
-  for (int i = threadIdx.x; i < K; i += kDecThreads)
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
     {
-      const float v = h2f (xl[i]);
-      s += v * v;
+      const int idx = threadIdx.x + j * kDecThreads;
+      if (idx * 8 >= K)
+        continue;
+      uint4 o = x.v[j];
+      if (NORM)
+        {
+          const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
+          // norm weights: from registers, or from where stash_norm parked them
+          const uint4 g0 = NLDS ? ((const uint4 *)nl)[2 * idx] : n.w[j][0];
+          const uint4 g1 = NLDS ? ((const uint4 *)nl)[2 * idx + 1] : n.w[j][1];
+          const uint32_t g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
+          uint32_t r[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            {
+              const float a = h2f ((uint16_t)(w[i] & 0xffff));
+              const float b = h2f ((uint16_t)(w[i] >> 16));
+              r[i] = (uint32_t)f2h (a * __uint_as_float (g[2 * i]) * alpha)
+                     | ((uint32_t)f2h (b * __uint_as_float (g[2 * i + 1]) * alpha) << 16);
+            }
+          o = make_uint4 (r[0], r[1], r[2], r[3]);
+        }
+      ((uint4 *)xl)[idx] = o;
     }
-  const float total = block_sum (s, red);
-  const float alpha = 1.0f / sqrtf (total / (float)K + eps);
-  for (int i = threadIdx.x; i < K; i += kDecThreads)
-    xl[i] = f2h (h2f (xl[i]) * w[i] * alpha);
   __syncthreads ();
 }
 
@@ -189,216 +349,371 @@ better (float v, uint32_t i, float bv, uint32_t bi)
   return v > bv || (v == bv && i < bi);
 }
 
-// MODE 0: y = x W^T (+ residual);  MODE 1: three matrices, three outputs;
-// MODE 2: y = silu(x W1^T) * (x W0^T)   (W0 = up, W1 = gate)
-template <int MODE, int NMAT, bool COH>
-__device__ __forceinline__ void
-gemv_phase (const QMat *mats, int N, int K, const uint16_t *xl,
-            const Epilogue &e, int wg, int G, float *red)
+// The pipeline's registers: two item buffers shared by every projection phase
+// (each item is 8 dwordx4 weight loads and 8 scales per lane), and the small
+// state of the phase in progress.  Keeping ONE pair of buffers for all phases
+// matters in the persistent kernel, where a phase's first items are issued
+// while the previous phase is still being finished.
+struct PipeBuf
 {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int Kp = ((K + 31) >> 5) << 5, nb = Kp >> 5;
-  const int lo = (int)((long long)N * wg / G) & ~1;
-  int hi = (int)((long long)N * (wg + 1) / G) & ~1;
-  if (wg == G - 1)
-    hi = N;
-  float best_v = -INFINITY;
-  uint32_t best_i = 0xffffffffu;
+  uint4 w[8];
+  uint16_t d[8];
+};
 
-  for (int r0 = lo + 2 * wave; r0 < hi; r0 += 2 * kDecWaves)
-    {
-      const int r1 = min (r0 + 1, N - 1);
-      float acc[NMAT][2];
-#pragma unroll
-      for (int t = 0; t < NMAT; ++t)
-        acc[t][0] = acc[t][1] = 0.f;
-      const size_t q0 = (size_t)r0 * Kp, q1 = (size_t)r1 * Kp;
-      const size_t d0 = (size_t)r0 * nb, d1 = (size_t)r1 * nb;
-#pragma unroll 2
-      for (int kk = lane * 16; kk < Kp; kk += VKL_WAVE * 16)
-        {
-          uint4 w[NMAT][2];
-          uint16_t d[NMAT][2];
-#pragma unroll
-          for (int t = 0; t < NMAT; ++t)
-            {
-              w[t][0] = *(const uint4 *)(mats[t].q + q0 + kk);
-              w[t][1] = *(const uint4 *)(mats[t].q + q1 + kk);
-              d[t][0] = mats[t].d[d0 + (kk >> 5)];
-              d[t][1] = mats[t].d[d1 + (kk >> 5)];
-            }
-          const uint4 *xp = (const uint4 *)(xl + kk);
-          const uint4 x0 = xp[0], x1 = xp[1];
-          const h16x2 xv[8]
-              = { __builtin_bit_cast (h16x2, x0.x), __builtin_bit_cast (h16x2, x0.y),
-                  __builtin_bit_cast (h16x2, x0.z), __builtin_bit_cast (h16x2, x0.w),
-                  __builtin_bit_cast (h16x2, x1.x), __builtin_bit_cast (h16x2, x1.y),
-                  __builtin_bit_cast (h16x2, x1.z), __builtin_bit_cast (h16x2, x1.w) };
-#pragma unroll
-          for (int t = 0; t < NMAT; ++t)
-            {
-              acc[t][0] += dot16_q8 (w[t][0], xv, 0.f) * h2f (d[t][0]);
-              acc[t][1] += dot16_q8 (w[t][1], xv, 0.f) * h2f (d[t][1]);
-            }
-        }
-#pragma unroll
-      for (int t = 0; t < NMAT; ++t)
-        {
-          acc[t][0] = wave_sum (acc[t][0]);
-          acc[t][1] = wave_sum (acc[t][1]);
-        }
-      if (lane != 0)
-        continue;
-      const bool two = r0 + 1 < N;
-      if (MODE == 1)
-        {
-#pragma unroll
-          for (int t = 0; t < NMAT; ++t)
-            {
-              const uint32_t pk = (uint32_t)f2h (acc[t][0])
-                                  | ((uint32_t)f2h (acc[t][1]) << 16);
-              if (two)
-                st_u32<COH> ((uint32_t *)(e.y[t] + r0), pk);
-              else
-                e.y[t][r0] = (uint16_t)pk;
-            }
-          continue;
-        }
-      uint16_t h0, h1;
-      if (MODE == 2)
-        {
-          h0 = f2h (silu (acc[NMAT - 1][0]) * acc[0][0]);
-          h1 = f2h (silu (acc[NMAT - 1][1]) * acc[0][1]);
-        }
-      else
-        {
-          h0 = f2h (acc[0][0]);
-          h1 = f2h (acc[0][1]);
-          if (e.residual)
-            {
-              uint32_t rr;
-              if (two)
-                rr = ld_u32<COH> ((const uint32_t *)(e.residual + r0));
-              else
-                rr = e.residual[r0];
-              h0 = f2h (h2f (h0) + h2f ((uint16_t)(rr & 0xffff)));
-              h1 = f2h (h2f (h1) + h2f ((uint16_t)(rr >> 16)));
-            }
-        }
-      const uint32_t pk = (uint32_t)h0 | ((uint32_t)h1 << 16);
-      if (two)
-        st_u32<COH> ((uint32_t *)(e.y[0] + r0), pk);
-      else
-        e.y[0][r0] = h0;
-      if (MODE == 0 && e.y32)
-        {
-          e.y32[r0] = h2f (h0);
-          if (two)
-            e.y32[r0 + 1] = h2f (h1);
-        }
-      if (MODE == 0 && e.amax_val)
-        {
-          if (better (h2f (h0), (uint32_t)r0, best_v, best_i))
-            best_v = h2f (h0), best_i = (uint32_t)r0;
-          if (two && better (h2f (h1), (uint32_t)r0 + 1, best_v, best_i))
-            best_v = h2f (h1), best_i = (uint32_t)r0 + 1;
-        }
-    }
+struct PipeState
+{
+  // MODE 1 reaches its second and third matrix through byte offsets from the
+  // first: selecting among pointers held here by a runtime index would force
+  // the whole pipeline state out of registers into scratch
+  QMat m0;
+  long long dq1, dq2, dd1, dd2;
+  int mode, N, Kp, nb, nch;
+  int lane, wave, wg;
+  int u_lo, nit, primed;
+  float best_v;
+  uint32_t best_i;
+};
 
-  if (MODE == 0 && e.amax_val)
-    {
-      // lane 0 of each wave holds that wave's best; combine in LDS
-      float *bv = red;
-      uint32_t *bi = (uint32_t *)(red + kDecWaves);
-      __syncthreads ();
-      if (lane == 0)
-        {
-          bv[wave] = best_v;
-          bi[wave] = best_i;
-        }
-      __syncthreads ();
-      if (threadIdx.x == 0)
-        {
-          float v = bv[0];
-          uint32_t i = bi[0];
-          for (int w = 1; w < kDecWaves; ++w)
-            if (better (bv[w], bi[w], v, i))
-              v = bv[w], i = bi[w];
-          st_u32<COH> ((uint32_t *)(e.amax_val + wg), __float_as_uint (v));
-          st_u32<COH> (e.amax_idx + wg, i);
-        }
-    }
-}
+// mode 0: y = x W^T (+ residual); a unit is 2 consecutive rows of m0
+// mode 1: three matrices with three outputs; a unit is 2 rows of one of them
+// mode 2: y = silu(x Wgate^T) * (x Wup^T); a unit is row r of m0 (up) and
+//         row r of m1 (gate); the result goes out as one 32-bit word per
+//         element (fp16 in the low half) so that it can be stored with a
+//         32-bit write-through atomic
+// One copy of the code serves all three (the mode only steers the cheap row
+// addressing and the lane-0 epilogue), which keeps the persistent kernel
+// inside the instruction cache.
+template <bool COH> struct Gemv
+{
+  static constexpr int R = 2; // rows per unit
+  static constexpr int S = 4; // k-steps of 1024 per item
+  static constexpr int CHUNK = S * VKL_WAVE * 16;
+
+  static __device__ __forceinline__ void
+  rows_of (const PipeState &ps, int u, const uint8_t *(&q)[R],
+           const uint16_t *(&d)[R])
+  {
+    const int Kp = ps.Kp, nb = ps.nb;
+    if (ps.mode == 0)
+      {
+        const int r0 = 2 * u;
+        const int r1 = min (r0 + 1, ps.N - 1);
+        q[0] = ps.m0.q + (size_t)r0 * Kp, d[0] = ps.m0.d + (size_t)r0 * nb;
+        q[1] = ps.m0.q + (size_t)r1 * Kp, d[1] = ps.m0.d + (size_t)r1 * nb;
+      }
+    else if (ps.mode == 1)
+      {
+        const int half = ps.N >> 1;
+        const int mat = u / half, r0 = 2 * (u - mat * half);
+        const long long oq = (mat == 1 ? ps.dq1 : 0) + (mat == 2 ? ps.dq2 : 0);
+        const long long od = (mat == 1 ? ps.dd1 : 0) + (mat == 2 ? ps.dd2 : 0);
+        q[0] = ps.m0.q + oq + (size_t)r0 * Kp;
+        d[0] = (const uint16_t *)((const uint8_t *)ps.m0.d + od) + (size_t)r0 * nb;
+        q[1] = q[0] + Kp, d[1] = d[0] + nb;
+      }
+    else
+      {
+        q[0] = ps.m0.q + (size_t)u * Kp, d[0] = ps.m0.d + (size_t)u * nb;
+        q[1] = ps.m0.q + ps.dq1 + (size_t)u * Kp;
+        d[1] = (const uint16_t *)((const uint8_t *)ps.m0.d + ps.dd1) + (size_t)u * nb;
+      }
+  }
+
+  // the range of units of this workgroup / wave; issues the first `depth`
+  // (0..2) items
+  static __device__ __forceinline__ void
+  begin (PipeState &ps, PipeBuf &A, PipeBuf &B, int mode, const QMat a,
+         const QMat b, const QMat c, int N, int K, int wg, int G, int depth)
+  {
+    ps.mode = mode;
+    ps.m0 = a;
+    ps.dq1 = b.q - a.q, ps.dq2 = c.q - a.q;
+    ps.dd1 = (const uint8_t *)b.d - (const uint8_t *)a.d;
+    ps.dd2 = (const uint8_t *)c.d - (const uint8_t *)a.d;
+    ps.N = N;
+    ps.Kp = ((K + 31) >> 5) << 5, ps.nb = ps.Kp >> 5;
+    ps.nch = (ps.Kp + CHUNK - 1) / CHUNK;
+    ps.lane = threadIdx.x & 63, ps.wave = threadIdx.x >> 6, ps.wg = wg;
+    const int U = mode == 0 ? (N + 1) >> 1 : (mode == 1 ? 3 * (N >> 1) : N);
+    const int lo = (int)((unsigned)U * (unsigned)wg / (unsigned)G);
+    const int hi = (int)((unsigned)U * (unsigned)(wg + 1) / (unsigned)G);
+    ps.u_lo = lo + ps.wave;
+    const int nunits
+        = ps.u_lo < hi ? (hi - ps.u_lo + kDecWaves - 1) / kDecWaves : 0;
+    ps.nit = nunits * ps.nch;
+    ps.best_v = -INFINITY, ps.best_i = 0xffffffffu;
+    ps.primed = 0;
+    prime (ps, A, B, depth);
+  }
+
+  // issues the first `depth` (<= 2) items if they are not in flight yet
+  static __device__ __forceinline__ void
+  prime (PipeState &ps, PipeBuf &A, PipeBuf &B, int depth)
+  {
+    if (ps.primed < 1 && depth >= 1 && ps.nit > 0)
+      {
+        issue (ps, A, 0);
+        ps.primed = 1;
+      }
+    if (ps.primed < 2 && depth >= 2 && ps.nit > 1)
+      {
+        issue (ps, B, 1);
+        ps.primed = 2;
+      }
+  }
+
+  static __device__ __forceinline__ void
+  issue (const PipeState &ps, PipeBuf &b, int it)
+  {
+    const int ui = it / ps.nch, c = it - ui * ps.nch;
+    const int u = ps.u_lo + ui * kDecWaves;
+    const uint8_t *q[R];
+    const uint16_t *d[R];
+    rows_of (ps, u, q, d);
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+      {
+        const int kk = c * CHUNK + s * (VKL_WAVE * 16) + ps.lane * 16;
+        const bool ok = kk < ps.Kp;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          {
+            b.w[r * S + s] = ok ? ldg4 (q[r] + kk) : make_uint4 (0, 0, 0, 0);
+            b.d[r * S + s] = ok ? ldg (d[r] + (kk >> 5)) : (uint16_t)0;
+          }
+      }
+  }
+
+  static __device__ __forceinline__ void
+  consume (PipeState &ps, float (&acc)[R], const PipeBuf &b, int it,
+           const uint16_t *xl, const Epilogue &e)
+  {
+    const int ui = it / ps.nch, c = it - ui * ps.nch;
+    if (c == 0)
+      {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          acc[r] = 0.f;
+      }
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+      {
+        const int kk = c * CHUNK + s * (VKL_WAVE * 16) + ps.lane * 16;
+        if (kk < ps.Kp)
+          {
+            const uint4 *xp = (const uint4 *)(xl + kk);
+            const uint4 x0 = xp[0], x1 = xp[1];
+            const h16x2 xv[8]
+                = { __builtin_bit_cast (h16x2, x0.x), __builtin_bit_cast (h16x2, x0.y),
+                    __builtin_bit_cast (h16x2, x0.z), __builtin_bit_cast (h16x2, x0.w),
+                    __builtin_bit_cast (h16x2, x1.x), __builtin_bit_cast (h16x2, x1.y),
+                    __builtin_bit_cast (h16x2, x1.z), __builtin_bit_cast (h16x2, x1.w) };
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+              acc[r] += dot16_q8 (b.w[r * S + s], xv, 0.f) * h2f (b.d[r * S + s]);
+          }
+      }
+    if (c == ps.nch - 1)
+      finish (ps, acc, ps.u_lo + ui * kDecWaves, e);
+  }
+
+  static __device__ __forceinline__ void
+  finish (PipeState &ps, const float (&acc)[R], int u, const Epilogue &e)
+  {
+    float v[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      v[r] = wave_sum (acc[r]);
+    if (ps.lane != 0)
+      return;
+    const int N = ps.N;
+    if (ps.mode == 1)
+      {
+        const int half = N >> 1;
+        const int mat = u / half, r0 = 2 * (u - mat * half);
+        // the three outputs are N elements apart
+        uint16_t *y = e.y[0] + (size_t)mat * N;
+        st_u32<COH> ((uint32_t *)(y + r0),
+                     (uint32_t)f2h (v[0]) | ((uint32_t)f2h (v[1]) << 16));
+        return;
+      }
+    if (ps.mode == 2)
+      {
+        st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[1]) * v[0]));
+        return;
+      }
+    const int r0 = 2 * u;
+    const bool two = r0 + 1 < N;
+    uint16_t h0 = f2h (v[0]), h1 = f2h (v[1]);
+    if (e.residual)
+      {
+        const uint32_t rr
+            = two ? ld_u32<COH> ((const uint32_t *)(e.residual + r0))
+                  : (uint32_t)ldg (e.residual + r0);
+        h0 = f2h (h2f (h0) + h2f ((uint16_t)(rr & 0xffff)));
+        h1 = f2h (h2f (h1) + h2f ((uint16_t)(rr >> 16)));
+      }
+    if (two)
+      st_u32<COH> ((uint32_t *)(e.y[0] + r0), (uint32_t)h0 | ((uint32_t)h1 << 16));
+    else
+      stg (e.y[0] + r0, h0);
+    if (e.y32)
+      {
+        stg (e.y32 + r0, h2f (h0));
+        if (two)
+          stg (e.y32 + r0 + 1, h2f (h1));
+      }
+    if (e.amax_val)
+      {
+        if (better (h2f (h0), (uint32_t)r0, ps.best_v, ps.best_i))
+          ps.best_v = h2f (h0), ps.best_i = (uint32_t)r0;
+        if (two && better (h2f (h1), (uint32_t)r0 + 1, ps.best_v, ps.best_i))
+          ps.best_v = h2f (h1), ps.best_i = (uint32_t)r0 + 1;
+      }
+  }
+
+  // all items; xl must be staged.  `red` = 2*kDecWaves LDS words.
+  static __device__ __forceinline__ void
+  run (PipeState &ps, PipeBuf &A, PipeBuf &B, const uint16_t *xl,
+       const Epilogue &e, float *red)
+  {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      acc[r] = 0.f;
+    prime (ps, A, B, 1);
+    const int nit = ps.nit;
+    for (int it = 0; it < nit; it += 2)
+      {
+        if (it + 1 < nit && !(it == 0 && ps.primed == 2))
+          issue (ps, B, it + 1);
+        consume (ps, acc, A, it, xl, e);
+        if (it + 1 < nit)
+          {
+            if (it + 2 < nit)
+              issue (ps, A, it + 2);
+            consume (ps, acc, B, it + 1, xl, e);
+          }
+      }
+    if (e.amax_val)
+      {
+        // lane 0 of each wave holds that wave's best; combine in LDS
+        float *bv = red;
+        uint32_t *bi = (uint32_t *)(red + kDecWaves);
+        __syncthreads ();
+        if (ps.lane == 0)
+          {
+            bv[ps.wave] = ps.best_v;
+            bi[ps.wave] = ps.best_i;
+          }
+        __syncthreads ();
+        if (threadIdx.x == 0)
+          {
+            float v = bv[0];
+            uint32_t i = bi[0];
+            for (int w = 1; w < kDecWaves; ++w)
+              if (better (bv[w], bi[w], v, i))
+                v = bv[w], i = bi[w];
+            st_u32<COH> ((uint32_t *)(e.amax_val + ps.wg), __float_as_uint (v));
+            st_u32<COH> (e.amax_idx + ps.wg, i);
+          }
+      }
+  }
+};
 
 // ---------------------------------------------------------------------------
 // attention for one head, context length L = pos + 1
 // ---------------------------------------------------------------------------
-// LDS use: qk[3*HD] fp16 (rotated q, rotated k, v), sc[maxlen] fp32, part[...]
+// LDS use: qk[3*HD] fp16 (rotated q, rotated k, v), sc[maxlen] fp32,
+// part[RPB][HD] fp32, red[2*kDecWaves].
 template <int HD, bool COH>
 __device__ __forceinline__ void
 attention_head (const Params &p, const vkl_layer_weights &lw, int head,
                 uint8_t *lds)
 {
-  constexpr int LPR = HD / 8;             // lanes per cache row (16 B each)
-  constexpr int RPB = kDecThreads / LPR;  // rows handled per sweep
+  constexpr int LPR = HD / 8;            // lanes per cache row (16 B each)
+  constexpr int RPB = kDecThreads / LPR; // cache rows per sweep
+  constexpr int PRE = 4;                 // sweeps prefetched up front
   const int dim = p.m.dim, maxlen = p.m.maxlen;
   const uint32_t pos = p.pos;
   const int L = (int)pos + 1;
-  uint16_t *qk = (uint16_t *)lds;                    // [3*HD]
-  float *sc = (float *)(lds + 1024);                 // [maxlen]
-  float *part = sc + maxlen;                         // [RPB][HD]
-  float *red = part + RPB * HD;                      // [2*kDecWaves]
+  uint16_t *qk = (uint16_t *)lds;    // [3*HD]
+  float *sc = (float *)(lds + 1024); // [maxlen]
+  float *part = sc + maxlen;         // [RPB][HD]
+  float *red = part + RPB * HD;      // [2*kDecWaves]
   uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
   uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
   const uint16_t *kin = p.s.kqv + head * HD;
   const uint16_t *qin = p.s.kqv + dim + head * HD;
   const uint16_t *vin = p.s.kqv + 2 * dim + head * HD;
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR, grp = tid / LPR;
+
+  // rows written by earlier steps do not depend on this token: fetch the
+  // first sweeps of K and V before anything else
+  uint4 kpre[PRE], vpre[PRE];
+#pragma unroll
+  for (int j = 0; j < PRE; ++j)
+    {
+      const int l = grp + j * RPB;
+      kpre[j] = vpre[j] = make_uint4 (0, 0, 0, 0);
+      if (l < (int)pos)
+        {
+          kpre[j] = ldg4 (kc + (size_t)l * HD + sub * 8);
+          vpre[j] = ldg4 (vc + (size_t)l * HD + sub * 8);
+        }
+    }
 
   // RoPE on adjacent pairs at position pos; K and V rows go to the cache
-  const int tid = threadIdx.x;
   if (tid < HD) // HD/2 pairs of q, HD/2 pairs of k
     {
       const bool is_k = tid >= HD / 2;
       const int i = is_k ? tid - HD / 2 : tid;
       const uint32_t v = ld_u32<COH> ((const uint32_t *)(is_k ? kin : qin) + i);
-      const float c = p.m.freqc[(size_t)pos * (HD / 2) + i];
-      const float s = p.m.freqs[(size_t)pos * (HD / 2) + i];
+      const float c = ldg (p.m.freqc + (size_t)pos * (HD / 2) + i);
+      const float s = ldg (p.m.freqs + (size_t)pos * (HD / 2) + i);
       const float a = h2f ((uint16_t)(v & 0xffff)), b = h2f ((uint16_t)(v >> 16));
       const uint32_t r = (uint32_t)f2h (a * c - b * s)
                          | ((uint32_t)f2h (a * s + b * c) << 16);
       ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + i] = r;
       if (is_k)
-        ((uint32_t *)(kc + (size_t)pos * HD))[i] = r;
+        stg ((uint32_t *)(kc + (size_t)pos * HD) + i, r);
     }
   else if (tid < HD + HD / 2)
     {
       const int i = tid - HD;
       const uint32_t v = ld_u32<COH> ((const uint32_t *)vin + i);
-      ((uint32_t *)(vc + (size_t)pos * HD))[i] = v;
+      stg ((uint32_t *)(vc + (size_t)pos * HD) + i, v);
       ((uint32_t *)qk)[HD + i] = v;
     }
   __syncthreads ();
 
   // scores[l] = fp16(dot(q, K[l]) / sqrt(HD)); LPR lanes share one cache row
-  const int sub = tid % LPR, grp = tid / LPR;
   const float scale = 1.0f / sqrtf ((float)HD);
   const uint4 qv = ((const uint4 *)qk)[sub];
-  for (int l0 = 0; l0 < L; l0 += RPB)
+  auto score_row = [&] (int l, const uint4 kv) {
+    float s = l < L ? dot8_f16 (qv, kv, 0.f) : 0.f;
+#pragma unroll
+    for (int o = LPR >> 1; o > 0; o >>= 1)
+      s += __shfl_xor (s, o, 64);
+    if (l < L && sub == 0)
+      sc[l] = h2f (f2h (s * scale + 0.f));
+  };
+#pragma unroll
+  for (int j = 0; j < PRE; ++j)
+    {
+      const int l = grp + j * RPB;
+      if (j * RPB < L) // wave-uniform
+        score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kpre[j]);
+    }
+  for (int l0 = PRE * RPB; l0 < L; l0 += RPB)
     {
       const int l = l0 + grp;
-      float s = 0.f;
+      uint4 kv = make_uint4 (0, 0, 0, 0);
       if (l < L)
-        {
-          const uint4 kv = l == (int)pos
-                               ? ((const uint4 *)(qk + HD))[sub]
-                               : ((const uint4 *)(kc + (size_t)l * HD))[sub];
-          s = dot8_f16 (qv, kv, 0.f);
-        }
-#pragma unroll
-      for (int o = LPR >> 1; o > 0; o >>= 1)
-        s += __shfl_xor (s, o, 64);
-      if (l < L && sub == 0)
-        sc[l] = h2f (f2h (s * scale + 0.f));
+        kv = l == (int)pos ? ((const uint4 *)(qk + HD))[sub]
+                           : ldg4 (kc + (size_t)l * HD + sub * 8);
+      score_row (l, kv);
     }
   __syncthreads ();
 
@@ -427,20 +742,27 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
 #pragma unroll
   for (int j = 0; j < 8; ++j)
     acc[j] = 0.f;
-  for (int l = grp; l < L; l += RPB)
-    {
-      const float pl = sc[l];
-      const uint4 vv = l == (int)pos
-                           ? ((const uint4 *)(qk + 2 * HD))[sub]
-                           : ((const uint4 *)(vc + (size_t)l * HD))[sub];
-      const uint32_t w[4] = { vv.x, vv.y, vv.z, vv.w };
+  auto pv_row = [&] (int l, const uint4 vv) {
+    if (l >= L)
+      return;
+    const float pl = sc[l];
+    const uint32_t w[4] = { vv.x, vv.y, vv.z, vv.w };
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        {
-          acc[2 * j] += pl * h2f ((uint16_t)(w[j] & 0xffff));
-          acc[2 * j + 1] += pl * h2f ((uint16_t)(w[j] >> 16));
-        }
+    for (int j = 0; j < 4; ++j)
+      {
+        acc[2 * j] += pl * h2f ((uint16_t)(w[j] & 0xffff));
+        acc[2 * j + 1] += pl * h2f ((uint16_t)(w[j] >> 16));
+      }
+  };
+#pragma unroll
+  for (int j = 0; j < PRE; ++j)
+    {
+      const int l = grp + j * RPB;
+      pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vpre[j]);
     }
+  for (int l = grp + PRE * RPB; l < L; l += RPB)
+    pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub]
+                             : ldg4 (vc + (size_t)l * HD + sub * 8));
 #pragma unroll
   for (int j = 0; j < 8; ++j)
     part[grp * HD + sub * 8 + j] = acc[j];
@@ -463,7 +785,8 @@ __host__ __device__ inline size_t
 lds_bytes_needed (int dim, int ffn, int maxlen, int hd)
 {
   const size_t kmax = (size_t)(dim > ffn ? dim : ffn);
-  const size_t stage = ((kmax + 31) / 32 * 32) * 2 + 256;
+  // staged activation row + reduction words + parked norm weights
+  const size_t stage = ((kmax + 31) / 32 * 32) * 2 + 256 + (size_t)dim * 4;
   const size_t rpb = kDecThreads / (hd / 8);
   const size_t attn = 1024 + (size_t)maxlen * 4 + rpb * hd * 4 + 256;
   return stage > attn ? stage : attn;
@@ -485,46 +808,174 @@ enum Phase
 
 template <bool COH>
 __device__ __forceinline__ void
-run_phase (const Params &p, int layer, int phase, int wg, int G, uint8_t *lds)
+final_argmax (const Params &p, int G, uint8_t *lds)
+{
+  // G per-workgroup partials -> first maximum
+  float v = -INFINITY;
+  uint32_t idx = 0xffffffffu;
+  for (int i = threadIdx.x; i < G; i += kDecThreads)
+    {
+      const float pv = __uint_as_float (
+          ld_u32<COH> ((const uint32_t *)(p.s.amax_val + i)));
+      const uint32_t pi = ld_u32<COH> (p.s.amax_idx + i);
+      if (better (pv, pi, v, idx))
+        v = pv, idx = pi;
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    {
+      const float ov = __shfl_xor (v, o, 64);
+      const uint32_t oi = __shfl_xor (idx, o, 64);
+      if (better (ov, oi, v, idx))
+        v = ov, idx = oi;
+    }
+  float *bv = (float *)lds;
+  uint32_t *bi = (uint32_t *)(lds + 64);
+  if ((threadIdx.x & 63) == 0)
+    {
+      bv[threadIdx.x >> 6] = v;
+      bi[threadIdx.x >> 6] = idx;
+    }
+  __syncthreads ();
+  if (threadIdx.x == 0)
+    {
+      for (int w = 1; w < kDecWaves; ++w)
+        if (better (bv[w], bi[w], v, idx))
+          v = bv[w], idx = bi[w];
+      stg (p.next_tok, idx == 0xffffffffu ? 0u : idx);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// overlapped launches
+// ---------------------------------------------------------------------------
+// In this mode consecutive phases are separate launches on two alternating
+// streams, so the next phase's workgroups become resident while the current
+// phase is still running: they fetch their kernel arguments, warm the
+// instruction cache and put their first two weight items in flight, and only
+// then wait (bounded) for the arrival counter to show that every workgroup of
+// the previous phases has finished.  Each workgroup adds one arrival when its
+// stores are complete.  Activations travel through write-through atomics, as
+// in the persistent kernel.  Wave 0 polls the counter, so it primes its own
+// pipeline after the wait (loads return in order).
+template <bool COH>
+__device__ __forceinline__ void
+phase_wait (const Params &p)
+{
+  if (!COH)
+    return;
+  if (threadIdx.x == 0)
+    {
+      bool ok = false;
+      for (int spin = 0; spin < (1 << 22); ++spin)
+        {
+          const uint32_t v = ld_coherent_u32 (p.s.sync);
+          if ((int32_t)(v - p.wait_target) >= 0)
+            {
+              ok = true;
+              break;
+            }
+          __builtin_amdgcn_s_sleep (1);
+        }
+      if (!ok)
+        st_coherent_u32 (p.s.sync + 1, 1u);
+    }
+  __builtin_amdgcn_s_barrier ();
+}
+
+template <bool COH>
+__device__ __forceinline__ void
+phase_signal (const Params &p)
+{
+  if (!COH)
+    return;
+  __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0): this wave's stores are done
+  __builtin_amdgcn_s_barrier ();
+  if (threadIdx.x == 0)
+    __hip_atomic_fetch_add (p.s.sync, 1u, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Every projection phase runs in this order: activation loads, norm-weight
+// loads, first weight item (all issued back to back), then the activation is
+// normalised / written to LDS, then the weight pipeline runs.
+template <bool COH>
+__device__ __forceinline__ void
+run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
+           int wg, int G, uint8_t *lds)
 {
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
-  const int dimp = ((dim + 31) >> 5) << 5, ffnp = ((ffn + 31) >> 5) << 5;
   uint16_t *xl = (uint16_t *)lds;
-  const int kstage = phase == PH_DOWN ? ffnp : dimp;
-  float *red = (float *)(lds + (size_t)kstage * 2); // 2*kDecWaves floats
+  const int kstage = phase == PH_DOWN ? ffn : dim;
+  float *red = (float *)(lds + (size_t)kstage * 2); // 2*kDecWaves words
+  uint8_t *nl = lds + (size_t)kstage * 2 + 256;     // parked norm weights
   Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
+  // overlapped mode: weights first, then the wait, then the activations
+  const int pre = (threadIdx.x >> 6) == 0 ? 0 : 2;
   switch (phase)
     {
     case PH_KQV:
       {
-        const vkl_layer_weights &lw = m.layers[layer];
+        const QMat wk = qmat (lw.wk, dim, dim), wq = qmat (lw.wq, dim, dim),
+                   wv = qmat (lw.wv, dim, dim);
+        if (COH)
+          {
+            issue_norm (lw.attn_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, pre);
+            stash_norm (nw, dim, nl);
+            phase_wait<COH> (p);
+          }
         if (layer == 0)
           {
-            uint32_t tok = p.tok[0];
+            uint32_t tok = COH ? ld_coherent_u32 (p.tok) : ldg (p.tok);
             if (tok >= (uint32_t)m.vocab)
               tok = 0;
-            stage_embed_q8 (qmat (m.tok_embd, m.vocab, dim), tok, dim, dimp, xl);
-            __syncthreads ();
-            if (wg == 0) // the residual stream starts as the embedding row
-              for (int i = threadIdx.x; i < dim / 2; i += kDecThreads)
-                st_u32<COH> ((uint32_t *)p.s.x + i, ((const uint32_t *)xl)[i]);
+            issue_embed_q8 (qmat (m.tok_embd, m.vocab, dim), tok, dim, x);
+          }
+        else
+          issue_x<COH> (p.s.x, dim, x);
+        if (COH)
+          {
+            Gemv<COH>::prime (ps, A, B, 2);
           }
         else
           {
-            stage_raw<COH> (p.s.x, dim, dimp, xl);
-            __syncthreads ();
+            issue_norm (lw.attn_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1);
           }
-        norm_staged (xl, dim, lw.attn_norm, m.eps, red);
-        const QMat mats[3] = { qmat (lw.wk, dim, dim), qmat (lw.wq, dim, dim),
-                               qmat (lw.wv, dim, dim) };
+        if (layer == 0)
+          {
+            dequant_embed (x);
+            if (wg == 0) // the residual stream starts as the embedding row
+              {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  {
+                    const int idx = threadIdx.x + j * kDecThreads;
+                    if (idx * 8 < dim)
+                      {
+                        uint32_t *dst = (uint32_t *)p.s.x + idx * 4;
+                        st_u32<COH> (dst, x.v[j].x);
+                        st_u32<COH> (dst + 1, x.v[j].y);
+                        st_u32<COH> (dst + 2, x.v[j].z);
+                        st_u32<COH> (dst + 3, x.v[j].w);
+                      }
+                  }
+              }
+          }
+        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
-        gemv_phase<1, 3, COH> (mats, dim, dim, xl, e, wg, G, red);
+        Gemv<COH>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ATTN:
       {
-        const vkl_layer_weights &lw = m.layers[layer];
+        phase_wait<COH> (p);
         for (int h = wg; h < m.n_heads; h += G)
           {
             if (m.head_dim == 128)
@@ -536,95 +987,393 @@ run_phase (const Params &p, int layer, int phase, int wg, int G, uint8_t *lds)
       }
     case PH_WO:
       {
-        const vkl_layer_weights &lw = m.layers[layer];
-        stage_raw<COH> (p.s.att, dim, dimp, xl);
-        __syncthreads ();
-        const QMat mats[1] = { qmat (lw.wo, dim, dim) };
+        VKL_TR (0);
+        const QMat w = qmat (lw.wo, dim, dim);
+        if (COH)
+          {
+            Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre);
+            phase_wait<COH> (p);
+          }
+        issue_x<COH> (p.s.att, dim, x);
+        if (COH)
+          Gemv<COH>::prime (ps, A, B, 2);
+        else
+          Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1);
+        VKL_TR (1);
+        finish_x<false> (x, dim, xl, nw, 0.f, red);
+        VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        gemv_phase<0, 1, COH> (mats, dim, dim, xl, e, wg, G, red);
+        Gemv<COH>::run (ps, A, B, xl, e, red);
+        VKL_TR (4);
         break;
       }
     case PH_UPGATE:
       {
-        const vkl_layer_weights &lw = m.layers[layer];
-        stage_raw<COH> (p.s.x, dim, dimp, xl);
-        __syncthreads ();
-        norm_staged (xl, dim, lw.ffn_norm, m.eps, red);
-        const QMat mats[2] = { qmat (lw.w_up, ffn, dim),
-                               qmat (lw.w_gate, ffn, dim) };
+        VKL_TR (0);
+        const QMat up = qmat (lw.w_up, ffn, dim), gate = qmat (lw.w_gate, ffn, dim);
+        if (COH)
+          {
+            issue_norm (lw.ffn_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, pre);
+            stash_norm (nw, dim, nl);
+            phase_wait<COH> (p);
+          }
+        issue_x<COH> (p.s.x, dim, x);
+        if (COH)
+          {
+            Gemv<COH>::prime (ps, A, B, 2);
+          }
+        else
+          {
+            issue_norm (lw.ffn_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
+          }
+        VKL_TR (1);
+        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl);
+        VKL_TR (3);
         e.y[0] = p.s.t;
-        gemv_phase<2, 2, COH> (mats, ffn, dim, xl, e, wg, G, red);
+        Gemv<COH>::run (ps, A, B, xl, e, red);
+        VKL_TR (4);
         break;
       }
     case PH_DOWN:
       {
-        const vkl_layer_weights &lw = m.layers[layer];
-        stage_raw<COH> (p.s.t, ffn, ffnp, xl);
-        __syncthreads ();
-        const QMat mats[1] = { qmat (lw.w_down, dim, ffn) };
+        const QMat w = qmat (lw.w_down, dim, ffn);
+        if (COH)
+          {
+            Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre);
+            phase_wait<COH> (p);
+          }
+        issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
+        if (COH)
+          Gemv<COH>::prime (ps, A, B, 2);
+        else
+          Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1);
+        finish_x<false> (x, ffn, xl, nw, 0.f, red);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        gemv_phase<0, 1, COH> (mats, dim, ffn, xl, e, wg, G, red);
+        Gemv<COH>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_HEAD:
       {
-        stage_raw<COH> (p.s.x, dim, dimp, xl);
-        __syncthreads ();
-        norm_staged (xl, dim, m.output_norm, m.final_eps, red);
-        const QMat mats[1] = { qmat (m.output, m.vocab, dim) };
+        const QMat w = qmat (m.output, m.vocab, dim);
+        if (COH)
+          {
+            issue_norm (m.output_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, pre);
+            stash_norm (nw, dim, nl);
+            phase_wait<COH> (p);
+          }
+        issue_x<COH> (p.s.x, dim, x);
+        if (COH)
+          {
+            Gemv<COH>::prime (ps, A, B, 2);
+          }
+        else
+          {
+            issue_norm (m.output_norm, dim, nw);
+            Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
+          }
+        finish_x<true, COH> (x, dim, xl, nw, m.final_eps, red, nl);
         e.y[0] = p.s.logits16, e.y32 = p.logits32;
         e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
-        gemv_phase<0, 1, COH> (mats, m.vocab, dim, xl, e, wg, G, red);
+        Gemv<COH>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ARGMAX:
-      {
-        if (wg != 0 || !p.next_tok)
-          break;
-        // G partials -> first maximum
-        float v = -INFINITY;
-        uint32_t idx = 0xffffffffu;
-        for (int i = threadIdx.x; i < G; i += kDecThreads)
-          {
-            const float pv = __uint_as_float (
-                ld_u32<COH> ((const uint32_t *)(p.s.amax_val + i)));
-            const uint32_t pi = ld_u32<COH> (p.s.amax_idx + i);
-            if (better (pv, pi, v, idx))
-              v = pv, idx = pi;
-          }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1)
-          {
-            const float ov = __shfl_xor (v, o, 64);
-            const uint32_t oi = __shfl_xor (idx, o, 64);
-            if (better (ov, oi, v, idx))
-              v = ov, idx = oi;
-          }
-        float *bv = (float *)lds;
-        uint32_t *bi = (uint32_t *)(lds + 64);
-        if ((threadIdx.x & 63) == 0)
-          {
-            bv[threadIdx.x >> 6] = v;
-            bi[threadIdx.x >> 6] = idx;
-          }
-        __syncthreads ();
-        if (threadIdx.x == 0)
-          {
-            for (int w = 1; w < kDecWaves; ++w)
-              if (better (bv[w], bi[w], v, idx))
-                v = bv[w], idx = bi[w];
-            p.next_tok[0] = idx;
-          }
-        break;
-      }
+      phase_wait<COH> (p);
+      if (wg == 0 && p.next_tok)
+        final_argmax<COH> (p, G, lds);
+      break;
     }
+  phase_signal<COH> (p);
 }
 
+template <int PHASE>
 __global__ __launch_bounds__ (kDecThreads) void
-decode_phase_kernel (const Params p, int layer, int phase)
+decode_phase_kernel (const Params p, const vkl_layer_weights lw, int layer,
+                     int G)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
-  run_phase<false> (p, layer, phase, (int)blockIdx.x, (int)gridDim.x, lds);
+  run_phase<false> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
+}
+
+// overlapped launches: two of these are resident per compute unit
+template <int PHASE>
+__global__ __launch_bounds__ (kDecThreads, 4) void
+decode_phase_overlap_kernel (const Params p, const vkl_layer_weights lw,
+                             int layer, int G)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  run_phase<true> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
+}
+
+// ---------------------------------------------------------------------------
+// persistent mode: one launch per token, phases separated by grid barriers
+// ---------------------------------------------------------------------------
+// All G workgroups are resident (G = number of compute units, one workgroup
+// each).  A barrier is a monotonically increasing arrival counter in device
+// memory: workgroup-level s_barrier, one relaxed agent-scope atomic add by
+// thread 0, which then polls the counter (bounded) while the other waves wait
+// on a second s_barrier.  Activations cross the barrier through agent-scope
+// relaxed atomic stores / loads, which bypass the per-XCD L2, so no cache
+// write-back or invalidate is needed.
+//
+// Waves 1..7 issue the first two weight items of the NEXT phase before they
+// enter the barrier, so HBM keeps streaming while the barrier and the
+// activation reload take place; wave 0 (which must read the counter, and whose
+// loads return in order) primes its pipeline after the barrier instead.
+// The per-layer pointer table is read-only for the lifetime of a launch:
+// reading it through the constant address space lets the compiler use scalar
+// loads (SGPR results, tracked by the scalar counter) instead of per-lane
+// vector loads whose wait would also drain every weight load in flight.
+__device__ __forceinline__ vkl_layer_weights
+load_layer (const vkl_layer_weights *table, int layer)
+{
+  typedef const __attribute__ ((address_space (4))) unsigned long long *cptr;
+  cptr t = (cptr) (table + layer);
+  vkl_layer_weights lw;
+  lw.wk = (const void *)t[0], lw.wq = (const void *)t[1];
+  lw.wv = (const void *)t[2], lw.wo = (const void *)t[3];
+  lw.w_gate = (const void *)t[4], lw.w_up = (const void *)t[5];
+  lw.w_down = (const void *)t[6];
+  lw.attn_norm = (const float *)t[7], lw.ffn_norm = (const float *)t[8];
+  lw.kcache = (void *)t[9], lw.vcache = (void *)t[10];
+  return lw;
+}
+
+struct GridSync
+{
+  uint32_t *counter; // arrivals so far
+  uint32_t *error;   // set when a wait gives up
+  uint32_t target;   // arrivals that complete the next barrier
+  uint32_t G;
+};
+
+__device__ __forceinline__ void
+grid_barrier (GridSync &g)
+{
+  // results of this phase were stored with write-through atomics; they are
+  // complete once this wave's vector-memory counter drains (the caller has
+  // not issued the next phase's prefetch yet for wave 0, see above)
+  __builtin_amdgcn_s_barrier ();
+  if (threadIdx.x == 0)
+    {
+      __hip_atomic_fetch_add (g.counter, 1u, __ATOMIC_RELAXED,
+                              __HIP_MEMORY_SCOPE_AGENT);
+      bool ok = false;
+      for (int spin = 0; spin < (1 << 22); ++spin)
+        {
+          const uint32_t v = ld_coherent_u32 (g.counter);
+          if ((int32_t)(v - g.target) >= 0)
+            {
+              ok = true;
+              break;
+            }
+          __builtin_amdgcn_s_sleep (1);
+        }
+      if (!ok)
+        st_coherent_u32 (g.error, 1u);
+    }
+  __builtin_amdgcn_s_barrier ();
+  g.target += g.G;
+}
+
+// stores of this wave complete (and every earlier load consumed)
+__device__ __forceinline__ void
+drain_vmem ()
+{
+  __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0) only
+}
+
+// kinds of phase in the flat sequence [5 per layer] + output layer
+enum Kind
+{
+  K_KQV = 0,
+  K_ATTN,
+  K_WO,
+  K_UPGATE,
+  K_DOWN,
+  K_HEAD
+};
+
+template <int HD>
+__global__ __launch_bounds__ (kDecThreads) void
+decode_mega_kernel (const Params p, int G, uint32_t sync_base)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  const vkl_decode_model &m = p.m;
+  const int wg = (int)blockIdx.x;
+  const int dim = m.dim, ffn = m.ffn, L = m.n_layers;
+  uint16_t *xl = (uint16_t *)lds;
+  GridSync gs = { p.s.sync, p.s.sync + 1, sync_base + (uint32_t)G, (uint32_t)G };
+  const int depth = (threadIdx.x >> 6) == 0 ? 0 : 2; // see the comment above
+
+  PipeState ps;
+  PipeBuf A, B;
+  XRegs x;
+  NormRegs nw;
+
+  // K/Q/V of layer 0 has no barrier in front of it: every wave primes its
+  // pipeline (the activation, the token's embedding row, is fetched in the
+  // loop below like any other)
+  {
+    const vkl_layer_weights lw = load_layer (m.layers, 0);
+    Gemv<true>::begin (ps, A, B, 1, qmat (lw.wk, dim, dim),
+                       qmat (lw.wq, dim, dim), qmat (lw.wv, dim, dim), dim,
+                       dim, wg, G, 2);
+  }
+
+  // Each call below appears once in the loop body on purpose: the compiler
+  // inlines every call site, and the whole kernel has to stay inside the
+  // 64 KiB instruction cache.
+  const int nph = 5 * L + 1;
+  for (int ph = 0; ph < nph; ++ph)
+    {
+      const int layer = ph < 5 * L ? ph / 5 : L - 1;
+      const int kind = ph < 5 * L ? ph - 5 * layer : K_HEAD;
+      const vkl_layer_weights lw = load_layer (m.layers, layer);
+#ifdef VKL_TRACE
+#define VKL_TRM(slot)                                                         \
+  if (threadIdx.x == 0 && p.trace)                                            \
+    p.trace[((size_t)ph * 1024 + wg) * 8 + (slot)] = wall_clock64 ();
+#else
+#define VKL_TRM(slot)
+#endif
+      VKL_TRM (0);
+      if (kind == K_ATTN)
+        {
+          if (wg < m.n_heads)
+            {
+              // nothing is in flight in these workgroups (see below); saying
+              // so lets the attention code use the buffers' registers
+              A = PipeBuf{};
+              B = PipeBuf{};
+              for (int h = wg; h < m.n_heads; h += G)
+                attention_head<HD, true> (p, lw, h, lds);
+            }
+        }
+      else
+        {
+          // activation source, its length, the norm that may precede the
+          // projection, and where the results go
+          const int K = kind == K_DOWN ? ffn : dim;
+          const bool norm = kind == K_KQV || kind == K_UPGATE || kind == K_HEAD;
+          const float *nwp = kind == K_KQV ? lw.attn_norm
+                             : (kind == K_UPGATE ? lw.ffn_norm : m.output_norm);
+          const float eps = kind == K_HEAD ? m.final_eps : m.eps;
+          // x and nw are (re)defined on every path, so neither stays live
+          // around the loop
+          if (ph == 0)
+            {
+              uint32_t tok = ld_coherent_u32 (p.tok);
+              if (tok >= (uint32_t)m.vocab)
+                tok = 0;
+              issue_embed_q8 (qmat (m.tok_embd, m.vocab, dim), tok, dim, x);
+            }
+          else if (kind == K_DOWN)
+            issue_x32<true> ((const uint32_t *)p.s.t, K, x);
+          else
+            issue_x<true> (kind == K_WO ? p.s.att : p.s.x, K, x);
+          if (norm)
+            issue_norm (nwp, dim, nw);
+          else
+            nw = NormRegs{};
+          Gemv<true>::prime (ps, A, B, 2);
+          if (ph == 0)
+            {
+              dequant_embed (x);
+              if (wg == 0) // the residual stream starts as the embedding row
+                {
+#pragma unroll
+                  for (int j = 0; j < 4; ++j)
+                    {
+                      const int idx = threadIdx.x + j * kDecThreads;
+                      if (idx * 8 < dim)
+                        {
+                          uint32_t *dst = (uint32_t *)p.s.x + idx * 4;
+                          st_coherent_u32 (dst, x.v[j].x);
+                          st_coherent_u32 (dst + 1, x.v[j].y);
+                          st_coherent_u32 (dst + 2, x.v[j].z);
+                          st_coherent_u32 (dst + 3, x.v[j].w);
+                        }
+                    }
+                }
+            }
+          float *red = (float *)(lds + (size_t)K * 2);
+          VKL_TRM (1);
+          if (norm)
+            finish_x<true> (x, K, xl, nw, eps, red);
+          else
+            finish_x<false> (x, K, xl, nw, 0.f, red);
+          VKL_TRM (2);
+          Epilogue e = {};
+          if (kind == K_KQV)
+            e.y[0] = p.s.kqv;
+          else if (kind == K_UPGATE)
+            e.y[0] = p.s.t;
+          else if (kind == K_HEAD)
+            {
+              e.y[0] = p.s.logits16, e.y32 = p.logits32;
+              e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
+            }
+          else
+            e.y[0] = p.s.x, e.residual = p.s.x;
+          Gemv<true>::run (ps, A, B, xl, e, red);
+        }
+      VKL_TRM (3);
+      if (ph + 1 == nph)
+        break;
+      // this phase's stores are complete; start the next projection's weights
+      // (after K/Q/V that is Wo, which streams while attention runs)
+      drain_vmem ();
+      VKL_TRM (4);
+      // Workgroups that run an attention head start Wo after it (the
+      // attention code needs the registers the pipeline buffers would hold);
+      // all others start Wo right after K/Q/V.
+      const bool attn_wg = wg < m.n_heads;
+      if (kind == K_ATTN ? attn_wg : !(kind == K_KQV && attn_wg))
+        {
+          int mode = 0, N = dim, K = dim;
+          QMat a, b, c;
+          if (kind == K_KQV || kind == K_ATTN)
+            a = b = c = qmat (lw.wo, dim, dim);
+          else if (kind == K_WO)
+            {
+              mode = 2, N = ffn;
+              a = c = qmat (lw.w_up, ffn, dim);
+              b = qmat (lw.w_gate, ffn, dim);
+            }
+          else if (kind == K_UPGATE)
+            {
+              K = ffn;
+              a = b = c = qmat (lw.w_down, dim, ffn);
+            }
+          else if (layer + 1 < L)
+            {
+              const vkl_layer_weights nx = load_layer (m.layers, layer + 1);
+              mode = 1;
+              a = qmat (nx.wk, dim, dim), b = qmat (nx.wq, dim, dim);
+              c = qmat (nx.wv, dim, dim);
+            }
+          else
+            {
+              N = m.vocab;
+              a = b = c = qmat (m.output, m.vocab, dim);
+            }
+          Gemv<true>::begin (ps, A, B, mode, a, b, c, N, K, wg, G, depth);
+        }
+      VKL_TRM (5);
+      grid_barrier (gs);
+      VKL_TRM (6);
+    }
+  if (p.next_tok)
+    {
+      drain_vmem ();
+      grid_barrier (gs);
+      if (wg == 0)
+        final_argmax<true> (p, G, lds);
+    }
 }
 
 int
@@ -636,13 +1385,165 @@ check_model (const vkl_decode_model *m)
   VKL_CHECK_ARG (m->head_dim == 64 || m->head_dim == 128);
   VKL_CHECK_ARG (m->n_heads * m->head_dim == m->dim);
   VKL_CHECK_ARG ((m->dim % 32) == 0 && (m->ffn % 32) == 0 && m->ffn > 0);
+  VKL_CHECK_ARG (m->dim <= 16384 && m->ffn <= 16384);
   VKL_CHECK_ARG (m->vocab > 0 && (m->vocab % 2) == 0 && m->maxlen > 0);
-  VKL_CHECK_ARG (m->layers && m->tok_embd && m->output && m->output_norm);
+  VKL_CHECK_ARG (m->layers && m->layers_h && m->tok_embd && m->output
+                 && m->output_norm);
   VKL_CHECK_ARG (m->freqc && m->freqs && m->scratch);
   VKL_CHECK_ARG (lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim)
                  <= 160 * 1024);
   return 0;
 }
+
+template <int PHASE>
+int
+launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
+              int grid, int G, size_t lds, hipStream_t s)
+{
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_phase_kernel<PHASE>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  decode_phase_kernel<PHASE>
+      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
+                                                                 G);
+  return 0;
+}
+// The arrival counter in a scratch buffer is never reset; the host keeps the
+// number of arrivals it has scheduled so far (a fresh, zeroed scratch buffer
+// starts a fresh count).
+uint32_t &
+arrivals_of (const void *sync)
+{
+  static const void *seen = nullptr;
+  static uint32_t arrivals = 0;
+  if (seen != sync)
+    {
+      seen = sync;
+      arrivals = 0;
+    }
+  return arrivals;
+}
+
+// Persistent launch.  The grid must be co-resident: one workgroup per compute
+// unit is checked against the occupancy the runtime reports.  The arrival
+// counter is never reset; the host tracks how far it has advanced.
+int
+launch_mega (const Params &p, int G, size_t lds, hipStream_t s)
+{
+  static size_t lds_set = 0;
+  static int resident = -1;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_mega_kernel<64>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_mega_kernel<128>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+      resident = -1;
+    }
+  if (resident < 0)
+    {
+      int per_cu = 0;
+      VKL_HIP (hipOccupancyMaxActiveBlocksPerMultiprocessor (
+          &per_cu, (const void *)decode_mega_kernel<128>, kDecThreads, lds));
+      resident = per_cu;
+    }
+  if (resident < 1)
+    return (int)hipErrorLaunchOutOfResources;
+  uint32_t &arrivals = arrivals_of (p.s.sync);
+  const uint32_t nbar
+      = (uint32_t)(5 * p.m.n_layers + (p.next_tok ? 1 : 0));
+  if (p.m.head_dim == 128)
+    decode_mega_kernel<128><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
+        p, G, arrivals);
+  else
+    decode_mega_kernel<64><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
+        p, G, arrivals);
+  arrivals += nbar * (uint32_t)G;
+  return vkl_launch_status ();
+}
+// Overlapped launches: phases alternate between the caller's stream and a
+// second stream of the library, so two consecutive phases are resident at the
+// same time and hand over through the arrival counter (see phase_wait).
+struct OverlapState
+{
+  hipStream_t second = nullptr;
+  hipEvent_t ev_in = nullptr, ev_out = nullptr;
+};
+
+template <int PHASE>
+int
+launch_overlap (Params &p, const vkl_layer_weights &lw, int layer, int grid,
+                int G, size_t lds, hipStream_t s, uint32_t &arrivals)
+{
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_phase_overlap_kernel<PHASE>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  p.wait_target = arrivals;
+  decode_phase_overlap_kernel<PHASE>
+      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G);
+  arrivals += (uint32_t)grid;
+  return 0;
+}
+
+int
+launch_overlapped_step (Params &p, const vkl_decode_model *m, int G,
+                        size_t lds, hipStream_t s0)
+{
+  static OverlapState st;
+  if (!st.second)
+    {
+      VKL_HIP (hipStreamCreateWithFlags (&st.second, hipStreamNonBlocking));
+      VKL_HIP (hipEventCreateWithFlags (&st.ev_in, hipEventDisableTiming));
+      VKL_HIP (hipEventCreateWithFlags (&st.ev_out, hipEventDisableTiming));
+    }
+  // two workgroups of 512 threads with this much LDS must fit a compute unit
+  VKL_CHECK_ARG (2 * lds <= 160 * 1024);
+  uint32_t &arrivals = arrivals_of (p.s.sync);
+  // the second stream starts after whatever the caller queued before
+  VKL_HIP (hipEventRecord (st.ev_in, s0));
+  VKL_HIP (hipStreamWaitEvent (st.second, st.ev_in, 0));
+  hipStream_t ss[2] = { s0, st.second };
+  int k = 0;
+  for (int l = 0; l < m->n_layers; ++l)
+    {
+      const vkl_layer_weights &lw = m->layers_h[l];
+      if (int e = launch_overlap<PH_KQV> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
+        return e;
+      if (int e = launch_overlap<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads, lds,
+                                           ss[k++ & 1], arrivals))
+        return e;
+      if (int e = launch_overlap<PH_WO> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
+        return e;
+      if (int e = launch_overlap<PH_UPGATE> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
+        return e;
+      if (int e = launch_overlap<PH_DOWN> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
+        return e;
+    }
+  const vkl_layer_weights none = {};
+  if (int e = launch_overlap<PH_HEAD> (p, none, 0, G, G, lds, ss[k++ & 1], arrivals))
+    return e;
+  if (p.next_tok)
+    if (int e = launch_overlap<PH_ARGMAX> (p, none, 0, 1, G, lds, ss[k++ & 1], arrivals))
+      return e;
+  // later work on the caller's stream follows both streams
+  VKL_HIP (hipEventRecord (st.ev_out, st.second));
+  VKL_HIP (hipStreamWaitEvent (s0, st.ev_out, 0));
+  return vkl_launch_status ();
+}
+
 } // namespace
 } // namespace vkl
 
@@ -664,6 +1565,15 @@ vkl_decode_logits_f16 (const vkl_decode_model *m)
   return carve (m->scratch, m->dim, m->ffn, m->vocab).logits16;
 }
 
+#ifdef VKL_TRACE
+static unsigned long long *g_trace = nullptr;
+extern "C" void
+vkl_debug_set_trace (void *buf)
+{
+  g_trace = (unsigned long long *)buf;
+}
+#endif
+
 extern "C" int
 vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
                  int mode, float *logits32, uint32_t *next_tok, void *stream)
@@ -671,9 +1581,8 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (int e = check_model (m))
     return e;
   VKL_CHECK_ARG (tok != nullptr && pos < (uint32_t)m->maxlen);
-  VKL_CHECK_ARG (mode == 0);
+  VKL_CHECK_ARG (mode >= 0 && mode <= 2);
   static int n_cu = 0;
-  static size_t lds_set = 0;
   if (n_cu == 0)
     {
       int dev = 0;
@@ -683,13 +1592,6 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
     }
   const size_t lds
       = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_kernel,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
   Params p;
   p.m = *m;
   p.s = carve (m->scratch, m->dim, m->ffn, m->vocab);
@@ -697,15 +1599,37 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.pos = pos;
   p.logits32 = logits32 ? logits32 : p.s.logits32;
   p.next_tok = next_tok;
+#ifdef VKL_TRACE
+  p.trace = g_trace;
+#endif
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid ((unsigned)n_cu), block (kDecThreads);
+  const int G = n_cu;
+  p.wait_target = 0;
+  if (mode == 1)
+    return launch_mega (p, G, lds, s);
+  if (mode == 2)
+    return launch_overlapped_step (p, m, G, lds, s);
   for (int l = 0; l < m->n_layers; ++l)
-    for (int ph = PH_KQV; ph <= PH_DOWN; ++ph)
-      decode_phase_kernel<<<ph == PH_ATTN ? dim3 ((unsigned)m->n_heads) : grid,
-                            block, lds, s>>> (p, l, ph);
-  decode_phase_kernel<<<grid, block, lds, s>>> (p, 0, PH_HEAD);
+    {
+      const vkl_layer_weights &lw = m->layers_h[l];
+      if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e
+          = launch_phase<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads, lds, s))
+        return e;
+      if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s))
+        return e;
+    }
+  const vkl_layer_weights none = {};
+  if (int e = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s))
+    return e;
   if (next_tok)
-    decode_phase_kernel<<<dim3 (1), block, lds, s>>> (p, 0, PH_ARGMAX);
+    if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
+      return e;
   return vkl_launch_status ();
 }
 

@@ -55,7 +55,8 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
       return absl::OkStatus ();
     }
 
-  std::vector<vkl_layer_weights> lw (blocks.size ());
+  std::vector<vkl_layer_weights> &lw = layers_h_;
+  lw.assign (blocks.size (), vkl_layer_weights{});
   for (size_t i = 0; i < blocks.size (); ++i)
     {
       auto *a = blocks[i]->attention ();
@@ -92,6 +93,7 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
   desc_.eps = eps;
   desc_.final_eps = out->norm ()->eps ();
   desc_.layers = (const vkl_layer_weights *)layers_.data ();
+  desc_.layers_h = layers_h_.data ();
   desc_.tok_embd = emb.data ();
   desc_.output = out->weight ().data ();
   desc_.output_norm = (const float *)out->norm ()->weight ().data ();

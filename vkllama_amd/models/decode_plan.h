@@ -42,6 +42,7 @@ private:
   int mode_;
   vkl_decode_model desc_;
   Tensor layers_;   // device array of vkl_layer_weights
+  std::vector<vkl_layer_weights> layers_h_; // host mirror
   Tensor scratch_;
   Tensor logits32_; // fp32 [vocab] written by the fused step
   Tensor tok_slot_; // pinned uint32
