@@ -160,7 +160,7 @@ def test_errors(small):
         M.Llama2(cfg, short)
 
 
-@pytest.mark.parametrize("mode", [1])
+@pytest.mark.parametrize("mode", [1, 2])
 @pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5), (TINY, 1234)])
 def test_other_decode_modes_match_oracle(cfg, seed, mode):
     """decode_mode 1: one persistent launch per token with grid barriers;

@@ -1413,25 +1413,17 @@ launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
                                                                  G);
   return 0;
 }
-// The arrival counter in a scratch buffer is never reset; the host keeps the
-// number of arrivals it has scheduled so far (a fresh, zeroed scratch buffer
-// starts a fresh count).
-uint32_t &
-arrivals_of (const void *sync)
+// The arrival counter of a scratch buffer restarts from zero with every token:
+// a one-thread kernel in front of the step clears it (a fill kernel rather
+// than a memset node, so that a caller may capture the step in a graph).
+__global__ void
+reset_arrivals_kernel (uint32_t *sync)
 {
-  static const void *seen = nullptr;
-  static uint32_t arrivals = 0;
-  if (seen != sync)
-    {
-      seen = sync;
-      arrivals = 0;
-    }
-  return arrivals;
+  st_coherent_u32 (sync, 0u);
 }
 
 // Persistent launch.  The grid must be co-resident: one workgroup per compute
-// unit is checked against the occupancy the runtime reports.  The arrival
-// counter is never reset; the host tracks how far it has advanced.
+// unit is checked against the occupancy the runtime reports.
 int
 launch_mega (const Params &p, int G, size_t lds, hipStream_t s)
 {
@@ -1457,16 +1449,13 @@ launch_mega (const Params &p, int G, size_t lds, hipStream_t s)
     }
   if (resident < 1)
     return (int)hipErrorLaunchOutOfResources;
-  uint32_t &arrivals = arrivals_of (p.s.sync);
-  const uint32_t nbar
-      = (uint32_t)(5 * p.m.n_layers + (p.next_tok ? 1 : 0));
+  reset_arrivals_kernel<<<dim3 (1), dim3 (1), 0, s>>> (p.s.sync);
   if (p.m.head_dim == 128)
     decode_mega_kernel<128><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
-        p, G, arrivals);
+        p, G, 0u);
   else
     decode_mega_kernel<64><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
-        p, G, arrivals);
-  arrivals += nbar * (uint32_t)G;
+        p, G, 0u);
   return vkl_launch_status ();
 }
 // Overlapped launches: phases alternate between the caller's stream and a
@@ -1511,7 +1500,8 @@ launch_overlapped_step (Params &p, const vkl_decode_model *m, int G,
     }
   // two workgroups of 512 threads with this much LDS must fit a compute unit
   VKL_CHECK_ARG (2 * lds <= 160 * 1024);
-  uint32_t &arrivals = arrivals_of (p.s.sync);
+  uint32_t arrivals = 0;
+  reset_arrivals_kernel<<<dim3 (1), dim3 (1), 0, s0>>> (p.s.sync);
   // the second stream starts after whatever the caller queued before
   VKL_HIP (hipEventRecord (st.ev_in, s0));
   VKL_HIP (hipStreamWaitEvent (st.second, st.ev_in, 0));
@@ -1603,7 +1593,10 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.trace = g_trace;
 #endif
   hipStream_t s = (hipStream_t)stream;
-  const int G = n_cu;
+  // launch-per-phase: two workgroups per compute unit (their registers and
+  // LDS fit side by side), which doubles the weight bytes in flight while the
+  // activation row is still being staged
+  const int G = mode == 0 ? n_cu * 2 : n_cu;
   p.wait_target = 0;
   if (mode == 1)
     return launch_mega (p, G, lds, s);
