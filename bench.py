@@ -10,9 +10,14 @@ tokens (K = 256 by default, contexts 33 .. 32+K).
 Prints ONE JSON line.  `value` is decode tokens per second with weights and
 KV cache resident in HBM, timed across the K steps between device
 synchronisations, including the on-device arg-max and the token hand-over.
-`roofline` prices the decode step against the 8 TB/s HBM peak with the
-algorithmic bytes per token; `cpu_baseline` is the CPU oracle timed on this
-box's host cores on a bounded sample.
+`roofline` covers the dominant kernel of the step (the phase kernel with the
+largest share of the step time, in practice the fused up/gate projection):
+algorithmic bytes of one launch divided by the average launch duration, which
+is measured with HIP event pairs on the launch stream in a second pass over
+the same K steps (the events would perturb the throughput pass).  The same
+object also carries the whole step priced the same way (`step_*`).
+`cpu_baseline` is the CPU oracle timed on this box's host cores on a bounded
+sample.
 """
 import argparse
 import json
@@ -35,6 +40,10 @@ WORKLOADS = {
                                     eps=1e-5, wtype=8, prompt=3968, prefill_kv=1),
 }
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of a kernel from hardware counters (FETCH_SIZE +
+# WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
+# filled in from the counter runs whose summaries are kept under profiles/
+TRAFFIC = {}
 
 
 def cpu_baseline(cfg, weights, n_tokens):
@@ -100,6 +109,22 @@ def main():
     step_bytes = float(np.mean([m.decode_step_bytes(int(L)) for L in (ctx[0], ctx[-1])]))
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # second pass over the same steps with an event pair around every phase launch
+    m.set_option("phase_timing", 1)
+    m.phase_times()
+    m.generate_greedy(prompt, steps + 1)
+    m.set_option("phase_timing", 0)
+    phases = m.phase_times()
+    L_mid = int(ctx[len(ctx) // 2])
+    per_phase = {}
+    for name, (ms, n) in phases.items():
+        if n:
+            per_phase[name] = {"launches_per_step": n // steps, "avg_us": round(ms * 1e3 / n, 3),
+                               "us_per_step": round(ms * 1e3 / steps, 1),
+                               "bytes_per_launch": m.phase_bytes(name, L_mid)}
+    dom = max(per_phase, key=lambda k: per_phase[k]["us_per_step"])
+    dom_gbs = per_phase[dom]["bytes_per_launch"] / (per_phase[dom]["avg_us"] * 1e-6) / 1e9
+
     result = {
         "metric": "decode_tokens_per_second_bs1",
         "value": round(tok_s, 2),
@@ -117,10 +142,14 @@ def main():
                    "decode_mode": ("launch-per-phase", "persistent", "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "decode step (all phases of one token)",
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get((args.workload, dom)),
+                     "kernel": "decode_phase_kernel<%s>" % dom,
+                     "avg_launch_us": per_phase[dom]["avg_us"],
+                     "bytes_per_launch": per_phase[dom]["bytes_per_launch"],
+                     "step_achieved": round(achieved, 1), "step_frac": round(achieved / HBM_PEAK_GBS, 4),
                      "bytes_per_step": int(step_bytes)},
+        "phases": per_phase,
         "load_seconds": {"synthesize": round(t_synth, 1), "upload": round(t_load, 1)},
         "first_ids": [int(t) for t in ids[:8]],
     }
@@ -128,7 +157,7 @@ def main():
 
     cpu_tokens = args.cpu_tokens
     if cpu_tokens < 0:
-        cpu_tokens = 8 if cfg["dim"] >= 4096 else 64
+        cpu_tokens = 128 if cfg["dim"] >= 4096 else 1024
     if cpu_tokens > 0:
         v, dt = cpu_baseline(cfg, weights, cpu_tokens)
         result["cpu_baseline"] = {

@@ -62,6 +62,22 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
                      uint32_t pos, int mode, float *logits32,
                      uint32_t *next_tok, void *stream);
 
+/* Phase timing (mode 0 only; a measuring aid without counterpart in the
+ * reference, whose GPUDevice timestamps play this role in
+ * src/core/gpu_device.cpp).  While enabled, vkl_decode_step brackets every
+ * phase launch with a pair of HIP events on the launch stream and
+ * synchronises the stream before it returns.  vkl_decode_phase_times adds up,
+ * per phase kind (0 K/Q/V, 1 attention, 2 Wo, 3 up/gate, 4 down, 5 lm_head,
+ * 6 arg-max), the elapsed milliseconds and the number of launches since the
+ * last call, and clears both. */
+#define VKL_DECODE_PHASES 7
+int vkl_decode_phase_timing (int enable);
+int vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
+                            uint64_t launches[VKL_DECODE_PHASES]);
+/* algorithmic bytes one launch of phase `kind` moves at context length L
+ * (weights + scales read once; activations, KV rows and results once) */
+size_t vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L);
+
 /* device pointer to the fp16 logits [vocab] of the last step inside scratch */
 const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
 /* arg-max over fp32 values (first maximum); out is device-visible */

@@ -59,13 +59,17 @@ int vkl_model_generate_greedy (vkl_model *m, const uint32_t *prompt_h,
                                uint32_t *out_ids_h, double *prefill_ms,
                                double *decode_ms);
 /* options: fused one-token decode on/off, decode launch mode (0 = one launch
- * per phase, 1 = persistent), the reference's last-block RoPE position quirk */
+ * per phase, 1 = persistent, 2 = overlapped launches), the reference's last-block RoPE position quirk */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);
 /* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */
 int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,
                              uint16_t *out_h, size_t n);
 /* algorithmic bytes of one decode step at context length L */
 size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
+/* per-phase measurements of the fused decode step: option "phase_timing"
+ * switches them on; see vkl_decode_phase_times / vkl_decode_phase_bytes */
+int vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7]);
+size_t vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L);
 
 /* ---- synthetic weights (seeded, host) ----------------------------------
  * N(0, std) values from a counter-based generator: element i of stream

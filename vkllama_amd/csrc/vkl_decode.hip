@@ -21,6 +21,7 @@
 // activations (a few KiB) come from L2.
 #include "../../include/vkl_decode.h"
 #include "vkl_decode_dev.h"
+#include <vector>
 
 namespace vkl
 {
@@ -1395,11 +1396,64 @@ check_model (const vkl_decode_model *m)
   return 0;
 }
 
+// phase timing: event pairs recorded around launches, read back after the
+// step's stream synchronisation
+struct PhaseTimer
+{
+  bool on = false;
+  std::vector<hipEvent_t> pool; // start/stop pairs
+  std::vector<int> kind;        // phase kind of pair i of the current step
+  double ms[VKL_DECODE_PHASES] = {};
+  uint64_t n[VKL_DECODE_PHASES] = {};
+};
+PhaseTimer g_timer;
+
+int
+timer_mark (int kind, bool stop, hipStream_t s)
+{
+  PhaseTimer &t = g_timer;
+  if (!t.on)
+    return 0;
+  const size_t i = stop ? t.kind.size () - 1 : t.kind.size ();
+  if (!stop)
+    {
+      t.kind.push_back (kind);
+      while (t.pool.size () < 2 * t.kind.size ())
+        {
+          hipEvent_t e;
+          VKL_HIP (hipEventCreate (&e));
+          t.pool.push_back (e);
+        }
+    }
+  VKL_HIP (hipEventRecord (t.pool[2 * i + (stop ? 1 : 0)], s));
+  return 0;
+}
+
+int
+timer_collect (hipStream_t s)
+{
+  PhaseTimer &t = g_timer;
+  if (!t.on)
+    return 0;
+  VKL_HIP (hipStreamSynchronize (s));
+  for (size_t i = 0; i < t.kind.size (); ++i)
+    {
+      float ms = 0.f;
+      VKL_HIP (hipEventElapsedTime (&ms, t.pool[2 * i], t.pool[2 * i + 1]));
+      t.ms[t.kind[i]] += ms;
+      t.n[t.kind[i]] += 1;
+    }
+  t.kind.clear ();
+  return 0;
+}
+
 template <int PHASE>
 int
 launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
               int grid, int G, size_t lds, hipStream_t s)
 {
+  if (int e = timer_mark (PHASE, false, s))
+    return e;
   static size_t lds_set = 0;
   if (lds > lds_set)
     {
@@ -1411,7 +1465,7 @@ launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
   decode_phase_kernel<PHASE>
       <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
                                                                  G);
-  return 0;
+  return timer_mark (PHASE, true, s);
 }
 // The arrival counter of a scratch buffer restarts from zero with every token:
 // a one-thread kernel in front of the step clears it (a fill kernel rather
@@ -1623,7 +1677,57 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (next_tok)
     if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
       return e;
+  if (int e = timer_collect (s))
+    return e;
   return vkl_launch_status ();
+}
+
+extern "C" int
+vkl_decode_phase_timing (int enable)
+{
+  g_timer.on = enable != 0;
+  g_timer.kind.clear ();
+  return 0;
+}
+
+extern "C" int
+vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
+                        uint64_t launches[VKL_DECODE_PHASES])
+{
+  VKL_CHECK_ARG (ms_sum && launches);
+  for (int i = 0; i < VKL_DECODE_PHASES; ++i)
+    {
+      ms_sum[i] = g_timer.ms[i], launches[i] = g_timer.n[i];
+      g_timer.ms[i] = 0.0, g_timer.n[i] = 0;
+    }
+  return 0;
+}
+
+extern "C" size_t
+vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L)
+{
+  if (!m || kind < 0 || kind >= VKL_DECODE_PHASES)
+    return 0;
+  const size_t dim = (size_t)m->dim, ffn = (size_t)m->ffn, V = (size_t)m->vocab;
+  // a Q8_0 matrix [N, K]: N*K quants + N*K/32 fp16 scales
+  auto mat = [] (size_t N, size_t K) { return N * K + N * (K / 32) * 2; };
+  switch (kind)
+    {
+    case PH_KQV: // x + norm weights in, three projections out
+      return 3 * mat (dim, dim) + dim * 2 + dim * 4 + 3 * dim * 2;
+    case PH_ATTN: // q/k/v in, K and V rows of L positions, new rows, output
+      return 3 * dim * 2 + 2 * L * dim * 2 + 2 * dim * 2 + dim * 2;
+    case PH_WO:
+      return mat (dim, dim) + dim * 2 + 2 * dim * 2;
+    case PH_UPGATE:
+      return 2 * mat (ffn, dim) + dim * 2 + dim * 4 + ffn * 4;
+    case PH_DOWN:
+      return mat (dim, ffn) + ffn * 4 + 2 * dim * 2;
+    case PH_HEAD:
+      return mat (V, dim) + dim * 2 + dim * 4 + V * 2 + V * 4;
+    default:
+      return (size_t)1024 * 8;
+    }
 }
 
 namespace

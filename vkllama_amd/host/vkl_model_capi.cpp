@@ -2,6 +2,7 @@
 // (include/vkl_model.h).
 #include "vkl_model.h"
 #include "models/llama2.h"
+#include "vkl_decode.h"
 #include "vkl_hip.h"
 #include <cmath>
 #include <map>
@@ -165,6 +166,8 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_lastblock_rope_quirk (value != 0);
   else if (n == "decode_mode")
     m->model->set_decode_mode (value);
+  else if (n == "phase_timing")
+    vkl_decode_phase_timing (value);
   else
     return fail (m, absl::InvalidArgumentError ("unknown option " + n));
   return 0;
@@ -190,6 +193,22 @@ extern "C" size_t
 vkl_model_decode_step_bytes (const vkl_model *m, size_t L)
 {
   return m && m->model ? m->model->decode_step_bytes (L) : 0;
+}
+
+extern "C" int
+vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7])
+{
+  if (!m || !ms_sum || !launches)
+    return (int)absl::StatusCode::kInvalidArgument;
+  return vkl_decode_phase_times (ms_sum, launches) == 0
+             ? 0
+             : (int)absl::StatusCode::kInternal;
+}
+
+extern "C" size_t
+vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L)
+{
+  return m && m->model ? m->model->decode_phase_bytes (kind, L) : 0;
 }
 
 // ---------------------------------------------------------------------------

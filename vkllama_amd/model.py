@@ -31,6 +31,8 @@ SIGNATURES = {
     "vkl_model_set_option": (i32, [vp, C.c_char_p, i32]),
     "vkl_model_read_kv_cache": (i32, [vp, sz, i32, vp, sz]),
     "vkl_model_decode_step_bytes": (sz, [vp, sz]),
+    "vkl_model_phase_times": (i32, [vp, vp, vp]),
+    "vkl_model_phase_bytes": (sz, [vp, i32, sz]),
     "vkl_synth_normal_f32": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_f16": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_q8_0": (None, [u64, sz, sz, C.c_float, vp]),
@@ -169,6 +171,19 @@ class Llama2:
 
     def decode_step_bytes(self, L):
         return int(lib().vkl_model_decode_step_bytes(self._h, L))
+
+    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax")
+
+    def phase_times(self):
+        """{phase: (milliseconds summed, launches)} since the last call; filled
+        while the option "phase_timing" is on."""
+        ms = np.zeros(7, np.float64)
+        n = np.zeros(7, np.uint64)
+        self._check(lib().vkl_model_phase_times(self._h, ms.ctypes.data, n.ctypes.data), "phase_times")
+        return {k: (float(ms[i]), int(n[i])) for i, k in enumerate(self.PHASES)}
+
+    def phase_bytes(self, kind, L):
+        return int(lib().vkl_model_phase_bytes(self._h, self.PHASES.index(kind), L))
 
 
 TINY_SMOKE_CFG = dict(dim=256, n_layers=2, n_heads=4, ffn=704, vocab=1024, maxlen=64, eps=1e-5, wtype=8)

@@ -26,6 +26,7 @@ struct DecodePlan
   // true when the fused kernels cover this model (Q8_0, head width 64/128)
   bool usable () const { return usable_; }
   void set_mode (int mode) { mode_ = mode; }
+  const vkl_decode_model &desc () const { return desc_; }
   // token id given by the host / read from device-visible memory
   absl::Status step_host_token (uint32_t tok, size_t offset);
   absl::Status step_device_token (const uint32_t *tok, size_t offset);

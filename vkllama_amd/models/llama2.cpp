@@ -557,4 +557,12 @@ Model::decode_step_bytes (size_t L) const
   const size_t kv = blocks_.size () * 2 * dim_ * 2;
   return wbytes + norm + emb + kv * L + kv;
 }
+
+size_t
+Model::decode_phase_bytes (int kind, size_t L) const
+{
+  if (!plan_ || !plan_->usable ())
+    return 0;
+  return vkl_decode_phase_bytes (&plan_->desc (), kind, L);
+}
 }

@@ -175,6 +175,8 @@ public:
   size_t block_count () const { return blocks_.size (); }
   // algorithmic bytes one decode step at context length L reads and writes
   size_t decode_step_bytes (size_t L) const;
+  // algorithmic bytes of one launch of a decode phase (see vkl_decode.h)
+  size_t decode_phase_bytes (int kind, size_t L) const;
 
 private:
   absl::StatusOr<Tensor> forward_ (std::vector<uint32_t> const &toks,
