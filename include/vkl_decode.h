@@ -74,6 +74,17 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
 int vkl_decode_phase_timing (int enable);
 int vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
                             uint64_t launches[VKL_DECODE_PHASES]);
+/* Launches phase `kind` (0..4: of every layer in turn; 5: lm_head) `rounds`
+ * times back to back on `stream` between ONE pair of events and returns the
+ * average milliseconds per launch: the kernel's duration without the cost of
+ * an event pair per launch.  The phase's outputs in scratch are overwritten
+ * (a following vkl_decode_step recomputes them); the KV cache is not touched
+ * for kinds other than 1, and kind 1 rewrites the rows of position `pos` with
+ * what scratch currently holds, so call it before, not between, real steps of
+ * a sequence you still need. */
+int vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
+                             int rounds, void *stream, double *avg_ms,
+                             uint64_t *launches);
 /* algorithmic bytes one launch of phase `kind` moves at context length L
  * (weights + scales read once; activations, KV rows and results once) */
 size_t vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L);

@@ -70,6 +70,9 @@ size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
  * switches them on; see vkl_decode_phase_times / vkl_decode_phase_bytes */
 int vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7]);
 size_t vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L);
+/* vkl_decode_phase_replay on this model's stream; overwrites decode scratch */
+int vkl_model_phase_replay (vkl_model *m, int kind, size_t pos, int rounds,
+                            double *avg_ms, uint64_t *launches);
 
 /* ---- synthetic weights (seeded, host) ----------------------------------
  * N(0, std) values from a counter-based generator: element i of stream

@@ -1703,6 +1703,91 @@ vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
   return 0;
 }
 
+extern "C" int
+vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
+                         int rounds, void *stream, double *avg_ms,
+                         uint64_t *launches)
+{
+  if (int e = check_model (m))
+    return e;
+  VKL_CHECK_ARG (kind >= PH_KQV && kind <= PH_HEAD && rounds > 0 && avg_ms);
+  VKL_CHECK_ARG (pos < (uint32_t)m->maxlen);
+  int dev = 0, n_cu = 0;
+  VKL_HIP (hipGetDevice (&dev));
+  VKL_HIP (hipDeviceGetAttribute (&n_cu, hipDeviceAttributeMultiprocessorCount,
+                                  dev));
+  const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
+  Params p;
+  p.m = *m;
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab);
+  p.tok = (const uint32_t *)p.s.amax_idx; // any device word: ids >= vocab read row 0
+  p.pos = pos;
+  p.logits32 = p.s.logits32;
+  p.next_tok = nullptr;
+  p.wait_target = 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int G = n_cu * 2;
+  const bool was_on = g_timer.on;
+  g_timer.on = false;
+  hipEvent_t e0, e1;
+  VKL_HIP (hipEventCreate (&e0));
+  VKL_HIP (hipEventCreate (&e1));
+  uint64_t n = 0;
+  int err = 0;
+  VKL_HIP (hipEventRecord (e0, s));
+  for (int r = 0; r < rounds && !err; ++r)
+    {
+      if (kind == PH_HEAD)
+        {
+          const vkl_layer_weights none = {};
+          err = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s), ++n;
+          continue;
+        }
+      for (int l = 0; l < m->n_layers && !err; ++l, ++n)
+        {
+          const vkl_layer_weights &lw = m->layers_h[l];
+          // layer 0's K/Q/V reads the embedding row instead of the residual
+          // stream; replay it as an inner layer so every launch is alike
+          const int li = kind == PH_KQV && l == 0 ? 1 : l;
+          switch (kind)
+            {
+            case PH_KQV:
+              err = launch_phase<PH_KQV> (p, lw, li, G, G, lds, s);
+              break;
+            case PH_ATTN:
+              err = launch_phase<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads,
+                                           lds, s);
+              break;
+            case PH_WO:
+              err = launch_phase<PH_WO> (p, lw, l, G, G, lds, s);
+              break;
+            case PH_UPGATE:
+              err = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s);
+              break;
+            default:
+              err = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s);
+              break;
+            }
+        }
+    }
+  hipError_t e = hipEventRecord (e1, s);
+  if (e == hipSuccess)
+    e = hipEventSynchronize (e1);
+  float ms = 0.f;
+  if (e == hipSuccess)
+    e = hipEventElapsedTime (&ms, e0, e1);
+  (void)hipEventDestroy (e0);
+  (void)hipEventDestroy (e1);
+  g_timer.on = was_on;
+  if (err)
+    return err;
+  VKL_HIP (e);
+  *avg_ms = n ? (double)ms / (double)n : 0.0;
+  if (launches)
+    *launches = n;
+  return vkl_launch_status ();
+}
+
 extern "C" size_t
 vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L)
 {

@@ -205,6 +205,16 @@ vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7])
              : (int)absl::StatusCode::kInternal;
 }
 
+extern "C" int
+vkl_model_phase_replay (vkl_model *m, int kind, size_t pos, int rounds,
+                        double *avg_ms, uint64_t *launches)
+{
+  if (!m || !m->model || !avg_ms)
+    return (int)absl::StatusCode::kInvalidArgument;
+  auto s = m->model->decode_phase_replay (kind, pos, rounds, avg_ms, launches);
+  return s.ok () ? 0 : fail (m, s);
+}
+
 extern "C" size_t
 vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L)
 {

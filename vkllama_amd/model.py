@@ -33,6 +33,7 @@ SIGNATURES = {
     "vkl_model_decode_step_bytes": (sz, [vp, sz]),
     "vkl_model_phase_times": (i32, [vp, vp, vp]),
     "vkl_model_phase_bytes": (sz, [vp, i32, sz]),
+    "vkl_model_phase_replay": (i32, [vp, i32, sz, i32, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
     "vkl_synth_normal_f32": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_f16": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_q8_0": (None, [u64, sz, sz, C.c_float, vp]),
@@ -181,6 +182,14 @@ class Llama2:
         n = np.zeros(7, np.uint64)
         self._check(lib().vkl_model_phase_times(self._h, ms.ctypes.data, n.ctypes.data), "phase_times")
         return {k: (float(ms[i]), int(n[i])) for i, k in enumerate(self.PHASES)}
+
+    def phase_replay(self, kind, pos, rounds):
+        """Average microseconds per launch of one phase kernel launched back
+        to back (all layers, `rounds` times) between one pair of HIP events."""
+        ms, n = C.c_double(0), C.c_uint64(0)
+        self._check(lib().vkl_model_phase_replay(self._h, self.PHASES.index(kind), pos, rounds, C.byref(ms),
+                                                 C.byref(n)), "phase_replay")
+        return ms.value * 1e3, int(n.value)
 
     def phase_bytes(self, kind, L):
         return int(lib().vkl_model_phase_bytes(self._h, self.PHASES.index(kind), L))

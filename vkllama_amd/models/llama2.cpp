@@ -566,3 +566,22 @@ Model::decode_phase_bytes (int kind, size_t L) const
   return vkl_decode_phase_bytes (&plan_->desc (), kind, L);
 }
 }
+
+namespace vkllama
+{
+absl::Status
+Model::decode_phase_replay (int kind, size_t pos, int rounds, double *avg_ms,
+                            uint64_t *launches)
+{
+  if (!plan_ || !plan_->usable ())
+    return absl::FailedPreconditionError (
+        "fused decode does not cover this model");
+  const int e = vkl_decode_phase_replay (&plan_->desc (), kind, (uint32_t)pos,
+                                         rounds, gpu_->stream (), avg_ms,
+                                         launches);
+  if (e)
+    return absl::InternalError (
+        absl::StrFormat ("phase replay failed: %s", vkl_error_string (e)));
+  return absl::OkStatus ();
+}
+}

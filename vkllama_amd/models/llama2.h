@@ -177,6 +177,8 @@ public:
   size_t decode_step_bytes (size_t L) const;
   // algorithmic bytes of one launch of a decode phase (see vkl_decode.h)
   size_t decode_phase_bytes (int kind, size_t L) const;
+  absl::Status decode_phase_replay (int kind, size_t pos, int rounds,
+                                    double *avg_ms, uint64_t *launches);
 
 private:
   absl::StatusOr<Tensor> forward_ (std::vector<uint32_t> const &toks,
