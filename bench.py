@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of a kernel from hardware counters (FETCH_SIZE +
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
-TRAFFIC = {}
+TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96258458}
 
 
 def cpu_baseline(cfg, weights, n_tokens):
@@ -71,6 +71,9 @@ def main():
     ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS))
     ap.add_argument("--decode-mode", type=int, default=0)
     ap.add_argument("--cpu-tokens", type=int, default=-1, help="decode tokens of the CPU baseline (0 = skip)")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
+                    help="before the timed region, launch the library's copy kernel N times on 1 GiB "
+                         "(the known-size launch that traffic counters are scaled by)")
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -96,6 +99,15 @@ def main():
     m = M.Llama2(cfg, weights)
     m.set_option("decode_mode", args.decode_mode)
     t_load = time.perf_counter() - t0
+
+    if args.copy_calibration > 0:
+        dev = capi.Device(0)
+        a, b = dev.alloc(1 << 30), dev.alloc(1 << 30)
+        a.zero()
+        for _ in range(args.copy_calibration):
+            capi.check(capi.lib().vkl_copy_kernel(b.ptr, a.ptr, 1 << 30, dev.stream), "vkl_copy_kernel")
+        dev.sync()
+        a.free(), b.free()
 
     # warm-up: prompt pass + W decode steps, untimed
     m.generate_greedy(prompt, warmup + 1)

@@ -58,6 +58,10 @@ int vkl_memcpy_h2d (void *dst, const void *src_h, size_t bytes, void *stream);
 int vkl_memcpy_d2h (void *dst_h, const void *src, size_t bytes, void *stream);
 int vkl_memcpy_d2d (void *dst, const void *src, size_t bytes, void *stream);
 int vkl_memset (void *dst, int value, size_t bytes, void *stream);
+/* device-to-device copy by a plain streaming kernel (bytes % 16 == 0, both
+ * pointers 16-byte aligned): the known-size launch that hardware traffic
+ * counters are calibrated against; no counterpart in the reference */
+int vkl_copy_kernel (void *dst, const void *src, size_t bytes, void *stream);
 /* timing: replaces the timestamp queries of src/core/pipeline.cpp:425-445 */
 int vkl_event_create (void **ev);
 int vkl_event_destroy (void *ev);

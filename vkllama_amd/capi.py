@@ -40,6 +40,7 @@ SIGNATURES = {
     "vkl_memcpy_d2h": (i32, [vp, vp, sz, vp]),
     "vkl_memcpy_d2d": (i32, [vp, vp, sz, vp]),
     "vkl_memset": (i32, [vp, i32, sz, vp]),
+    "vkl_copy_kernel": (i32, [vp, vp, sz, vp]),
     "vkl_event_create": (i32, [C.POINTER(vp)]),
     "vkl_event_destroy": (i32, [vp]),
     "vkl_event_record": (i32, [vp, vp]),

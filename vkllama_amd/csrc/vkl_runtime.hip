@@ -133,6 +133,31 @@ vkl_memcpy_d2d (void *dst, const void *src, size_t bytes, void *stream)
   return 0;
 }
 
+// A plain streaming copy (16 bytes per lane and iteration).  It is the unit
+// against which hardware traffic counters are calibrated: one launch reads
+// and writes exactly `n16` * 16 bytes.
+__global__ __launch_bounds__ (512) void
+copy_bytes_kernel (const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                   size_t n16)
+{
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += stride)
+    dst[i] = src[i];
+}
+
+int
+vkl_copy_kernel (void *dst, const void *src, size_t bytes, void *stream)
+{
+  VKL_CHECK_ARG (dst && src && (bytes % 16) == 0);
+  VKL_CHECK_ARG (((uintptr_t)dst % 16) == 0 && ((uintptr_t)src % 16) == 0);
+  if (bytes == 0)
+    return 0;
+  copy_bytes_kernel<<<dim3 (2048), dim3 (512), 0, (hipStream_t)stream>>> (
+      (const uint4 *)src, (uint4 *)dst, bytes / 16);
+  return vkl_launch_status ();
+}
+
 __global__ void
 fill_bytes_kernel (uint8_t *dst, uint8_t v, size_t n)
 {
