@@ -142,6 +142,17 @@ def main():
     dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
     dom_gbs = per_phase[dom]["bytes_per_launch"] / (dom_us * 1e-6) / 1e9
 
+    # the same loop through Model::operator() (token id from the host, 128 KB of
+    # logits back to the host per token, host arg-max): the PCIe-inclusive rate
+    n_host = min(32, steps)
+    logits = m.forward(prompt, 0)
+    tok, pos = int(np.argmax(logits)), n_prompt
+    t0 = time.perf_counter()
+    for _ in range(n_host):
+        logits = m.forward([tok], pos)
+        tok, pos = int(np.argmax(logits)), pos + 1
+    host_tok_s = n_host / (time.perf_counter() - t0)
+
     result = {
         "metric": "decode_tokens_per_second_bs1",
         "value": round(tok_s, 2),
@@ -158,6 +169,7 @@ def main():
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
                    "decode_mode": ("launch-per-phase", "persistent", "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
+        "decode_tokens_per_second_host_interface": round(host_tok_s, 1),
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get((args.workload, dom)),
