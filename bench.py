@@ -134,13 +134,21 @@ def main():
             per_phase[name] = {"launches_per_step": n // steps, "avg_us": round(ms * 1e3 / n, 3),
                                "us_per_step": round(ms * 1e3 / steps, 1),
                                "bytes_per_launch": m.phase_bytes(name, L_mid)}
-    dom = max(per_phase, key=lambda k: per_phase[k]["us_per_step"])
-    # the dominant kernel again, launched back to back (every layer's weights in
-    # turn) between ONE event pair: its duration without a pair's own cost
-    rounds = max(2, steps // 8)
-    m.phase_replay(dom, L_mid - 1, 1)
-    dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
-    dom_gbs = per_phase[dom]["bytes_per_launch"] / (dom_us * 1e-6) / 1e9
+    if per_phase:
+        dom = max(per_phase, key=lambda k: per_phase[k]["us_per_step"])
+        # the dominant kernel again, launched back to back (every layer's weights
+        # in turn) between ONE event pair: its duration without a pair's own cost
+        rounds = max(2, steps // 8)
+        m.phase_replay(dom, L_mid - 1, 1)
+        dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
+        dom_bytes = per_phase[dom]["bytes_per_launch"]
+        dom_kernel, dom_pair_us = "decode_phase_kernel<%s>" % dom, per_phase[dom]["avg_us"]
+    else:
+        # persistent / overlapped modes: one launch (or one overlapped train of
+        # launches) per token, priced as a whole
+        dom, dom_us, dom_n, dom_bytes = None, ms_per_step * 1e3, steps, step_bytes
+        dom_kernel, dom_pair_us = "decode step (all phases of one token)", None
+    dom_gbs = dom_bytes / (dom_us * 1e-6) / 1e9
 
     # the same loop through Model::operator() (token id from the host, 128 KB of
     # logits back to the host per token, host arg-max): the PCIe-inclusive rate
@@ -173,10 +181,10 @@ def main():
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get((args.workload, dom)),
-                     "kernel": "decode_phase_kernel<%s>" % dom,
+                     "kernel": dom_kernel,
                      "avg_launch_us": round(dom_us, 3), "launches_timed": dom_n,
-                     "avg_launch_us_with_event_pair": per_phase[dom]["avg_us"],
-                     "bytes_per_launch": per_phase[dom]["bytes_per_launch"],
+                     "avg_launch_us_with_event_pair": dom_pair_us,
+                     "bytes_per_launch": int(dom_bytes),
                      "step_achieved": round(achieved, 1), "step_frac": round(achieved / HBM_PEAK_GBS, 4),
                      "bytes_per_step": int(step_bytes)},
         "phases": per_phase,

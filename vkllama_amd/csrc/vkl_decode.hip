@@ -85,8 +85,11 @@ struct Params
   if (threadIdx.x == 0 && p.trace)                                            \
     p.trace[((size_t)(layer * 8 + phase) * 1024 + wg) * 8 + (slot)]           \
         = wall_clock64 ();
+#define VKL_TRP                                                               \
+  (p.trace ? p.trace + ((size_t)(layer * 8 + phase) * 1024 + wg) * 8 : nullptr)
 #else
 #define VKL_TR(slot)
+#define VKL_TRP nullptr
 #endif
 
 // ---------------------------------------------------------------------------
@@ -280,9 +283,18 @@ stash_norm (const NormRegs &n, int K, uint8_t *nl)
 template <bool NORM, bool NLDS = false>
 __device__ __forceinline__ void
 finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
-          float *red, const uint8_t *nl = nullptr)
+          float *red, const uint8_t *nl = nullptr,
+          unsigned long long *tr = nullptr)
 {
   float alpha = 0.f;
+#ifdef VKL_TRACE
+  if (tr && threadIdx.x == 0)
+    {
+      // x has arrived once its first word can be read
+      asm volatile("" ::"v"(x.v[0].x), "v"(x.v[3].w));
+      tr[1] = wall_clock64 ();
+    }
+#endif
   if (NORM)
     {
       float s = 0.f;
@@ -300,6 +312,10 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
             }
         }
       const float total = block_sum (s, red);
+#ifdef VKL_TRACE
+      if (tr && threadIdx.x == 0)
+        tr[3] = wall_clock64 ();
+#endif
       alpha = 1.0f / sqrtf (total / (float)K + eps);
     }
 #pragma unroll
@@ -918,6 +934,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
   PipeBuf A, B;
   // overlapped mode: weights first, then the wait, then the activations
   const int pre = (threadIdx.x >> 6) == 0 ? 0 : 2;
+  VKL_TR (0);
   switch (phase)
     {
     case PH_KQV:
@@ -930,6 +947,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             Gemv<COH>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
+            VKL_TR (5);
           }
         if (layer == 0)
           {
@@ -969,7 +987,8 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
                   }
               }
           }
-        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl);
+        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
+        VKL_TR (2);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
         Gemv<COH>::run (ps, A, B, xl, e, red);
         break;
@@ -977,6 +996,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
     case PH_ATTN:
       {
         phase_wait<COH> (p);
+            VKL_TR (5);
         for (int h = wg; h < m.n_heads; h += G)
           {
             if (m.head_dim == 128)
@@ -988,29 +1008,26 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
       }
     case PH_WO:
       {
-        VKL_TR (0);
         const QMat w = qmat (lw.wo, dim, dim);
         if (COH)
           {
             Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre);
             phase_wait<COH> (p);
+            VKL_TR (5);
           }
         issue_x<COH> (p.s.att, dim, x);
         if (COH)
           Gemv<COH>::prime (ps, A, B, 2);
         else
           Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1);
-        VKL_TR (1);
-        finish_x<false> (x, dim, xl, nw, 0.f, red);
+        finish_x<false> (x, dim, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
         Gemv<COH>::run (ps, A, B, xl, e, red);
-        VKL_TR (4);
         break;
       }
     case PH_UPGATE:
       {
-        VKL_TR (0);
         const QMat up = qmat (lw.w_up, ffn, dim), gate = qmat (lw.w_gate, ffn, dim);
         if (COH)
           {
@@ -1018,6 +1035,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
+            VKL_TR (5);
           }
         issue_x<COH> (p.s.x, dim, x);
         if (COH)
@@ -1029,12 +1047,10 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             issue_norm (lw.ffn_norm, dim, nw);
             Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
           }
-        VKL_TR (1);
-        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl);
-        VKL_TR (3);
+        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
+        VKL_TR (2);
         e.y[0] = p.s.t;
         Gemv<COH>::run (ps, A, B, xl, e, red);
-        VKL_TR (4);
         break;
       }
     case PH_DOWN:
@@ -1044,13 +1060,15 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
           {
             Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre);
             phase_wait<COH> (p);
+            VKL_TR (5);
           }
         issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
         if (COH)
           Gemv<COH>::prime (ps, A, B, 2);
         else
           Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1);
-        finish_x<false> (x, ffn, xl, nw, 0.f, red);
+        finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
+        VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
         Gemv<COH>::run (ps, A, B, xl, e, red);
         break;
@@ -1064,6 +1082,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
+            VKL_TR (5);
           }
         issue_x<COH> (p.s.x, dim, x);
         if (COH)
@@ -1075,7 +1094,8 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             issue_norm (m.output_norm, dim, nw);
             Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
           }
-        finish_x<true, COH> (x, dim, xl, nw, m.final_eps, red, nl);
+        finish_x<true, COH> (x, dim, xl, nw, m.final_eps, red, nl, VKL_TRP);
+        VKL_TR (2);
         e.y[0] = p.s.logits16, e.y32 = p.logits32;
         e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
         Gemv<COH>::run (ps, A, B, xl, e, red);
@@ -1083,11 +1103,14 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
       }
     case PH_ARGMAX:
       phase_wait<COH> (p);
+            VKL_TR (5);
       if (wg == 0 && p.next_tok)
         final_argmax<COH> (p, G, lds);
       break;
     }
+  VKL_TR (4);
   phase_signal<COH> (p);
+  VKL_TR (6);
 }
 
 template <int PHASE>

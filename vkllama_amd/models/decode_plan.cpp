@@ -121,7 +121,8 @@ DecodePlan::step_host_token (uint32_t tok, size_t offset)
 }
 
 absl::Status
-DecodePlan::step_device_token (const uint32_t *tok, size_t offset)
+DecodePlan::step_device_token (const uint32_t *tok, size_t offset,
+                               uint32_t *next_tok)
 {
   if (!usable_)
     return absl::FailedPreconditionError (
@@ -129,7 +130,7 @@ DecodePlan::step_device_token (const uint32_t *tok, size_t offset)
   adopted_valid_ = false;
   return hip_status ("decode step",
                      vkl_decode_step (&desc_, tok, (uint32_t)offset, mode_,
-                                      (float *)logits32_.data (), nullptr,
+                                      (float *)logits32_.data (), next_tok,
                                       gpu_->stream ()));
 }
 

@@ -29,7 +29,9 @@ struct DecodePlan
   const vkl_decode_model &desc () const { return desc_; }
   // token id given by the host / read from device-visible memory
   absl::Status step_host_token (uint32_t tok, size_t offset);
-  absl::Status step_device_token (const uint32_t *tok, size_t offset);
+  // next_tok (optional, device-visible): receives the arg-max id of this step
+  absl::Status step_device_token (const uint32_t *tok, size_t offset,
+                                  uint32_t *next_tok = nullptr);
   // copies the fp32 logits of the last step (fused or adopted) to the host
   absl::Status read_logits (float *dst);
   // remember the fp32 logits tensor of an operator-chain pass

@@ -472,11 +472,12 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
         prompt.size (), n_gen, maxlen_));
   if (!plan_)
     return absl::InternalError ("model used before init()");
-  // generated ids live in pinned host memory that the device writes
+  // generated ids stay in device memory between steps (the arg-max of step i
+  // is the input token of step i + 1) and are copied out once at the end
   if (next_tok_.width () < n_gen)
     {
       VKLLAMA_STATUS_OK (output_command_->wait ());
-      next_tok_ = Tensor (1, 1, n_gen, gpu_, UINT32, true);
+      next_tok_ = Tensor (1, 1, n_gen, gpu_, UINT32, false);
       VKLLAMA_STATUS_OK (next_tok_.create ());
     }
   uint32_t *ids = (uint32_t *)next_tok_.data ();
@@ -503,14 +504,19 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
     {
       if (fused_decode_ && plan_->usable ())
         {
+          // the step's last launch reduces the arg-max partials into ids[i]
           VKLLAMA_STATUS_OK (
-              plan_->step_device_token (ids + (i - 1), n_toks - 1));
+              plan_->step_device_token (ids + (i - 1), n_toks - 1, ids + i));
+          continue;
         }
       else
         {
+          uint32_t prev = 0;
+          if (int e = vkl_memcpy_d2h (&prev, ids + (i - 1), sizeof (prev), s))
+            return absl::InternalError (vkl_error_string (e));
           if (int e = vkl_stream_sync (s))
             return absl::InternalError (vkl_error_string (e));
-          auto logits32 = forward_ ({ ids[i - 1] }, n_toks - 1);
+          auto logits32 = forward_ ({ prev }, n_toks - 1);
           VKLLAMA_STATUS_OK (logits32);
           VKLLAMA_STATUS_OK (plan_->adopt_logits (*logits32));
         }
@@ -524,7 +530,11 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
   for (auto *c : block_commands_)
     VKLLAMA_STATUS_OK (c->wait ());
   VKLLAMA_STATUS_OK (output_command_->wait ());
-  out.assign (ids, ids + n_gen);
+  out.resize (n_gen);
+  if (int e = vkl_memcpy_d2h (out.data (), ids, n_gen * sizeof (uint32_t), s))
+    return absl::InternalError (vkl_error_string (e));
+  if (int e = vkl_stream_sync (s))
+    return absl::InternalError (vkl_error_string (e));
   if (prefill_ms)
     *prefill_ms = std::chrono::duration<double, std::milli> (t1 - t0).count ();
   if (decode_ms)
