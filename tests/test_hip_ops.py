@@ -136,6 +136,71 @@ def test_matmul_q8_0_epilogue(dev, rng):
     assert np.array_equal(got32, got.astype(np.float32))  # the widening cast is exact
 
 
+# ------------------------------------------------- prompt-pass GEMM (MFMA) --
+@pytest.mark.parametrize("M,N,K", [(9, 128, 32), (16, 130, 512), (64, 256, 4096), (100, 200, 1376), (300, 1376, 512),
+                                   (129, 64, 11008), (65, 32000, 512)])
+def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
+    """M >= 9 token rows run on the matrix cores (weights dequantised to
+    fp16(q*d) on the way into LDS, fp32 accumulation)."""
+    raw, deq = q8_weights(rng, N, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    got = _run_matmul_q8(dev, x, raw, N, K)
+    if M * N * K <= 3e8:
+        want = O.matmul_q8_0(x, raw, K)
+        assert rel_err(got, want) < F16_REL_TOL
+    exact = x.astype(np.float64) @ deq[:, :K].T
+    assert rel_err(got, exact) < 2e-3
+
+
+def test_gemm_q8_0_epilogue_and_strides(dev, rng):
+    M, N, K = 40, 200, 512
+    raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    got = _run_matmul_q8(dev, x, raw, N, K, scale=0.5, bias=0.25, act=1)
+    assert rel_err(got, O.matmul_q8_0(x, raw, K, 0.5, 0.25, 1)) < F16_REL_TOL
+    got, got32 = _run_matmul_q8(dev, x, raw, N, K, residual=res, want32=True)
+    want = O.elementwise(O.matmul_q8_0(x, raw, K), res, 0)
+    assert rel_err(got, want) < F16_REL_TOL
+    assert np.array_equal(got32, got.astype(np.float32))
+    # rows of x and y embedded in wider buffers
+    xs, ys = K + 64, N + 8
+    xw = np.zeros((M, xs), np.float16)
+    xw[:, :K] = x
+    dx, dw = dev.upload(xw), dev.upload_q8_0(raw, N, K)
+    dy = dev.alloc(M * ys * 2)
+    dy.zero()
+    capi.check(L().vkl_matmul_q8_0(dx.ptr, dw.ptr, M, N, K, xs, ys, 1.0, 0.0, 0, None, dy.ptr, None, dev.stream))
+    yw = f16(dy, (M, ys))
+    assert rel_err(yw[:, :N], O.matmul_q8_0(x, raw, K)) < F16_REL_TOL
+    assert not yw[:, N:].any()
+
+
+@pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376)])
+def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
+    ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dx = dev.upload(x)
+    dws = [dev.upload_q8_0(w, N, K) for w in ws]
+    outs = [dev.alloc(M * N * 2) for _ in range(3)]
+    capi.check(L().vkl_kqv_q8_0(dx.ptr, dws[0].ptr, dws[1].ptr, dws[2].ptr, M, N, K, outs[0].ptr, outs[1].ptr,
+                                outs[2].ptr, dev.stream))
+    want = O.kqv_q8_0(x, ws[0], ws[1], ws[2], K)
+    for o, w in zip(outs, want):
+        assert rel_err(f16(o, (M, N)), w) < F16_REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512)])
+def test_ffn_upgate_q8_0_many_rows(dev, rng, M, N, K):
+    up, _ = q8_weights(rng, N, K)
+    gate, _ = q8_weights(rng, N, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dx, dup, dg = dev.upload(x), dev.upload_q8_0(up, N, K), dev.upload_q8_0(gate, N, K)
+    out = dev.alloc(M * N * 2)
+    capi.check(L().vkl_ffn_upgate_q8_0(dx.ptr, dup.ptr, dg.ptr, M, N, K, out.ptr, dev.stream))
+    assert rel_err(f16(out, (M, N)), O.ffn_upgate_q8_0(x, up, gate, K)) < F16_REL_TOL
+
+
 def test_kqv_q8_0(dev, rng):
     M, N, K = 3, 512, 512
     ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
@@ -172,6 +237,33 @@ def test_matmul_f16_tb(dev, rng, C, M, N, K):
     capi.check(L().vkl_matmul_f16_tb(da.ptr, db.ptr, C, M, N, K, M * K, K, N * K, K, M * N, N, 0.125, 0.0, 0,
                                      None, dy.ptr, None, dev.stream))
     assert rel_err(f16(dy, (C, M, N)), O.matmul_f16_tb(a, b, scale=0.125)) < F16_REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512)])
+def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
+    """FP16 weights, many token rows: the matrix-core path."""
+    a = rng.standard_normal((1, M, K)).astype(np.float16)
+    b = (rng.standard_normal((1, N, K)) * 0.05).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    da, db, dr = dev.upload(a), dev.upload(b), dev.upload(res)
+    dy, d32 = dev.alloc(M * N * 2), dev.alloc(M * N * 4)
+    capi.check(L().vkl_matmul_f16_tb(da.ptr, db.ptr, 1, M, N, K, M * K, K, N * K, K, M * N, N, 1.0, 0.0, 0,
+                                     dr.ptr, dy.ptr, d32.ptr, dev.stream))
+    want = O.elementwise(O.matmul_f16_tb(a, b)[0], res, 0)
+    got = f16(dy, (M, N))
+    assert rel_err(got, want) < F16_REL_TOL
+    assert np.array_equal(d32.read(np.float32, (M, N)), got.astype(np.float32))
+
+
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (130, 96, 4096)])
+def test_ffn_upgate_f16_many_rows(dev, rng, M, N, K):
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    up = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    gate = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    dx, du, dg = dev.upload(x), dev.upload(up), dev.upload(gate)
+    out = dev.alloc(M * N * 2)
+    capi.check(L().vkl_ffn_upgate_f16(dx.ptr, du.ptr, dg.ptr, M, N, K, out.ptr, dev.stream))
+    assert rel_err(f16(out, (M, N)), O.ffn_upgate_f16(x, up, gate)) < F16_REL_TOL
 
 
 def test_matmul_f16_tb_reads_cache_view(dev, rng):

@@ -1,0 +1,41 @@
+// Internal interface of the MFMA GEMM used for prompt passes (many token
+// rows): y[M,N] = x[M,K] W[N,K]^T with fp16 activations and either planar
+// Q8_0 or dense fp16 weights.  Called by the extern "C" launchers in
+// vkl_gemv_q8.hip and vkl_matmul_f16.hip when M is large enough.
+#ifndef VKL_GEMM_H
+#define VKL_GEMM_H
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace vkl
+{
+struct GemmArgs
+{
+  const uint16_t *x; // [M, K] fp16, row stride xs (elements)
+  size_t xs;
+  int M, N, K;       // K: valid columns of x
+  int Kp;            // K rounded up to 32 (rows of the int8 plane)
+  int wtype;         // 8 = planar Q8_0, 1 = fp16
+  int nmat;          // 1, or 3 independent matrices/outputs (grid z)
+  int upgate;        // 1: w[0] = up, w[1] = gate, y = silu(x gate^T) * (x up^T)
+  const uint8_t *wq[3];  // Q8_0: int8 planes [N, Kp]
+  const uint16_t *wd[3]; // Q8_0: fp16 scale planes [N, Kp/32]
+  const uint16_t *wh[3]; // fp16: [N, K], row stride ws
+  size_t ws;
+  uint16_t *y[3]; // [M, N] fp16, row stride ys
+  size_t ys;
+  float scale, bias;
+  int act;                  // 1: SiLU
+  const uint16_t *residual; // y = fp16(fp16(v) + residual), stride ys
+  float *y32;               // dense [M, N] widened copy
+};
+
+// smallest M for which the GEMM beats re-streaming the weights per 4 rows
+constexpr int kGemmMinRows = 9;
+
+// true if the shapes/alignments are ones the kernel covers
+bool gemm_mfma_supported (const GemmArgs &a);
+int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
+}
+#endif

@@ -8,6 +8,7 @@
 // weights, nothing is read twice at M <= MT.
 #include "../../include/vkl_hip.h"
 #include "vkl_common.h"
+#include "vkl_gemm.h"
 
 namespace
 {
@@ -208,6 +209,27 @@ fill_common (GemvQ8Args &a, const void *x, int M, int N, int K, size_t xs,
   return 0;
 }
 
+// the same problem on the matrix cores when there are enough token rows
+bool
+try_gemm (const GemvQ8Args &a, int nmat, int upgate, hipStream_t s, int &err)
+{
+  if (a.M < vkl::kGemmMinRows)
+    return false;
+  vkl::GemmArgs g = {};
+  g.x = a.x, g.xs = a.xs;
+  g.M = a.M, g.N = a.N, g.K = a.K, g.Kp = a.Kp;
+  g.wtype = 8, g.nmat = nmat, g.upgate = upgate;
+  for (int t = 0; t < 3; ++t)
+    g.wq[t] = a.wq[t], g.wd[t] = a.wd[t], g.y[t] = a.y[t];
+  g.ys = a.ys;
+  g.scale = a.scale, g.bias = a.bias, g.act = a.act;
+  g.residual = a.residual, g.y32 = a.y32;
+  if (!vkl::gemm_mfma_supported (g))
+    return false;
+  err = vkl::gemm_mfma_launch (g, s);
+  return true;
+}
+
 void
 set_mat (GemvQ8Args &a, int t, const void *w, void *y)
 {
@@ -236,6 +258,9 @@ vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
   a.act = act;
   a.residual = (const uint16_t *)residual;
   a.y32 = y32;
+  int err = 0;
+  if (try_gemm (a, 1, 0, (hipStream_t)stream, err))
+    return err;
   return launch<0, 1> (a, (hipStream_t)stream);
 }
 
@@ -250,6 +275,9 @@ vkl_kqv_q8_0 (const void *x, const void *wk, const void *wq, const void *wv,
   set_mat (a, 0, wk, k);
   set_mat (a, 1, wq, q);
   set_mat (a, 2, wv, v);
+  int err = 0;
+  if (try_gemm (a, 3, 0, (hipStream_t)stream, err))
+    return err;
   return launch<1, 3> (a, (hipStream_t)stream);
 }
 
@@ -266,5 +294,8 @@ vkl_ffn_upgate_q8_0 (const void *x, const void *wup, const void *wgate, int M,
   a.wq[2] = a.wq[0];
   a.wd[2] = a.wd[0];
   a.y[2] = a.y[0];
+  int err = 0;
+  if (try_gemm (a, 1, 1, (hipStream_t)stream, err))
+    return err;
   return launch<2, 2> (a, (hipStream_t)stream);
 }

@@ -6,6 +6,7 @@
 // KV cache in place.
 #include "../../include/vkl_hip.h"
 #include "vkl_common.h"
+#include "vkl_gemm.h"
 
 namespace
 {
@@ -178,6 +179,22 @@ vkl_matmul_f16_tb (const void *a, const void *b, int C, int M, int N, int K,
   p.C = C, p.M = M, p.N = N, p.K = K;
   p.acs = acs, p.ahs = ahs, p.bcs = bcs, p.bhs = bhs, p.ycs = ycs, p.yhs = yhs;
   p.scale = scale, p.bias = bias, p.act = act;
+  if (C == 1 && M >= vkl::kGemmMinRows)
+    {
+      // a projection over many token rows: matrix cores
+      vkl::GemmArgs g = {};
+      g.x = p.a, g.xs = ahs;
+      g.M = M, g.N = N, g.K = K, g.Kp = (K + 31) / 32 * 32;
+      g.wtype = 1, g.nmat = 1, g.upgate = 0;
+      g.wh[0] = g.wh[1] = g.wh[2] = p.b;
+      g.ws = bhs;
+      g.y[0] = g.y[1] = g.y[2] = p.y;
+      g.ys = yhs;
+      g.scale = scale, g.bias = bias, g.act = act;
+      g.residual = p.residual, g.y32 = y32;
+      if (vkl::gemm_mfma_supported (g))
+        return vkl::gemm_mfma_launch (g, (hipStream_t)stream);
+    }
   return launch_tb (p, false, (hipStream_t)stream);
 }
 
@@ -195,6 +212,20 @@ vkl_ffn_upgate_f16 (const void *x, const void *wup, const void *wgate, int M,
   p.acs = 0, p.ahs = (size_t)K, p.bcs = 0, p.bhs = (size_t)K;
   p.ycs = 0, p.yhs = (size_t)N;
   p.scale = 1.f, p.bias = 0.f, p.act = 0;
+  if (M >= vkl::kGemmMinRows)
+    {
+      vkl::GemmArgs g = {};
+      g.x = p.a, g.xs = (size_t)K;
+      g.M = M, g.N = N, g.K = K, g.Kp = (K + 31) / 32 * 32;
+      g.wtype = 1, g.nmat = 1, g.upgate = 1;
+      g.wh[0] = g.wh[2] = p.b, g.wh[1] = p.b2;
+      g.ws = (size_t)K;
+      g.y[0] = g.y[1] = g.y[2] = p.y;
+      g.ys = (size_t)N;
+      g.scale = 1.f;
+      if (vkl::gemm_mfma_supported (g))
+        return vkl::gemm_mfma_launch (g, (hipStream_t)stream);
+    }
   return launch_tb (p, true, (hipStream_t)stream);
 }
 
