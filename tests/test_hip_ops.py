@@ -266,6 +266,28 @@ def test_ffn_upgate_f16_many_rows(dev, rng, M, N, K):
     assert rel_err(f16(out, (M, N)), O.ffn_upgate_f16(x, up, gate)) < F16_REL_TOL
 
 
+@pytest.mark.parametrize("H,S,Lk,hd,maxlen", [(4, 40, 40, 64, 64), (3, 130, 200, 128, 256), (2, 9, 77, 64, 128)])
+def test_attention_products_many_rows(dev, rng, H, S, Lk, hd, maxlen):
+    """Prompt-pass attention: scores = Q K^T over a cache view and P V, batched
+    over heads on the matrix cores (Lk % 8 != 0 takes the scalar kernel for P V)."""
+    q = rng.standard_normal((H, S, hd)).astype(np.float16)
+    kc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    vc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    dq, dk, dv = dev.upload(q), dev.upload(kc), dev.upload(vc)
+    ds = dev.alloc(H * S * Lk * 2)
+    sc = 1.0 / np.sqrt(hd)
+    capi.check(L().vkl_matmul_f16_tb(dq.ptr, dk.ptr, H, S, Lk, hd, S * hd, hd, maxlen * hd, hd, S * Lk, Lk,
+                                     sc, 0.0, 0, None, ds.ptr, None, dev.stream))
+    want_s = O.matmul_f16_tb(q, np.ascontiguousarray(kc[:, :Lk]), scale=sc)
+    assert rel_err(f16(ds, (H, S, Lk)), want_s) < F16_REL_TOL
+    p = rng.uniform(0, 2.0 / Lk, (H, S, Lk)).astype(np.float16)
+    dp, do = dev.upload(p), dev.alloc(H * S * hd * 2)
+    capi.check(L().vkl_matmul_f16_nn(dp.ptr, dv.ptr, H, S, hd, Lk, S * Lk, Lk, maxlen * hd, hd, S * hd, hd,
+                                     1.0, 0.0, 0, do.ptr, dev.stream))
+    want_o = O.matmul_f16_nn(p, np.ascontiguousarray(vc[:, :Lk]))
+    assert rel_err(f16(do, (H, S, hd)), want_o) < F16_REL_TOL
+
+
 def test_matmul_f16_tb_reads_cache_view(dev, rng):
     """scores = Q K^T over the first L rows of a [H, maxlen, hd] cache."""
     H, maxlen, hd, Lk, S = 4, 64, 64, 37, 3

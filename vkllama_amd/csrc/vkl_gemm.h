@@ -16,12 +16,14 @@ struct GemmArgs
   size_t xs;
   int M, N, K;       // K: valid columns of x
   int Kp;            // K rounded up to 32 (rows of the int8 plane)
-  int wtype;         // 8 = planar Q8_0, 1 = fp16
+  int wtype;         // 8 = planar Q8_0, 1 = fp16 [N, K], 2 = fp16 [K, N]
+  int batch;         // independent problems (grid y); 0 means 1
+  size_t xbs, wbs, ybs; // element strides between the problems of a batch
   int nmat;          // 1, or 3 independent matrices/outputs (grid z)
   int upgate;        // 1: w[0] = up, w[1] = gate, y = silu(x gate^T) * (x up^T)
   const uint8_t *wq[3];  // Q8_0: int8 planes [N, Kp]
   const uint16_t *wd[3]; // Q8_0: fp16 scale planes [N, Kp/32]
-  const uint16_t *wh[3]; // fp16: [N, K], row stride ws
+  const uint16_t *wh[3]; // fp16: [N, K] (or [K, N] for wtype 2), row stride ws
   size_t ws;
   uint16_t *y[3]; // [M, N] fp16, row stride ys
   size_t ys;

@@ -1,5 +1,7 @@
 // y[M,N] = x[M,K] W[N,K]^T on the matrix cores (v_mfma_f32_32x32x16_f16),
-// fp16 activations, planar Q8_0 or dense fp16 weights, fp32 accumulation.
+// fp16 activations, planar Q8_0 or dense fp16 weights, fp32 accumulation;
+// also batched fp16 x fp16 products with the second operand stored [N, K]
+// (attention scores) or [K, N] (probabilities times V).
 //
 // Workgroup = 4 waves on a BM x 128 output tile (BM = 128 or 64), k-steps of
 // 32 (one Q8_0 block).  Per step the x tile and the weight tile go through
@@ -7,9 +9,9 @@
 // one block are summed by the MFMA from a zero accumulator and the block
 // scale is applied afterwards in fp32 (acc += partial * d), which is the
 // reference shader's arithmetic: sum over the block, then times d, in fp32.
-// Global loads for step k+1 are issued before
-// the MFMAs of step k and written to the other LDS buffer afterwards, so one
-// barrier per step suffices.  Each wave owns a (BM/2) x 64 sub-tile: TM x 2
+// Global loads run several k-steps ahead in registers and are written to the
+// other LDS buffer after the MFMAs of the current step, so one barrier per
+// step suffices.  Each wave owns a (BM/2) x 64 sub-tile: TM x 2
 // accumulators of 32x32.
 //
 // Tiles are numbered so that workgroups that land on the same XCD (id % 8)
@@ -28,11 +30,25 @@ typedef float float16v __attribute__ ((ext_vector_type (16)));
 constexpr int BN = 128, BK = 32;
 constexpr int LDK = BK + 8; // LDS row stride in halves (80 B: conflict-free b128 reads)
 constexpr int kGemmThreads = 256;
+// k-tiles in flight in registers: more for the small-M configuration, where
+// few workgroups run and each has to hide the memory latency alone
+template <int BM> struct GemmDepth
+{
+  static constexpr int value = BM <= 64 ? 4 : 2;
+};
 
 __device__ __forceinline__ uint4
 ldg16 (const void *p)
 {
   return ldg4 (p);
+}
+
+// v or zero, component by component (a select between two aggregates would
+// take their addresses and push the tile registers out to scratch memory)
+__device__ __forceinline__ uint4
+keep_if (bool c, const uint4 v)
+{
+  return make_uint4 (c ? v.x : 0u, c ? v.y : 0u, c ? v.z : 0u, c ? v.w : 0u);
 }
 
 template <int BM, int WT>
@@ -42,47 +58,74 @@ struct TileLoads
   uint4 a[ACH];
   uint4 b[2];  // fp16: two chunks; Q8_0: b[0] = 16 quants
   uint16_t bd; // Q8_0 block scale
+  uint32_t ok; // validity bits: x chunks from bit 0, weight chunks from bit 8
 };
 
-// weight row (within matrix t) that virtual row v of this workgroup's tile maps to
-__device__ __forceinline__ int
-tile_row (const GemmArgs &a, int n0, int v, int &mat)
+// Per-thread source addresses of the tile loads.  They depend on k only
+// through an added offset, so they are worked out once, before the k loop:
+// in particular the choice among the matrices of a fused launch (a pointer
+// picked from the argument block by a per-lane index) must not sit inside
+// the loop, where the wait for that pointer would also wait for every tile
+// load in flight.
+template <int BM, int WT>
+struct TileAddr
 {
-  if (a.upgate)
-    {
-      mat = v >> 6; // 64 up rows, then the matching 64 gate rows
-      return n0 + (v & 63);
-    }
-  return n0 + v;
+  static constexpr int ACH = BM * 4 / kGemmThreads;
+  const uint16_t *a[ACH]; // x chunk at k = 0, or null beyond M
+  int ak[ACH];            // its column offset within a k-step
+  const uint8_t *bq;      // Q8_0: quants of this thread's row at k = 0
+  const uint16_t *bd;     // Q8_0: its scales
+  const uint16_t *b[2];   // fp16: chunk pointers at k = 0
+  int bk[2];              // fp16 [N, K]: column offset; [K, N]: row offset
+};
+
+__device__ __forceinline__ const void *
+pick3 (const void *p0, const void *p1, const void *p2, int i)
+{
+  return i == 0 ? p0 : (i == 1 ? p1 : p2);
 }
 
 template <int BM, int WT>
 __device__ __forceinline__ void
-issue_tile (const GemmArgs &a, int zmat, int m0, int n0, int k0,
-            TileLoads<BM, WT> &t)
+tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
+                int n0, TileAddr<BM, WT> &ta)
 {
   const int tid = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < TileLoads<BM, WT>::ACH; ++i)
+  for (int i = 0; i < TileAddr<BM, WT>::ACH; ++i)
     {
       const int c = tid + i * kGemmThreads;
-      const int row = c >> 2, seg = c & 3;
-      const int m = m0 + row, k = k0 + seg * 8;
-      t.a[i] = make_uint4 (0, 0, 0, 0);
-      if (m < a.M && k < a.K)
-        t.a[i] = ldg16 (a.x + (size_t)m * a.xs + k);
+      const int m = m0 + (c >> 2);
+      ta.ak[i] = (c & 3) * 8;
+      ta.a[i] = m < a.M ? a.x + xoff + (size_t)m * a.xs + ta.ak[i] : nullptr;
     }
+  ta.bq = nullptr, ta.bd = nullptr;
+  ta.b[0] = ta.b[1] = nullptr;
+  ta.bk[0] = ta.bk[1] = 0;
   if (WT == 8)
     {
       const int v = tid >> 1, seg = tid & 1;
-      int mat = zmat;
-      const int n = tile_row (a, n0, v, mat);
-      t.b[0] = make_uint4 (0, 0, 0, 0);
-      t.bd = 0;
+      const int mat = a.upgate ? (v >> 6) : zmat;
+      const int n = a.upgate ? n0 + (v & 63) : n0 + v;
       if (n < a.N)
         {
-          t.b[0] = ldg16 (a.wq[mat] + (size_t)n * a.Kp + k0 + seg * 16);
-          t.bd = ldg (a.wd[mat] + (size_t)n * (a.Kp >> 5) + (k0 >> 5));
+          ta.bq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat)
+                  + (size_t)n * a.Kp + seg * 16;
+          ta.bd = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat)
+                  + (size_t)n * (a.Kp >> 5);
+        }
+    }
+  else if (WT == 2)
+    {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        {
+          const int c = tid + i * kGemmThreads;
+          const int n = n0 + (c & 15) * 8;
+          ta.bk[i] = c >> 4;
+          if (n < a.N)
+            ta.b[i] = (const uint16_t *)pick3 (a.wh[0], a.wh[1], a.wh[2], zmat)
+                      + woff + (size_t)ta.bk[i] * a.ws + n;
         }
     }
   else
@@ -91,15 +134,58 @@ issue_tile (const GemmArgs &a, int zmat, int m0, int n0, int k0,
       for (int i = 0; i < 2; ++i)
         {
           const int c = tid + i * kGemmThreads;
-          const int v = c >> 2, seg = c & 3;
-          int mat = zmat;
-          const int n = tile_row (a, n0, v, mat);
-          const int k = k0 + seg * 8;
-          t.b[i] = make_uint4 (0, 0, 0, 0);
-          if (n < a.N && k < a.K)
-            t.b[i] = ldg16 (a.wh[mat] + (size_t)n * a.ws + k);
+          const int v = c >> 2;
+          const int mat = a.upgate ? (v >> 6) : zmat;
+          const int n = a.upgate ? n0 + (v & 63) : n0 + v;
+          ta.bk[i] = (c & 3) * 8;
+          if (n < a.N)
+            ta.b[i] = (const uint16_t *)pick3 (a.wh[0], a.wh[1], a.wh[2], mat)
+                      + woff + (size_t)n * a.ws + ta.bk[i];
         }
     }
+}
+
+// Every load is issued unconditionally (from a clamped, always valid address)
+// and masked to zero when the tile is stored: with no branch around a load
+// the compiler can count the loads in flight and wait for exactly the tile it
+// needs instead of for all of them.
+template <int BM, int WT>
+__device__ __forceinline__ void
+issue_tile (const GemmArgs &a, const TileAddr<BM, WT> &ta, int k0,
+            TileLoads<BM, WT> &t)
+{
+  uint32_t ok = 0;
+#pragma unroll
+  for (int i = 0; i < TileLoads<BM, WT>::ACH; ++i)
+    {
+      const bool v = ta.a[i] != nullptr && k0 + ta.ak[i] < a.K;
+      const uint16_t *p = v ? ta.a[i] + k0 : a.x;
+      t.a[i] = ldg16 (p);
+      ok |= (v ? 1u : 0u) << i;
+    }
+  if (WT == 8)
+    {
+      const bool v = ta.bq != nullptr;
+      const uint8_t *pq = v ? ta.bq + k0 : a.wq[0];
+      const uint16_t *pd = v ? ta.bd + (k0 >> 5) : a.wd[0];
+      t.b[0] = ldg16 (pq);
+      t.bd = ldg (pd);
+      ok |= (v ? 1u : 0u) << 8;
+    }
+  else
+    {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        {
+          const bool v = ta.b[i] != nullptr && k0 + ta.bk[i] < a.K;
+          const uint16_t *p
+              = v ? ta.b[i] + (WT == 2 ? (size_t)k0 * a.ws : (size_t)k0)
+                  : a.wh[0];
+          t.b[i] = ldg16 (p);
+          ok |= (v ? 1u : 0u) << (8 + i);
+        }
+    }
+  t.ok = ok;
 }
 
 template <int BM, int WT>
@@ -113,13 +199,15 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
     {
       const int c = tid + i * kGemmThreads;
       const int row = c >> 2, seg = c & 3;
-      *(uint4 *)(As + row * LDK + seg * 8) = t.a[i];
+      *(uint4 *)(As + row * LDK + seg * 8) = keep_if ((t.ok >> i) & 1, t.a[i]);
     }
   if (WT == 8)
     {
       const int v = tid >> 1, seg = tid & 1;
+      const bool okb = (t.ok >> 8) & 1;
       if (seg == 0)
-        Ds[v] = t.bd;
+        Ds[v] = okb ? t.bd : (uint16_t)0;
+      // quants of rows beyond N need no masking: their scale is zero
       const uint32_t w[4] = { t.b[0].x, t.b[0].y, t.b[0].z, t.b[0].w };
       uint32_t o[8];
 #pragma unroll
@@ -134,6 +222,25 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
       dst[0] = make_uint4 (o[0], o[1], o[2], o[3]);
       dst[1] = make_uint4 (o[4], o[5], o[6], o[7]);
     }
+  else if (WT == 2)
+    {
+      // transpose on the way in: LDS holds the tile as [column][k]
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        {
+          const int c = tid + i * kGemmThreads;
+          const int kr = c >> 4, v = (c & 15) * 8;
+          const bool okb = (t.ok >> (8 + i)) & 1;
+          const uint32_t w[4] = { okb ? t.b[i].x : 0u, okb ? t.b[i].y : 0u,
+                                  okb ? t.b[i].z : 0u, okb ? t.b[i].w : 0u };
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              Bs[(v + 2 * j) * LDK + kr] = (uint16_t)(w[j] & 0xffff);
+              Bs[(v + 2 * j + 1) * LDK + kr] = (uint16_t)(w[j] >> 16);
+            }
+        }
+    }
   else
     {
 #pragma unroll
@@ -141,15 +248,77 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
         {
           const int c = tid + i * kGemmThreads;
           const int v = c >> 2, seg = c & 3;
-          *(uint4 *)(Bs + v * LDK + seg * 8) = t.b[i];
+          *(uint4 *)(Bs + v * LDK + seg * 8) = keep_if ((t.ok >> (8 + i)) & 1, t.b[i]);
         }
     }
+}
+
+template <int BM, int WT>
+__device__ __forceinline__ void
+gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
+           const uint16_t *Ac, const uint16_t *Bc, const uint16_t *Dc,
+           uint16_t *An, uint16_t *Bn, uint16_t *Dn, TileLoads<BM, WT> &tn,
+           float16v (&acc)[BM / 64][2], int wm, int vb0, int vb1)
+{
+  constexpr int TM = BM / 64;
+  constexpr int D = GemmDepth<BM>::value;
+  const int lane = threadIdx.x & 63;
+  half8 af[2][TM], bf[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+    {
+      const int kof = ks * 16 + (lane >> 5) * 8;
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+        af[ks][mi] = *(const half8 *)(Ac + (wm * (BM / 2) + mi * 32 + (lane & 31)) * LDK + kof);
+      bf[ks][0] = *(const half8 *)(Bc + (vb0 + (lane & 31)) * LDK + kof);
+      bf[ks][1] = *(const half8 *)(Bc + (vb1 + (lane & 31)) * LDK + kof);
+    }
+  if (WT == 8)
+    {
+      const float sc[2] = { h2f (Dc[vb0 + (lane & 31)]), h2f (Dc[vb1 + (lane & 31)]) };
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+          {
+            float16v part;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              part[r] = 0.f;
+            part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[0][mi], bf[0][ni], part, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[1][mi], bf[1][ni], part, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              acc[mi][ni][r] += part[r] * sc[ni];
+          }
+    }
+  else
+    {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni)
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (
+                af[ks][mi], bf[ks][ni], acc[mi][ni], 0, 0, 0);
+    }
+  store_tile<BM, WT> (tn, An, Bn, Dn);
+  const int knext = min (kt + 1 + D, nk - 1);
+  issue_tile<BM, WT> (a, ta, knext * BK, tn);
+  __syncthreads ();
 }
 
 template <int BM, int WT>
 __global__ __launch_bounds__ (kGemmThreads) void
 gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
 {
+  // element offsets of this problem of the batch (the argument block itself
+  // stays untouched in constant memory: it is indexed by a run-time matrix
+  // number below)
+  const size_t bi = a.batch > 1 ? blockIdx.y : 0;
+  const size_t xoff = bi * a.xbs, woff = bi * a.wbs, yoff = bi * a.ybs;
   constexpr int TM = BM / 64; // 32-row accumulators per wave along M
   __shared__ __align__ (16) uint16_t As[2][BM * LDK];
   __shared__ __align__ (16) uint16_t Bs[2][BN * LDK];
@@ -181,69 +350,57 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
         acc[mi][ni][r] = 0.f;
 
   const int nk = (a.wtype == 8 ? a.Kp : ((a.K + BK - 1) / BK) * BK) / BK;
-  TileLoads<BM, WT> t;
-  issue_tile<BM, WT> (a, zmat, m0, n0, 0, t);
-  store_tile<BM, WT> (t, As[0], Bs[0], Ds[0]);
+  // D tiles are in flight in registers (tile k + 1 .. k + D while tile k is
+  // being multiplied out of LDS): a k-step costs far less time than a trip to
+  // memory, so one tile of look-ahead would leave every step waiting
+  constexpr int D = GemmDepth<BM>::value;
+  TileAddr<BM, WT> ta;
+  tile_addresses<BM, WT> (a, xoff, woff, zmat, m0, n0, ta);
+  TileLoads<BM, WT> t[D];
+  issue_tile<BM, WT> (a, ta, 0, t[0]);
+  store_tile<BM, WT> (t[0], As[0], Bs[0], Ds[0]);
+  issue_tile<BM, WT> (a, ta, min (1, nk - 1) * BK, t[1 % D]);
+  issue_tile<BM, WT> (a, ta, min (2, nk - 1) * BK, t[2 % D]);
+  if (D > 2)
+    {
+      issue_tile<BM, WT> (a, ta, min (3, nk - 1) * BK, t[3]);
+      issue_tile<BM, WT> (a, ta, min (4, nk - 1) * BK, t[0]);
+    }
   __syncthreads ();
 
-  for (int kt = 0; kt < nk; ++kt)
+  // Each step multiplies tile kt out of LDS buffer kt & 1, moves tile kt + 1
+  // (issued D steps earlier) from its registers to the other buffer and
+  // reuses those registers for tile kt + 1 + D.  Stores and loads are
+  // unconditional (past the end they repeat the last tile, which nothing
+  // reads), so the waits in the unrolled body count loads exactly.
+#define VKL_GEMM_STEP(d)                                                      \
+  gemm_step<BM, WT> (a, ta, kt0 + (d), nk, As[(d) & 1], Bs[(d) & 1],        \
+                     Ds[(d) & 1], As[((d) & 1) ^ 1], Bs[((d) & 1) ^ 1],      \
+                     Ds[((d) & 1) ^ 1], t[((d) + 1) % D], acc, wm, vb0, vb1)
+  int kt0 = 0;
+  for (; kt0 + D <= nk; kt0 += D)
     {
-      const int cur = kt & 1;
-      if (kt + 1 < nk)
-        issue_tile<BM, WT> (a, zmat, m0, n0, (kt + 1) * BK, t);
-      const uint16_t *Ac = As[cur], *Bc = Bs[cur];
-      half8 af[2][TM], bf[2][2];
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+      VKL_GEMM_STEP (0);
+      VKL_GEMM_STEP (1);
+      if (D > 2)
         {
-          const int kof = ks * 16 + (lane >> 5) * 8;
-#pragma unroll
-          for (int mi = 0; mi < TM; ++mi)
-            af[ks][mi] = *(const half8 *)(Ac + (wm * (BM / 2) + mi * 32 + (lane & 31)) * LDK + kof);
-          bf[ks][0] = *(const half8 *)(Bc + (vb0 + (lane & 31)) * LDK + kof);
-          bf[ks][1] = *(const half8 *)(Bc + (vb1 + (lane & 31)) * LDK + kof);
+          VKL_GEMM_STEP (2);
+          VKL_GEMM_STEP (3);
         }
-      if (WT == 8)
-        {
-          const float sc[2] = { h2f (Ds[cur][vb0 + (lane & 31)]),
-                                h2f (Ds[cur][vb1 + (lane & 31)]) };
-#pragma unroll
-          for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-              {
-                float16v part;
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                  part[r] = 0.f;
-                part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (
-                    af[0][mi], bf[0][ni], part, 0, 0, 0);
-                part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (
-                    af[1][mi], bf[1][ni], part, 0, 0, 0);
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                  acc[mi][ni][r] += part[r] * sc[ni];
-              }
-        }
-      else
-        {
-#pragma unroll
-          for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-              for (int ni = 0; ni < 2; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (
-                    af[ks][mi], bf[ks][ni], acc[mi][ni], 0, 0, 0);
-        }
-      if (kt + 1 < nk)
-        store_tile<BM, WT> (t, As[cur ^ 1], Bs[cur ^ 1], Ds[cur ^ 1]);
-      __syncthreads ();
     }
+  if (kt0 + 0 < nk)
+    VKL_GEMM_STEP (0);
+  if (kt0 + 1 < nk)
+    VKL_GEMM_STEP (1);
+  if (D > 2 && kt0 + 2 < nk)
+    VKL_GEMM_STEP (2);
+#undef VKL_GEMM_STEP
 
   // epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) +
   // r%4, column l%32 of its 32x32 block
-  uint16_t *y = a.y[a.upgate ? 0 : zmat];
+  uint16_t *y = a.y[a.upgate ? 0 : zmat] + yoff;
+  const uint16_t *res = a.residual ? a.residual + yoff : nullptr;
+  float *y32 = a.y32 ? a.y32 + bi * (size_t)a.M * a.N : nullptr;
 #pragma unroll
   for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
@@ -277,11 +434,11 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
                   v = silu (v);
               }
             uint16_t h = f2h (v);
-            if (a.nmat == 1 && a.residual)
-              h = f2h (h2f (h) + h2f (ldg (a.residual + o)));
+            if (a.nmat == 1 && res)
+              h = f2h (h2f (h) + h2f (ldg (res + o)));
             y[o] = h;
-            if (a.nmat == 1 && a.y32)
-              a.y32[(size_t)m * a.N + n] = h2f (h);
+            if (a.nmat == 1 && y32)
+              y32[(size_t)m * a.N + n] = h2f (h);
           }
       }
 }
@@ -295,7 +452,8 @@ launch_cfg (const GemmArgs &a, hipStream_t s)
   const int tiles = tiles_m * tiles_n;
   const int per_xcd = (tiles + 7) / 8;
   gemm_mfma_kernel<BM, WT>
-      <<<dim3 ((unsigned)(per_xcd * 8), 1, (unsigned)(a.upgate ? 1 : a.nmat)),
+      <<<dim3 ((unsigned)(per_xcd * 8), (unsigned)(a.batch > 1 ? a.batch : 1),
+               (unsigned)(a.upgate ? 1 : a.nmat)),
          dim3 (kGemmThreads), 0, s>>> (a, tiles_m, tiles_n, per_xcd);
   return (int)hipGetLastError ();
 }
@@ -311,9 +469,15 @@ gemm_mfma_supported (const GemmArgs &a)
     return false;
   if (a.wtype == 8)
     return (a.Kp % 32) == 0;
+  if (a.batch > 65535)
+    return false;
+  if (a.wtype == 2) // [K, N] operand: vector loads along N
+    return a.nmat == 1 && !a.upgate && (a.N % 8) == 0 && (a.ws % 8) == 0
+           && ((uintptr_t)a.wh[0] % 16) == 0 && (a.wbs % 8) == 0
+           && (a.xbs % 8) == 0;
   if (a.wtype == 1)
     {
-      if ((a.ws % 8) != 0)
+      if ((a.ws % 8) != 0 || (a.wbs % 8) != 0 || (a.xbs % 8) != 0)
         return false;
       for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
         if (((uintptr_t)a.wh[t] % 16) != 0)
@@ -331,6 +495,8 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
   const bool small = a.M <= 64;
   if (a.wtype == 8)
     return small ? launch_cfg<64, 8> (a, s) : launch_cfg<128, 8> (a, s);
+  if (a.wtype == 2)
+    return small ? launch_cfg<64, 2> (a, s) : launch_cfg<128, 2> (a, s);
   return small ? launch_cfg<64, 1> (a, s) : launch_cfg<128, 1> (a, s);
 }
 } // namespace vkl

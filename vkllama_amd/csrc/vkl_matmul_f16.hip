@@ -179,10 +179,11 @@ vkl_matmul_f16_tb (const void *a, const void *b, int C, int M, int N, int K,
   p.C = C, p.M = M, p.N = N, p.K = K;
   p.acs = acs, p.ahs = ahs, p.bcs = bcs, p.bhs = bhs, p.ycs = ycs, p.yhs = yhs;
   p.scale = scale, p.bias = bias, p.act = act;
-  if (C == 1 && M >= vkl::kGemmMinRows)
+  if (M >= vkl::kGemmMinRows)
     {
-      // a projection over many token rows: matrix cores
+      // many rows (a projection, or the scores of a prompt pass): matrix cores
       vkl::GemmArgs g = {};
+      g.batch = C, g.xbs = acs, g.wbs = bcs, g.ybs = ycs;
       g.x = p.a, g.xs = ahs;
       g.M = M, g.N = N, g.K = K, g.Kp = (K + 31) / 32 * 32;
       g.wtype = 1, g.nmat = 1, g.upgate = 0;
@@ -246,6 +247,21 @@ vkl_matmul_f16_nn (const void *a, const void *b, int C, int M, int N, int K,
   p.C = C, p.M = M, p.N = N, p.K = K;
   p.acs = acs, p.ahs = ahs, p.bcs = bcs, p.bhs = bhs, p.ycs = ycs, p.yhs = yhs;
   p.scale = scale, p.bias = bias, p.act = act;
+  if (M >= vkl::kGemmMinRows)
+    {
+      vkl::GemmArgs g = {};
+      g.batch = C, g.xbs = acs, g.wbs = bcs, g.ybs = ycs;
+      g.x = p.a, g.xs = ahs;
+      g.M = M, g.N = N, g.K = K, g.Kp = (K + 31) / 32 * 32;
+      g.wtype = 2, g.nmat = 1, g.upgate = 0;
+      g.wh[0] = g.wh[1] = g.wh[2] = p.b;
+      g.ws = bhs;
+      g.y[0] = g.y[1] = g.y[2] = p.y;
+      g.ys = yhs;
+      g.scale = scale, g.bias = bias, g.act = act;
+      if (vkl::gemm_mfma_supported (g))
+        return vkl::gemm_mfma_launch (g, (hipStream_t)stream);
+    }
   matmul_nn_kernel<<<dim3 ((unsigned)((N + 63) / 64), (unsigned)M, (unsigned)C),
                      dim3 (256), 0, (hipStream_t)stream>>> (p);
   return vkl_launch_status ();
