@@ -177,3 +177,29 @@ def test_other_decode_modes_match_oracle(cfg, seed, mode):
     want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 32)
     assert list(ids) == list(want)
     m.close()
+
+
+@pytest.mark.parametrize("heads", [4, 2])
+def test_long_context_decode_uses_split_attention(heads):
+    """Past 768 positions the decode step splits each head's context over
+    several workgroups (scores / values / combine launches); logits, greedy ids
+    and the cache rows written on the way must still match the oracle."""
+    cfg = dict(dim=256, n_layers=2, n_heads=heads, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
+    w = M.synth_weights(cfg, seed=21)
+    rng = np.random.default_rng(21)
+    prompt = rng.integers(3, cfg["vocab"], 800).astype(np.uint32)
+    m = M.Llama2(cfg, w)
+    om = O.OracleModel(cfg, w)
+    assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
+    pos = len(prompt)
+    for tok in (7, 300, 12, 5):
+        got, want = m.forward([tok], pos), om.forward([tok], pos)
+        assert logit_err(got, want) < 1e-2, pos
+        assert int(np.argmax(got)) == int(np.argmax(want))
+        pos += 1
+    for layer in range(cfg["n_layers"]):
+        for value in (0, 1):
+            g = m.read_kv_cache(layer, value)[:, 800:pos].astype(np.float32)
+            o = (om.vcache(layer) if value else om.kcache(layer))[:, 800:pos].astype(np.float32)
+            assert np.abs(g - o).max() <= 1e-2 * max(np.abs(o).max(), 1e-3), (layer, value)
+    m.close()

@@ -38,8 +38,16 @@ struct Scratch
   float *amax_val;    // [1024]
   uint32_t *amax_idx; // [1024]
   uint32_t *sync;     // barrier counter + error flag
+  // long-context attention, split over kAttnChunks chunks of the context
+  uint16_t *sc16;     // [heads][maxlen] fp16 scores
+  float *part_max;    // [heads][kAttnChunks]
+  float *part_sum;    // [heads][kAttnChunks]
+  float *part_out;    // [heads][kAttnChunks][head_dim]
   size_t bytes;
 };
+
+constexpr int kAttnChunks = 32;      // upper bound on chunks per head
+constexpr int kAttnSplitMinLen = 768; // shorter contexts use one workgroup per head
 
 __host__ __device__ inline size_t
 align256 (size_t v)
@@ -48,7 +56,7 @@ align256 (size_t v)
 }
 
 __host__ __device__ inline Scratch
-carve (void *base, int dim, int ffn, int vocab)
+carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd)
 {
   Scratch s;
   uint8_t *p = (uint8_t *)base;
@@ -62,6 +70,10 @@ carve (void *base, int dim, int ffn, int vocab)
   s.amax_val = (float *)(p + o), o += 4096;
   s.amax_idx = (uint32_t *)(p + o), o += 4096;
   s.sync = (uint32_t *)(p + o), o += 256;
+  s.sc16 = (uint16_t *)(p + o), o += align256 ((size_t)heads * maxlen * 2);
+  s.part_max = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
+  s.part_sum = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
+  s.part_out = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * hd * 4);
   s.bytes = o;
   return s;
 }
@@ -1113,6 +1125,209 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
   VKL_TR (6);
 }
 
+// ---------------------------------------------------------------------------
+// long contexts: attention split over chunks of the context
+// ---------------------------------------------------------------------------
+// One workgroup per head walks the cache row by row, which at several thousand
+// positions is a long chain of dependent sweeps on 32..40 compute units.  For
+// long contexts the head's rows are split into C chunks, one workgroup each
+// (grid C x heads), in three launches that keep the rounding points of the
+// single-workgroup version (scores and probabilities are fp16 values):
+//   1. attn_scores_kernel: RoPE of q (and of the new k, in the chunk that
+//      holds position pos, which also writes the new K and V rows); fp16
+//      scores of the chunk to scratch; the chunk's maximum m_c and
+//      sum_c = sum exp(s - m_c)
+//   2. attn_values_kernel: M = max m_c, S = sum sum_c exp(m_c - M);
+//      p = fp16(exp(s - M) / S); the chunk's part of sum_l p V[l] in fp32
+//   3. attn_combine_kernel: adds the C parts, rounds to fp16
+constexpr int kAttnThreads = 256;
+
+template <int HD>
+__global__ __launch_bounds__ (kAttnThreads) void
+attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
+{
+  constexpr int LPR = HD / 8;             // lanes per cache row
+  constexpr int RPS = kAttnThreads / LPR; // rows per sweep
+  constexpr int UN = 4;                   // sweeps in flight
+  extern __shared__ __align__ (16) uint8_t lds[];
+  uint16_t *qk = (uint16_t *)lds;         // [2*HD]: rotated q, rotated k
+  float *red = (float *)(lds + 1024);     // [8]
+  float *sc = (float *)(lds + 1024 + 64); // [rows of the chunk]
+  const int head = blockIdx.y, c = blockIdx.x;
+  const int maxlen = p.m.maxlen, dim = p.m.dim;
+  const int pos = (int)p.pos, L = pos + 1;
+  const int R = (L + C - 1) / C;
+  const int l0 = c * R, l1 = min (L, l0 + R);
+  const bool has_new = pos >= l0 && pos < l1;
+  uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
+  uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
+  const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
+
+  if (tid < HD && (tid < HD / 2 || has_new))
+    {
+      const bool is_k = tid >= HD / 2;
+      const int i = is_k ? tid - HD / 2 : tid;
+      const uint16_t *src = p.s.kqv + (is_k ? 0 : dim) + head * HD;
+      const uint32_t v = ldg ((const uint32_t *)src + i);
+      const float cs = ldg (p.m.freqc + (size_t)pos * (HD / 2) + i);
+      const float sn = ldg (p.m.freqs + (size_t)pos * (HD / 2) + i);
+      const float a = h2f ((uint16_t)(v & 0xffff)), b = h2f ((uint16_t)(v >> 16));
+      const uint32_t r = (uint32_t)f2h (a * cs - b * sn)
+                         | ((uint32_t)f2h (a * sn + b * cs) << 16);
+      ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + i] = r;
+      if (is_k)
+        stg ((uint32_t *)(kc + (size_t)pos * HD) + i, r);
+    }
+  else if (has_new && tid >= HD && tid < HD + HD / 2)
+    {
+      const int i = tid - HD;
+      stg ((uint32_t *)(vc + (size_t)pos * HD) + i,
+           ldg ((const uint32_t *)(p.s.kqv + 2 * dim + head * HD) + i));
+    }
+  __syncthreads ();
+
+  const float scale = 1.0f / sqrtf ((float)HD);
+  const uint4 qv = ((const uint4 *)qk)[sub];
+  float mx = -INFINITY;
+  for (int lb = l0; lb < l1; lb += UN * RPS)
+    {
+      uint4 kv[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        {
+          const int l = lb + j * RPS + grp;
+          kv[j] = make_uint4 (0, 0, 0, 0);
+          if (l < l1)
+            kv[j] = l == pos ? ((const uint4 *)(qk + HD))[sub]
+                             : ldg4 (kc + (size_t)l * HD + sub * 8);
+        }
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        {
+          const int l = lb + j * RPS + grp;
+          float sv = dot8_f16 (qv, kv[j], 0.f);
+#pragma unroll
+          for (int o = LPR >> 1; o > 0; o >>= 1)
+            sv += __shfl_xor (sv, o, 64);
+          if (l < l1 && sub == 0)
+            {
+              const uint16_t h = f2h (sv * scale + 0.f);
+              stg (p.s.sc16 + (size_t)head * maxlen + l, h);
+              sc[l - l0] = h2f (h);
+              mx = fmaxf (mx, h2f (h));
+            }
+        }
+    }
+  mx = wave_max (mx);
+  if ((tid & 63) == 0)
+    red[tid >> 6] = mx;
+  __syncthreads ();
+  mx = fmaxf (fmaxf (red[0], red[1]), fmaxf (red[2], red[3]));
+  float sum = 0.f;
+  for (int l = l0 + tid; l < l1; l += kAttnThreads)
+    sum += expf (sc[l - l0] - mx);
+  sum = wave_sum (sum);
+  __syncthreads ();
+  if ((tid & 63) == 0)
+    red[4 + (tid >> 6)] = sum;
+  __syncthreads ();
+  if (tid == 0)
+    {
+      // an empty chunk (l0 >= L) reports -inf / 0 and drops out of the sums
+      stg (p.s.part_max + head * kAttnChunks + c, mx);
+      stg (p.s.part_sum + head * kAttnChunks + c,
+           red[4] + red[5] + red[6] + red[7]);
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__ (kAttnThreads) void
+attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
+{
+  constexpr int LPR = HD / 8;
+  constexpr int RPS = kAttnThreads / LPR;
+  constexpr int UN = 4;
+  __shared__ float part[RPS * HD];
+  const int head = blockIdx.y, c = blockIdx.x;
+  const int maxlen = p.m.maxlen;
+  const int L = (int)p.pos + 1;
+  const int R = (L + C - 1) / C;
+  const int l0 = c * R, l1 = min (L, l0 + R);
+  const uint16_t *vc = (const uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
+  const uint16_t *sc16 = p.s.sc16 + (size_t)head * maxlen;
+  const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
+
+  float M = -INFINITY;
+  for (int i = 0; i < C; ++i)
+    M = fmaxf (M, ldg (p.s.part_max + head * kAttnChunks + i));
+  float S = 0.f;
+  for (int i = 0; i < C; ++i)
+    {
+      const float mi = ldg (p.s.part_max + head * kAttnChunks + i);
+      if (mi > -INFINITY)
+        S += ldg (p.s.part_sum + head * kAttnChunks + i) * expf (mi - M);
+    }
+
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    acc[j] = 0.f;
+  for (int lb = l0; lb < l1; lb += UN * RPS)
+    {
+      uint4 vv[UN];
+      uint16_t sh[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        {
+          const int l = lb + j * RPS + grp;
+          vv[j] = make_uint4 (0, 0, 0, 0);
+          sh[j] = 0;
+          if (l < l1)
+            {
+              vv[j] = ldg4 (vc + (size_t)l * HD + sub * 8);
+              sh[j] = ldg (sc16 + l);
+            }
+        }
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        {
+          const int l = lb + j * RPS + grp;
+          if (l >= l1)
+            continue;
+          const float pl = h2f (f2h (expf (h2f (sh[j]) - M) / S));
+          const uint32_t w[4] = { vv[j].x, vv[j].y, vv[j].z, vv[j].w };
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            {
+              acc[2 * i] += pl * h2f ((uint16_t)(w[i] & 0xffff));
+              acc[2 * i + 1] += pl * h2f ((uint16_t)(w[i] >> 16));
+            }
+        }
+    }
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    part[grp * HD + sub * 8 + j] = acc[j];
+  __syncthreads ();
+  if (tid < HD)
+    {
+      float o = 0.f;
+      for (int g = 0; g < RPS; ++g)
+        o += part[g * HD + tid];
+      stg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid, o);
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__ (HD) void
+attn_combine_kernel (const Params p, int C)
+{
+  const int head = blockIdx.x, tid = threadIdx.x;
+  float o = 0.f;
+  for (int c = 0; c < C; ++c)
+    o += ldg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid);
+  stg (p.s.att + head * HD + tid, f2h (o));
+}
+
 template <int PHASE>
 __global__ __launch_bounds__ (kDecThreads) void
 decode_phase_kernel (const Params p, const vkl_layer_weights lw, int layer,
@@ -1490,6 +1705,39 @@ launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
                                                                  G);
   return timer_mark (PHASE, true, s);
 }
+// attention of one layer: one workgroup per head, or the split form for long
+// contexts
+int
+launch_attention (const Params &p, const vkl_decode_model *m,
+                  const vkl_layer_weights &lw, int layer, int n_cu, size_t lds,
+                  hipStream_t s)
+{
+  const int L = (int)p.pos + 1;
+  if (L < kAttnSplitMinLen)
+    return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
+  int C = (2 * n_cu + m->n_heads - 1) / m->n_heads;
+  C = C < 1 ? 1 : (C > kAttnChunks ? kAttnChunks : C);
+  const int R = (L + C - 1) / C;
+  const size_t lds_a = 1024 + 64 + (size_t)R * 4;
+  VKL_CHECK_ARG (lds_a <= 64 * 1024);
+  if (int e = timer_mark (PH_ATTN, false, s))
+    return e;
+  const dim3 grid ((unsigned)C, (unsigned)m->n_heads);
+  if (m->head_dim == 128)
+    {
+      attn_scores_kernel<128><<<grid, dim3 (kAttnThreads), lds_a, s>>> (p, lw, C);
+      attn_values_kernel<128><<<grid, dim3 (kAttnThreads), 0, s>>> (p, lw, C);
+      attn_combine_kernel<128><<<dim3 ((unsigned)m->n_heads), dim3 (128), 0, s>>> (p, C);
+    }
+  else
+    {
+      attn_scores_kernel<64><<<grid, dim3 (kAttnThreads), lds_a, s>>> (p, lw, C);
+      attn_values_kernel<64><<<grid, dim3 (kAttnThreads), 0, s>>> (p, lw, C);
+      attn_combine_kernel<64><<<dim3 ((unsigned)m->n_heads), dim3 (64), 0, s>>> (p, C);
+    }
+  return timer_mark (PH_ATTN, true, s);
+}
+
 // The arrival counter of a scratch buffer restarts from zero with every token:
 // a one-thread kernel in front of the step clears it (a fill kernel rather
 // than a memset node, so that a caller may capture the step in a graph).
@@ -1621,7 +1869,7 @@ vkl_decode_scratch_bytes (const vkl_decode_model *m)
 {
   if (!m)
     return 0;
-  return carve (nullptr, m->dim, m->ffn, m->vocab).bytes;
+  return carve (nullptr, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim).bytes;
 }
 
 extern "C" const void *
@@ -1629,7 +1877,7 @@ vkl_decode_logits_f16 (const vkl_decode_model *m)
 {
   if (!m || !m->scratch)
     return nullptr;
-  return carve (m->scratch, m->dim, m->ffn, m->vocab).logits16;
+  return carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim).logits16;
 }
 
 #ifdef VKL_TRACE
@@ -1661,7 +1909,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
       = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
   Params p;
   p.m = *m;
-  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab);
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
   p.tok = tok;
   p.pos = pos;
   p.logits32 = logits32 ? logits32 : p.s.logits32;
@@ -1684,8 +1932,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
       const vkl_layer_weights &lw = m->layers_h[l];
       if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
         return e;
-      if (int e
-          = launch_phase<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads, lds, s))
+      if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
         return e;
       if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
         return e;
@@ -1742,7 +1989,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
   Params p;
   p.m = *m;
-  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab);
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
   p.tok = (const uint32_t *)p.s.amax_idx; // any device word: ids >= vocab read row 0
   p.pos = pos;
   p.logits32 = p.s.logits32;
@@ -1778,8 +2025,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
               err = launch_phase<PH_KQV> (p, lw, li, G, G, lds, s);
               break;
             case PH_ATTN:
-              err = launch_phase<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads,
-                                           lds, s);
+              err = launch_attention (p, m, lw, l, n_cu, lds, s);
               break;
             case PH_WO:
               err = launch_phase<PH_WO> (p, lw, l, G, G, lds, s);
