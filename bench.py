@@ -36,6 +36,9 @@ WORKLOADS = {
                              prompt=16, prefill_kv=0),
     "llama2-7b-q8_0": dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5,
                            wtype=8, prompt=32, prefill_kv=0),
+    # BASELINE config 4: FP16 weights, 2048-token prompt
+    "llama2-7b-f16": dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5,
+                          wtype=1, prompt=2048, prefill_kv=0),
     "llama2-13b-q8_0-ctx3968": dict(dim=5120, n_layers=40, n_heads=40, ffn=13824, vocab=32000, maxlen=4096,
                                     eps=1e-5, wtype=8, prompt=3968, prefill_kv=1),
 }
@@ -172,8 +175,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "q8_0 weights x f16 activations, f32 accumulate",
-        "data": "synthetic: random-init N(0,0.02) weights quantised to Q8_0, random prompt ids",
+        "dtype": ("q8_0" if cfg["wtype"] == 8 else "f16") + " weights x f16 activations, f32 accumulate",
+        "data": "synthetic: random-init N(0,0.02) weights" + (" quantised to Q8_0" if cfg["wtype"] == 8 else " in FP16")
+                + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
                    "decode_mode": ("launch-per-phase", "persistent", "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},

@@ -124,16 +124,20 @@ def test_lastblock_rope_quirk_switch(small):
         m.close()
 
 
-def test_fp16_weights_model_runs_on_operator_chain():
+@pytest.mark.parametrize("fused", [0, 1])
+def test_fp16_weights_model(fused):
+    """FP16 matrices: operator chain, and the fused decode step on its fp16
+    weight path."""
     cfg = dict(SMALL, wtype=1, n_layers=2)
     w = M.synth_weights(cfg, seed=3)
     prompt = np.array([5, 17, 99], np.uint32)
     m = M.Llama2(cfg, w)
+    m.set_option("fused_decode", fused)
     om = O.OracleModel(cfg, w)
     assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
     assert logit_err(m.forward([4], 3), om.forward([4], 3)) < 1e-2
-    ids, _, _ = m.generate_greedy(prompt, 8)
-    want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 8)
+    ids, _, _ = m.generate_greedy(prompt, 24)
+    want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 24)
     assert list(ids) == list(want)
     m.close()
 

@@ -383,6 +383,16 @@ better (float v, uint32_t i, float bv, uint32_t bi)
 // state of the phase in progress.  Keeping ONE pair of buffers for all phases
 // matters in the persistent kernel, where a phase's first items are issued
 // while the previous phase is still being finished.
+// weight matrix view: planar Q8_0 (quants + scales) or dense fp16 (bytes)
+template <int WT>
+__device__ __forceinline__ QMat
+wmat (const void *w, int N, int K)
+{
+  if (WT == 8)
+    return qmat (w, N, K);
+  return QMat{ (const uint8_t *)w, (const uint16_t *)w };
+}
+
 struct PipeBuf
 {
   uint4 w[8];
@@ -412,7 +422,10 @@ struct PipeState
 // One copy of the code serves all three (the mode only steers the cheap row
 // addressing and the lane-0 epilogue), which keeps the persistent kernel
 // inside the instruction cache.
-template <bool COH> struct Gemv
+// WT: 8 = planar Q8_0 weights, 1 = dense fp16 weights.  For fp16 a row is
+// addressed as 2*K bytes, so the 16-byte loads of an item are laid out exactly
+// as for the int8 plane; only the scale load and the dot product differ.
+template <bool COH, int WT = 8> struct Gemv
 {
   static constexpr int R = 2; // rows per unit
   static constexpr int S = 4; // k-steps of 1024 per item
@@ -460,7 +473,10 @@ template <bool COH> struct Gemv
     ps.dd1 = (const uint8_t *)b.d - (const uint8_t *)a.d;
     ps.dd2 = (const uint8_t *)c.d - (const uint8_t *)a.d;
     ps.N = N;
-    ps.Kp = ((K + 31) >> 5) << 5, ps.nb = ps.Kp >> 5;
+    if (WT == 8)
+      ps.Kp = ((K + 31) >> 5) << 5, ps.nb = ps.Kp >> 5;
+    else
+      ps.Kp = K * 2, ps.nb = 0; // row bytes
     ps.nch = (ps.Kp + CHUNK - 1) / CHUNK;
     ps.lane = threadIdx.x & 63, ps.wave = threadIdx.x >> 6, ps.wg = wg;
     const int U = mode == 0 ? (N + 1) >> 1 : (mode == 1 ? 3 * (N >> 1) : N);
@@ -508,7 +524,8 @@ template <bool COH> struct Gemv
         for (int r = 0; r < R; ++r)
           {
             b.w[r * S + s] = ok ? ldg4 (q[r] + kk) : make_uint4 (0, 0, 0, 0);
-            b.d[r * S + s] = ok ? ldg (d[r] + (kk >> 5)) : (uint16_t)0;
+            if (WT == 8)
+              b.d[r * S + s] = ok ? ldg (d[r] + (kk >> 5)) : (uint16_t)0;
           }
       }
   }
@@ -528,7 +545,17 @@ template <bool COH> struct Gemv
     for (int s = 0; s < S; ++s)
       {
         const int kk = c * CHUNK + s * (VKL_WAVE * 16) + ps.lane * 16;
-        if (kk < ps.Kp)
+        if (WT != 8)
+          {
+            if (kk < ps.Kp) // kk counts bytes of the fp16 row
+              {
+                const uint4 xv = *(const uint4 *)(xl + (kk >> 1));
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                  acc[r] = dot8_f16 (b.w[r * S + s], xv, acc[r]);
+              }
+          }
+        else if (kk < ps.Kp)
           {
             const uint4 *xp = (const uint4 *)(xl + kk);
             const uint4 x0 = xp[0], x1 = xp[1];
@@ -928,7 +955,7 @@ phase_signal (const Params &p)
 // Every projection phase runs in this order: activation loads, norm-weight
 // loads, first weight item (all issued back to back), then the activation is
 // normalised / written to LDS, then the weight pipeline runs.
-template <bool COH>
+template <bool COH, int WT = 8>
 __device__ __forceinline__ void
 run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
            int wg, int G, uint8_t *lds)
@@ -951,12 +978,12 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
     {
     case PH_KQV:
       {
-        const QMat wk = qmat (lw.wk, dim, dim), wq = qmat (lw.wq, dim, dim),
-                   wv = qmat (lw.wv, dim, dim);
+        const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
+                   wv = wmat<WT> (lw.wv, dim, dim);
         if (COH)
           {
             issue_norm (lw.attn_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
             VKL_TR (5);
@@ -966,22 +993,26 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
             uint32_t tok = COH ? ld_coherent_u32 (p.tok) : ldg (p.tok);
             if (tok >= (uint32_t)m.vocab)
               tok = 0;
-            issue_embed_q8 (qmat (m.tok_embd, m.vocab, dim), tok, dim, x);
+            if (WT == 8)
+              issue_embed_q8 (wmat<WT> (m.tok_embd, m.vocab, dim), tok, dim, x);
+            else
+              issue_x<false> ((const uint16_t *)m.tok_embd + (size_t)tok * dim, dim, x);
           }
         else
           issue_x<COH> (p.s.x, dim, x);
         if (COH)
           {
-            Gemv<COH>::prime (ps, A, B, 2);
+            Gemv<COH, WT>::prime (ps, A, B, 2);
           }
         else
           {
             issue_norm (lw.attn_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1);
+            Gemv<COH, WT>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1);
           }
         if (layer == 0)
           {
-            dequant_embed (x);
+            if (WT == 8)
+              dequant_embed (x);
             if (wg == 0) // the residual stream starts as the embedding row
               {
 #pragma unroll
@@ -1002,7 +1033,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
-        Gemv<COH>::run (ps, A, B, xl, e, red);
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ATTN:
@@ -1020,31 +1051,31 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
       }
     case PH_WO:
       {
-        const QMat w = qmat (lw.wo, dim, dim);
+        const QMat w = wmat<WT> (lw.wo, dim, dim);
         if (COH)
           {
-            Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre);
             phase_wait<COH> (p);
             VKL_TR (5);
           }
         issue_x<COH> (p.s.att, dim, x);
         if (COH)
-          Gemv<COH>::prime (ps, A, B, 2);
+          Gemv<COH, WT>::prime (ps, A, B, 2);
         else
-          Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1);
+          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1);
         finish_x<false> (x, dim, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        Gemv<COH>::run (ps, A, B, xl, e, red);
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_UPGATE:
       {
-        const QMat up = qmat (lw.w_up, ffn, dim), gate = qmat (lw.w_gate, ffn, dim);
+        const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
         if (COH)
           {
             issue_norm (lw.ffn_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
             VKL_TR (5);
@@ -1052,46 +1083,46 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         issue_x<COH> (p.s.x, dim, x);
         if (COH)
           {
-            Gemv<COH>::prime (ps, A, B, 2);
+            Gemv<COH, WT>::prime (ps, A, B, 2);
           }
         else
           {
             issue_norm (lw.ffn_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
+            Gemv<COH, WT>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
           }
         finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.t;
-        Gemv<COH>::run (ps, A, B, xl, e, red);
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_DOWN:
       {
-        const QMat w = qmat (lw.w_down, dim, ffn);
+        const QMat w = wmat<WT> (lw.w_down, dim, ffn);
         if (COH)
           {
-            Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre);
             phase_wait<COH> (p);
             VKL_TR (5);
           }
         issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
         if (COH)
-          Gemv<COH>::prime (ps, A, B, 2);
+          Gemv<COH, WT>::prime (ps, A, B, 2);
         else
-          Gemv<COH>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1);
+          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1);
         finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        Gemv<COH>::run (ps, A, B, xl, e, red);
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_HEAD:
       {
-        const QMat w = qmat (m.output, m.vocab, dim);
+        const QMat w = wmat<WT> (m.output, m.vocab, dim);
         if (COH)
           {
             issue_norm (m.output_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, pre);
             stash_norm (nw, dim, nl);
             phase_wait<COH> (p);
             VKL_TR (5);
@@ -1099,18 +1130,18 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         issue_x<COH> (p.s.x, dim, x);
         if (COH)
           {
-            Gemv<COH>::prime (ps, A, B, 2);
+            Gemv<COH, WT>::prime (ps, A, B, 2);
           }
         else
           {
             issue_norm (m.output_norm, dim, nw);
-            Gemv<COH>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
           }
         finish_x<true, COH> (x, dim, xl, nw, m.final_eps, red, nl, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.logits16, e.y32 = p.logits32;
         e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
-        Gemv<COH>::run (ps, A, B, xl, e, red);
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ARGMAX:
@@ -1328,13 +1359,13 @@ attn_combine_kernel (const Params p, int C)
   stg (p.s.att + head * HD + tid, f2h (o));
 }
 
-template <int PHASE>
+template <int PHASE, int WT>
 __global__ __launch_bounds__ (kDecThreads) void
 decode_phase_kernel (const Params p, const vkl_layer_weights lw, int layer,
                      int G)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
-  run_phase<false> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
+  run_phase<false, WT> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
 }
 
 // overlapped launches: two of these are resident per compute unit
@@ -1619,7 +1650,7 @@ int
 check_model (const vkl_decode_model *m)
 {
   VKL_CHECK_ARG (m != nullptr);
-  VKL_CHECK_ARG (m->wtype == 8);
+  VKL_CHECK_ARG (m->wtype == 8 || m->wtype == 1);
   VKL_CHECK_ARG (m->dim > 0 && m->n_layers > 0 && m->n_heads > 0);
   VKL_CHECK_ARG (m->head_dim == 64 || m->head_dim == 128);
   VKL_CHECK_ARG (m->n_heads * m->head_dim == m->dim);
@@ -1685,6 +1716,25 @@ timer_collect (hipStream_t s)
   return 0;
 }
 
+template <int PHASE, int WT>
+int
+launch_phase_wt (const Params &p, const vkl_layer_weights &lw, int layer,
+                 int grid, int G, size_t lds, hipStream_t s)
+{
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_phase_kernel<PHASE, WT>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  decode_phase_kernel<PHASE, WT>
+      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
+                                                                 G);
+  return 0;
+}
+
 template <int PHASE>
 int
 launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
@@ -1692,19 +1742,13 @@ launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
 {
   if (int e = timer_mark (PHASE, false, s))
     return e;
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_kernel<PHASE>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
-  decode_phase_kernel<PHASE>
-      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
-                                                                 G);
+  if (int e = p.m.wtype == 8
+                  ? launch_phase_wt<PHASE, 8> (p, lw, layer, grid, G, lds, s)
+                  : launch_phase_wt<PHASE, 1> (p, lw, layer, grid, G, lds, s))
+    return e;
   return timer_mark (PHASE, true, s);
 }
+
 // attention of one layer: one workgroup per head, or the split form for long
 // contexts
 int
@@ -1897,6 +1941,8 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
     return e;
   VKL_CHECK_ARG (tok != nullptr && pos < (uint32_t)m->maxlen);
   VKL_CHECK_ARG (mode >= 0 && mode <= 2);
+  // the persistent and overlapped modes exist for Q8_0 weights only
+  VKL_CHECK_ARG (mode == 0 || m->wtype == 8);
   static int n_cu = 0;
   if (n_cu == 0)
     {
@@ -2064,7 +2110,10 @@ vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L)
     return 0;
   const size_t dim = (size_t)m->dim, ffn = (size_t)m->ffn, V = (size_t)m->vocab;
   // a Q8_0 matrix [N, K]: N*K quants + N*K/32 fp16 scales
-  auto mat = [] (size_t N, size_t K) { return N * K + N * (K / 32) * 2; };
+  const bool q8 = m->wtype == 8;
+  auto mat = [q8] (size_t N, size_t K) {
+    return q8 ? N * K + N * (K / 32) * 2 : N * K * 2;
+  };
   switch (kind)
     {
     case PH_KQV: // x + norm weights in, three projections out

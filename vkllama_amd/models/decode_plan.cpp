@@ -44,11 +44,19 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
   const size_t hd = attn0->kcache ().width ();
   const size_t heads = attn0->kcache ().channels ();
   const size_t ffn = blocks[0]->feed_forward ()->w1 ().height ();
-  const bool q8 = emb.dtype () == Q8_0 && out->weight ().dtype () == Q8_0
-                  && attn0->wk ().dtype () == Q8_0
-                  && attn0->wo ().dtype () == Q8_0
-                  && blocks[0]->feed_forward ()->w1 ().dtype () == Q8_0;
-  if (!q8 || (hd != 64 && hd != 128) || heads * hd != dim || dim % 32
+  // the fused step takes models whose matrices are all Q8_0 or all FP16
+  const DType wt = emb.dtype ();
+  const bool uniform = (wt == Q8_0 || wt == FP16)
+                       && out->weight ().dtype () == wt
+                       && attn0->wk ().dtype () == wt
+                       && attn0->wo ().dtype () == wt
+                       && blocks[0]->feed_forward ()->w1 ().dtype () == wt;
+  // norm weights are read as fp32 by the fused kernels
+  bool norms32 = out->norm ()->weight ().dtype () == FP32;
+  for (auto *b : blocks)
+    norms32 = norms32 && b->attn_norm ()->weight ().dtype () == FP32
+              && b->ffn_norm ()->weight ().dtype () == FP32;
+  if (!uniform || !norms32 || (hd != 64 && hd != 128) || heads * hd != dim || dim % 32
       || ffn % 32 || vocab_ % 2)
     {
       usable_ = false; // the operator chain serves these models
@@ -89,7 +97,7 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
   desc_.ffn = (int)ffn;
   desc_.vocab = (int)vocab_;
   desc_.maxlen = (int)attn0->kcache ().height ();
-  desc_.wtype = 8;
+  desc_.wtype = wt == Q8_0 ? 8 : 1; // GGML type numbers
   desc_.eps = eps;
   desc_.final_eps = out->norm ()->eps ();
   desc_.layers = (const vkl_layer_weights *)layers_.data ();
