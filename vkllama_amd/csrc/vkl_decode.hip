@@ -397,6 +397,7 @@ struct PipeBuf
 {
   uint4 w[8];
   uint16_t d[8];
+  uint32_t res; // mode 0: the two residual values of the item's unit
 };
 
 struct PipeState
@@ -411,6 +412,7 @@ struct PipeState
   int u_lo, nit, primed;
   float best_v;
   uint32_t best_i;
+  const uint16_t *residual; // mode 0: fetched with each item, see issue ()
 };
 
 // mode 0: y = x W^T (+ residual); a unit is 2 consecutive rows of m0
@@ -465,9 +467,11 @@ template <bool COH, int WT = 8> struct Gemv
   // (0..2) items
   static __device__ __forceinline__ void
   begin (PipeState &ps, PipeBuf &A, PipeBuf &B, int mode, const QMat a,
-         const QMat b, const QMat c, int N, int K, int wg, int G, int depth)
+         const QMat b, const QMat c, int N, int K, int wg, int G, int depth,
+         const uint16_t *residual = nullptr)
   {
     ps.mode = mode;
+    ps.residual = residual;
     ps.m0 = a;
     ps.dq1 = b.q - a.q, ps.dq2 = c.q - a.q;
     ps.dd1 = (const uint8_t *)b.d - (const uint8_t *)a.d;
@@ -515,6 +519,11 @@ template <bool COH, int WT = 8> struct Gemv
     const uint8_t *q[R];
     const uint16_t *d[R];
     rows_of (ps, u, q, d);
+    // the residual pair of the unit travels with the item, so the epilogue
+    // does not start a dependent trip to memory at the end of the row
+    b.res = 0;
+    if (ps.residual && 2 * u + 1 < ps.N)
+      b.res = ld_u32<COH> ((const uint32_t *)(ps.residual + 2 * u));
 #pragma unroll
     for (int s = 0; s < S; ++s)
       {
@@ -570,11 +579,12 @@ template <bool COH, int WT = 8> struct Gemv
           }
       }
     if (c == ps.nch - 1)
-      finish (ps, acc, ps.u_lo + ui * kDecWaves, e);
+      finish (ps, acc, ps.u_lo + ui * kDecWaves, e, b.res);
   }
 
   static __device__ __forceinline__ void
-  finish (PipeState &ps, const float (&acc)[R], int u, const Epilogue &e)
+  finish (PipeState &ps, const float (&acc)[R], int u, const Epilogue &e,
+          uint32_t res)
   {
     float v[R];
 #pragma unroll
@@ -595,7 +605,12 @@ template <bool COH, int WT = 8> struct Gemv
       }
     if (ps.mode == 2)
       {
-        st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[1]) * v[0]));
+        // fp16 when kernel boundaries order the phases; one 32-bit word per
+        // element where it has to be a write-through atomic
+        if (COH)
+          st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[1]) * v[0]));
+        else
+          stg (e.y[0] + u, f2h (silu (v[1]) * v[0]));
         return;
       }
     const int r0 = 2 * u;
@@ -603,9 +618,11 @@ template <bool COH, int WT = 8> struct Gemv
     uint16_t h0 = f2h (v[0]), h1 = f2h (v[1]);
     if (e.residual)
       {
+        // prefetched with the item unless the phase was begun without it
         const uint32_t rr
-            = two ? ld_u32<COH> ((const uint32_t *)(e.residual + r0))
-                  : (uint32_t)ldg (e.residual + r0);
+            = !two ? (uint32_t)ldg (e.residual + r0)
+                   : (ps.residual ? res
+                                  : ld_u32<COH> ((const uint32_t *)(e.residual + r0)));
         h0 = f2h (h2f (h0) + h2f ((uint16_t)(rr & 0xffff)));
         h1 = f2h (h2f (h1) + h2f ((uint16_t)(rr >> 16)));
       }
@@ -1054,7 +1071,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         const QMat w = wmat<WT> (lw.wo, dim, dim);
         if (COH)
           {
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre, p.s.x);
             phase_wait<COH> (p);
             VKL_TR (5);
           }
@@ -1062,7 +1079,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         if (COH)
           Gemv<COH, WT>::prime (ps, A, B, 2);
         else
-          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1);
+          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x);
         finish_x<false> (x, dim, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
@@ -1101,15 +1118,18 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         const QMat w = wmat<WT> (lw.w_down, dim, ffn);
         if (COH)
           {
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre);
+            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre, p.s.x);
             phase_wait<COH> (p);
             VKL_TR (5);
           }
-        issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
+        if (COH)
+          issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
+        else
+          issue_x<COH> (p.s.t, ffn, x);
         if (COH)
           Gemv<COH, WT>::prime (ps, A, B, 2);
         else
-          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1);
+          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.s.x);
         finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
@@ -2123,9 +2143,9 @@ vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L)
     case PH_WO:
       return mat (dim, dim) + dim * 2 + 2 * dim * 2;
     case PH_UPGATE:
-      return 2 * mat (ffn, dim) + dim * 2 + dim * 4 + ffn * 4;
+      return 2 * mat (ffn, dim) + dim * 2 + dim * 4 + ffn * 2;
     case PH_DOWN:
-      return mat (dim, ffn) + ffn * 4 + 2 * dim * 2;
+      return mat (dim, ffn) + ffn * 2 + 2 * dim * 2;
     case PH_HEAD:
       return mat (V, dim) + dim * 2 + dim * 4 + V * 2 + V * 4;
     default:
