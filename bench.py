@@ -125,10 +125,12 @@ def main():
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # second pass over the same steps with an event pair around every phase launch
+    m.set_option("decode_graph", 0)      # event pairs need the step-by-step launches
     m.set_option("phase_timing", 1)
     m.phase_times()
     m.generate_greedy(prompt, steps + 1)
     m.set_option("phase_timing", 0)
+    m.set_option("decode_graph", 1)
     phases = m.phase_times()
     L_mid = int(ctx[len(ctx) // 2])
     per_phase = {}
@@ -179,7 +181,8 @@ def main():
         "data": "synthetic: random-init N(0,0.02) weights" + (" quantised to Q8_0" if cfg["wtype"] == 8 else " in FP16")
                 + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
-                   "decode_mode": ("launch-per-phase", "persistent", "overlapped-launches")[args.decode_mode],
+                   "decode_mode": ("launch-per-phase, replayed from a HIP graph", "persistent",
+                                   "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "decode_tokens_per_second_host_interface": round(host_tok_s, 1),
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),

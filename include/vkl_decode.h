@@ -62,6 +62,16 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
                      uint32_t pos, int mode, float *logits32,
                      uint32_t *next_tok, void *stream);
 
+/* n_steps greedy tokens without a host round trip per token: step i reads
+ * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
+ * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the
+ * device.  The launches of one step are captured once in a HIP graph (per
+ * model / buffers / attention form) and replayed; results are identical to
+ * n_steps calls of vkl_decode_step in mode 0.  logits32 (optional) receives
+ * the logits of the last step.  The stream must not be capturing. */
+int vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
+                     int n_steps, float *logits32, void *stream);
+
 /* Phase timing (mode 0 only; a measuring aid without counterpart in the
  * reference, whose GPUDevice timestamps play this role in
  * src/core/gpu_device.cpp).  While enabled, vkl_decode_step brackets every

@@ -207,3 +207,25 @@ def test_long_context_decode_uses_split_attention(heads):
             o = (om.vcache(layer) if value else om.kcache(layer))[:, 800:pos].astype(np.float32)
             assert np.abs(g - o).max() <= 1e-2 * max(np.abs(o).max(), 1e-3), (layer, value)
     m.close()
+
+
+@pytest.mark.parametrize("n_prompt,n_gen", [(4, 40), (760, 24)])
+def test_graph_replayed_loop_equals_stepwise_and_oracle(n_prompt, n_gen):
+    """generate_greedy replays one captured step per token (token index and
+    position advance in device memory); the ids must equal those of the
+    step-by-step launches and the oracle's, also across the switch of the
+    attention phase to its split form at 768 positions, and on a second use
+    of the cached graphs."""
+    cfg = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
+    w = M.synth_weights(cfg, seed=33)
+    rng = np.random.default_rng(33)
+    prompt = rng.integers(3, cfg["vocab"], n_prompt).astype(np.uint32)
+    want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, n_gen)
+    m = M.Llama2(cfg, w)
+    for graph in (1, 0, 1):
+        m.set_option("decode_graph", graph)
+        ids, _, _ = m.generate_greedy(prompt, n_gen)
+        assert list(ids) == list(want), graph
+        # eager work between replays: a plain forward pass
+        m.forward(prompt[:3], 0)
+    m.close()

@@ -21,6 +21,7 @@
 // activations (a few KiB) come from L2.
 #include "../../include/vkl_decode.h"
 #include "vkl_decode_dev.h"
+#include <algorithm>
 #include <vector>
 
 namespace vkl
@@ -87,6 +88,10 @@ struct Params
   float *logits32;    // destination of the widened logits
   uint32_t *next_tok; // may be null
   uint32_t wait_target; // overlapped launches: arrivals to wait for
+  // replayed loop (vkl_decode_loop): token index and position live in device
+  // memory so that every step is the same sequence of launches
+  const uint32_t *loop; // {index into ids, position}, or null
+  uint32_t *ids;        // loop: input token ids[index], result to ids[index + 1]
 #ifdef VKL_TRACE
   unsigned long long *trace; // [phase slot][wg][8] wall-clock stamps
 #endif
@@ -103,6 +108,20 @@ struct Params
 #define VKL_TR(slot)
 #define VKL_TRP nullptr
 #endif
+
+// position and token of the step: kernel arguments, or the device-resident
+// loop state when the step is replayed from a graph
+__device__ __forceinline__ uint32_t
+step_pos (const Params &p)
+{
+  return p.loop ? ldg (p.loop + 1) : p.pos;
+}
+
+__device__ __forceinline__ const uint32_t *
+step_tok (const Params &p)
+{
+  return p.loop ? p.ids + ldg (p.loop) : p.tok;
+}
 
 // ---------------------------------------------------------------------------
 // activation staging
@@ -708,7 +727,7 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   constexpr int RPB = kDecThreads / LPR; // cache rows per sweep
   constexpr int PRE = 4;                 // sweeps prefetched up front
   const int dim = p.m.dim, maxlen = p.m.maxlen;
-  const uint32_t pos = p.pos;
+  const uint32_t pos = step_pos (p);
   const int L = (int)pos + 1;
   uint16_t *qk = (uint16_t *)lds;    // [3*HD]
   float *sc = (float *)(lds + 1024); // [maxlen]
@@ -915,7 +934,17 @@ final_argmax (const Params &p, int G, uint8_t *lds)
       for (int w = 1; w < kDecWaves; ++w)
         if (better (bv[w], bi[w], v, idx))
           v = bv[w], idx = bi[w];
-      stg (p.next_tok, idx == 0xffffffffu ? 0u : idx);
+      const uint32_t id = idx == 0xffffffffu ? 0u : idx;
+      if (p.loop)
+        {
+          // hand the token to the next replay of the step
+          const uint32_t i = ldg (p.loop), ps = ldg (p.loop + 1);
+          stg (p.ids + i + 1, id);
+          stg ((uint32_t *)p.loop, i + 1);
+          stg ((uint32_t *)p.loop + 1, ps + 1);
+        }
+      else
+        stg (p.next_tok, id);
     }
 }
 
@@ -1007,7 +1036,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
           }
         if (layer == 0)
           {
-            uint32_t tok = COH ? ld_coherent_u32 (p.tok) : ldg (p.tok);
+            uint32_t tok = COH ? ld_coherent_u32 (p.tok) : ldg (step_tok (p));
             if (tok >= (uint32_t)m.vocab)
               tok = 0;
             if (WT == 8)
@@ -1167,7 +1196,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
     case PH_ARGMAX:
       phase_wait<COH> (p);
             VKL_TR (5);
-      if (wg == 0 && p.next_tok)
+      if (wg == 0 && (p.next_tok || p.loop))
         final_argmax<COH> (p, G, lds);
       break;
     }
@@ -1206,7 +1235,7 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
   float *sc = (float *)(lds + 1024 + 64); // [rows of the chunk]
   const int head = blockIdx.y, c = blockIdx.x;
   const int maxlen = p.m.maxlen, dim = p.m.dim;
-  const int pos = (int)p.pos, L = pos + 1;
+  const int pos = (int)step_pos (p), L = pos + 1;
   const int R = (L + C - 1) / C;
   const int l0 = c * R, l1 = min (L, l0 + R);
   const bool has_new = pos >= l0 && pos < l1;
@@ -1301,7 +1330,7 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
   __shared__ float part[RPS * HD];
   const int head = blockIdx.y, c = blockIdx.x;
   const int maxlen = p.m.maxlen;
-  const int L = (int)p.pos + 1;
+  const int L = (int)step_pos (p) + 1;
   const int R = (L + C - 1) / C;
   const int l0 = c * R, l1 = min (L, l0 + R);
   const uint16_t *vc = (const uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
@@ -1776,6 +1805,8 @@ launch_attention (const Params &p, const vkl_decode_model *m,
                   const vkl_layer_weights &lw, int layer, int n_cu, size_t lds,
                   hipStream_t s)
 {
+  // p.pos is the position of a single step, or the last position of the
+  // steps a replayed loop will cover in this form (the LDS need grows with it)
   const int L = (int)p.pos + 1;
   if (L < kAttnSplitMinLen)
     return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
@@ -1953,6 +1984,38 @@ vkl_debug_set_trace (void *buf)
 }
 #endif
 
+namespace
+{
+// the launches of one token, one per phase
+int
+launch_step (const Params &p, const vkl_decode_model *m, int n_cu, int G,
+             size_t lds, hipStream_t s)
+{
+  for (int l = 0; l < m->n_layers; ++l)
+    {
+      const vkl_layer_weights &lw = m->layers_h[l];
+      if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
+        return e;
+      if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s))
+        return e;
+      if (int e = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s))
+        return e;
+    }
+  const vkl_layer_weights none = {};
+  if (int e = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s))
+    return e;
+  if (p.next_tok || p.loop)
+    if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
+      return e;
+  return 0;
+}
+
+}
+
 extern "C" int
 vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
                  int mode, float *logits32, uint32_t *next_tok, void *stream)
@@ -1980,6 +2043,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.pos = pos;
   p.logits32 = logits32 ? logits32 : p.s.logits32;
   p.next_tok = next_tok;
+  p.loop = nullptr, p.ids = nullptr;
 #ifdef VKL_TRACE
   p.trace = g_trace;
 #endif
@@ -1993,29 +2057,156 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
     return launch_mega (p, G, lds, s);
   if (mode == 2)
     return launch_overlapped_step (p, m, G, lds, s);
-  for (int l = 0; l < m->n_layers; ++l)
-    {
-      const vkl_layer_weights &lw = m->layers_h[l];
-      if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
-        return e;
-      if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
-        return e;
-      if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
-        return e;
-      if (int e = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s))
-        return e;
-      if (int e = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s))
-        return e;
-    }
-  const vkl_layer_weights none = {};
-  if (int e = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s))
+  if (int e = launch_step (p, m, n_cu, G, lds, s))
     return e;
-  if (next_tok)
-    if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
-      return e;
   if (int e = timer_collect (s))
     return e;
   return vkl_launch_status ();
+}
+
+namespace
+{
+__global__ void
+set_loop_state_kernel (uint32_t *state, uint32_t index, uint32_t pos)
+{
+  state[0] = index;
+  state[1] = pos;
+}
+
+// One captured step per (model, id buffer, logits buffer, attention form).
+struct StepGraph
+{
+  const void *scratch = nullptr, *ids = nullptr, *logits = nullptr;
+  uint64_t model_hash = 0; // over every pointer and dimension the launches hold
+  int long_ctx = 0;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  uint64_t used = 0;
+};
+constexpr int kStepGraphs = 8;
+StepGraph g_graphs[kStepGraphs];
+uint64_t g_graph_clock = 0;
+
+uint64_t
+hash_model (const vkl_decode_model *m)
+{
+  uint64_t h = 1469598103934665603ull;
+  auto mix = [&h] (const void *p, size_t n) {
+    const uint8_t *b = (const uint8_t *)p;
+    for (size_t i = 0; i < n; ++i)
+      h = (h ^ b[i]) * 1099511628211ull;
+  };
+  mix (m, sizeof (*m));
+  mix (m->layers_h, sizeof (vkl_layer_weights) * (size_t)m->n_layers);
+  return h;
+}
+
+void
+drop_graph (StepGraph &g)
+{
+  if (g.exec)
+    (void)hipGraphExecDestroy (g.exec);
+  if (g.graph)
+    (void)hipGraphDestroy (g.graph);
+  g = StepGraph ();
+}
+}
+
+// Greedy steps replayed from a captured graph.  The launches of one token are
+// recorded once per form of the attention phase (one workgroup per head below
+// kAttnSplitMinLen positions, split above); token index and position live in
+// device memory and are advanced by the step's last kernel, so every replay
+// is the identical sequence of launches with identical arguments.
+extern "C" int
+vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
+                 int n_steps, float *logits32, void *stream)
+{
+  if (int e = check_model (m))
+    return e;
+  VKL_CHECK_ARG (ids != nullptr && n_steps >= 0);
+  VKL_CHECK_ARG ((uint64_t)pos0 + (uint64_t)n_steps <= (uint64_t)m->maxlen);
+  if (n_steps == 0)
+    return 0;
+  int dev = 0, n_cu = 0;
+  VKL_HIP (hipGetDevice (&dev));
+  VKL_HIP (hipDeviceGetAttribute (&n_cu, hipDeviceAttributeMultiprocessorCount,
+                                  dev));
+  const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
+  hipStream_t s = (hipStream_t)stream;
+  Params p;
+  p.m = *m;
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
+  p.tok = nullptr;
+  p.logits32 = logits32 ? logits32 : p.s.logits32;
+  p.next_tok = nullptr;
+  p.loop = p.s.sync + 16;
+  p.ids = ids;
+  p.wait_target = 0;
+#ifdef VKL_TRACE
+  p.trace = nullptr;
+#endif
+  const int G = n_cu * 2;
+  const bool timing = g_timer.on;
+  g_timer.on = false;
+  const uint64_t mh = hash_model (m);
+  set_loop_state_kernel<<<dim3 (1), dim3 (1), 0, s>>> ((uint32_t *)p.loop, 0u, pos0);
+  int err = 0;
+  int done = 0;
+  while (done < n_steps && !err)
+    {
+      // steps [done, upto) share one form of the attention phase
+      const int L_first = (int)pos0 + done + 1;
+      const int long_ctx = L_first >= kAttnSplitMinLen ? 1 : 0;
+      int upto = n_steps;
+      if (!long_ctx)
+        upto = std::min (n_steps, kAttnSplitMinLen - 1 - (int)pos0);
+      StepGraph *g = nullptr, *lru = &g_graphs[0];
+      for (StepGraph &c : g_graphs)
+        {
+          if (c.exec && c.scratch == m->scratch && c.ids == ids
+              && c.logits == p.logits32 && c.model_hash == mh
+              && c.long_ctx == long_ctx)
+            g = &c;
+          if (c.used < lru->used)
+            lru = &c;
+        }
+      if (!g)
+        {
+          g = lru;
+          drop_graph (*g);
+          // the position only sizes the attention launch: the largest one
+          // this form will see
+          p.pos = long_ctx ? (uint32_t)m->maxlen - 1 : (uint32_t)kAttnSplitMinLen - 2;
+          hipError_t e = hipStreamBeginCapture (s, hipStreamCaptureModeThreadLocal);
+          if (e != hipSuccess)
+            {
+              err = (int)e;
+              break;
+            }
+          err = launch_step (p, m, n_cu, G, lds, s);
+          e = hipStreamEndCapture (s, &g->graph);
+          if (!err && e != hipSuccess)
+            err = (int)e;
+          if (!err)
+            {
+              e = hipGraphInstantiate (&g->exec, g->graph, nullptr, nullptr, 0);
+              if (e != hipSuccess)
+                err = (int)e;
+            }
+          if (err)
+            {
+              drop_graph (*g);
+              break;
+            }
+          g->scratch = m->scratch, g->ids = ids, g->logits = p.logits32;
+          g->model_hash = mh, g->long_ctx = long_ctx;
+        }
+      g->used = ++g_graph_clock;
+      for (; done < upto && !err; ++done)
+        err = (int)hipGraphLaunch (g->exec, s);
+    }
+  g_timer.on = timing;
+  return err ? err : vkl_launch_status ();
 }
 
 extern "C" int
@@ -2060,6 +2251,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.pos = pos;
   p.logits32 = p.s.logits32;
   p.next_tok = nullptr;
+  p.loop = nullptr, p.ids = nullptr;
   p.wait_target = 0;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;

@@ -166,6 +166,8 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_lastblock_rope_quirk (value != 0);
   else if (n == "decode_mode")
     m->model->set_decode_mode (value);
+  else if (n == "decode_graph")
+    m->model->set_decode_graph (value != 0);
   else if (n == "phase_timing")
     vkl_decode_phase_timing (value);
   else

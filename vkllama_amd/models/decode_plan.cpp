@@ -143,6 +143,19 @@ DecodePlan::step_device_token (const uint32_t *tok, size_t offset,
 }
 
 absl::Status
+DecodePlan::loop (uint32_t *ids, size_t pos0, size_t n_steps)
+{
+  if (!usable_)
+    return absl::FailedPreconditionError (
+        "fused decode does not cover this model");
+  adopted_valid_ = false;
+  return hip_status ("decode loop",
+                     vkl_decode_loop (&desc_, ids, (uint32_t)pos0, (int)n_steps,
+                                      (float *)logits32_.data (),
+                                      gpu_->stream ()));
+}
+
+absl::Status
 DecodePlan::adopt_logits (Tensor logits32)
 {
   if (logits32.dtype () != FP32 || logits32.size () < vocab_)

@@ -32,6 +32,10 @@ struct DecodePlan
   // next_tok (optional, device-visible): receives the arg-max id of this step
   absl::Status step_device_token (const uint32_t *tok, size_t offset,
                                   uint32_t *next_tok = nullptr);
+  // n_steps greedy tokens replayed from a captured graph (vkl_decode_loop);
+  // ids is device memory, ids[0] the first input token
+  absl::Status loop (uint32_t *ids, size_t pos0, size_t n_steps);
+  int mode () const { return mode_; }
   // copies the fp32 logits of the last step (fused or adopted) to the host
   absl::Status read_logits (float *dst);
   // remember the fp32 logits tensor of an operator-chain pass

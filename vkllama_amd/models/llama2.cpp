@@ -500,7 +500,15 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
     return absl::InternalError (vkl_error_string (e));
   const auto t1 = clock::now ();
   size_t n_toks = prompt.size () + 1;
-  for (size_t i = 1; i < n_gen; ++i, ++n_toks)
+  size_t i0 = 1;
+  if (fused_decode_ && plan_->usable () && decode_graph_ && plan_->mode () == 0
+      && n_gen > 1)
+    {
+      // ids[0] is at position prompt.size (); each replay appends one id
+      VKLLAMA_STATUS_OK (plan_->loop (ids, prompt.size (), n_gen - 1));
+      i0 = n_gen;
+    }
+  for (size_t i = i0; i < n_gen; ++i, ++n_toks)
     {
       if (fused_decode_ && plan_->usable ())
         {

@@ -159,6 +159,9 @@ public:
   void set_lastblock_rope_quirk (bool on);
   // 0 = one launch per decode phase, 1 = one persistent launch per token
   void set_decode_mode (int mode);
+  // greedy loop replayed from a captured HIP graph (default) or launched
+  // step by step
+  void set_decode_graph (bool on) { decode_graph_ = on; }
   // Greedy loop of app/llama2_infer.cpp:140-218: prompt at offset 0, then one
   // token at a time at offset toks.size()-1; n_gen ids are written to out.
   // The wall-clock times of the two phases are returned in milliseconds.
@@ -198,6 +201,7 @@ private:
   Tensor next_tok_;
   std::unique_ptr<ArgMax> argmax_;
   DecodePlan *plan_;
+  bool decode_graph_ = true;
 };
 
 }
