@@ -112,7 +112,9 @@ def main():
         dev.sync()
         a.free(), b.free()
 
-    # warm-up: prompt pass + W decode steps, untimed
+    # warm-up: prompt pass + W decode steps, untimed (the prompt pass twice: its
+    # first two runs also load code objects and fill the tensor pool)
+    m.generate_greedy(prompt, 1)
     m.generate_greedy(prompt, warmup + 1)
     # timed: prompt pass (reported as prefill), then exactly `steps` decode steps
     ids, prefill_ms, decode_ms = m.generate_greedy(prompt, steps + 1)

@@ -16,8 +16,82 @@ GPUDevice::~GPUDevice ()
   if (stream_)
     {
       vkl_stream_sync (stream_);
+      trim ();
       vkl_stream_destroy (stream_);
     }
+}
+
+namespace
+{
+// size classes: 256 B steps below 1 MiB, 64 KiB steps above
+size_t
+size_class (size_t bytes)
+{
+  if (bytes == 0)
+    bytes = 1;
+  const size_t step = bytes < ((size_t)1 << 20) ? 256 : ((size_t)64 << 10);
+  return (bytes + step - 1) / step * step;
+}
+constexpr size_t kPoolLimit = (size_t)8 << 30;  // bytes kept for reuse
+constexpr size_t kPoolBlockMax = (size_t)1 << 30; // larger blocks go straight back
+}
+
+int
+GPUDevice::alloc (void **p, size_t bytes, bool host_visible)
+{
+  const size_t cls = size_class (bytes);
+  auto it = pool_.find ({ cls, host_visible });
+  if (it != pool_.end () && !it->second.empty ())
+    {
+      *p = it->second.back ();
+      it->second.pop_back ();
+      pooled_bytes_ -= cls;
+      return 0;
+    }
+  int e = host_visible ? vkl_host_malloc_h (p, cls) : vkl_malloc (p, cls);
+  if (e && pooled_bytes_)
+    {
+      // out of memory with blocks parked in the pool: give them back, retry
+      vkl_stream_sync (stream_);
+      trim ();
+      e = host_visible ? vkl_host_malloc_h (p, cls) : vkl_malloc (p, cls);
+    }
+  return e;
+}
+
+void
+GPUDevice::release (void *p, size_t bytes, bool host_visible)
+{
+  if (!p)
+    return;
+  const size_t cls = size_class (bytes);
+  if (cls > kPoolBlockMax || pooled_bytes_ + cls > kPoolLimit)
+    {
+      if (host_visible)
+        vkl_host_free_h (p);
+      else
+        vkl_free (p);
+      return;
+    }
+  pool_[{ cls, host_visible }].push_back (p);
+  pooled_bytes_ += cls;
+}
+
+void
+GPUDevice::trim ()
+{
+  for (auto &kv : pool_)
+    {
+      for (void *p : kv.second)
+        {
+          if (kv.first.second)
+            vkl_host_free_h (p);
+          else
+            vkl_free (p);
+        }
+      kv.second.clear ();
+    }
+  pooled_bytes_ = 0;
 }
 
 absl::Status

@@ -5,8 +5,11 @@
 #ifndef __VKLLAMA_CPP_GPU_DEVICE_H__
 #define __VKLLAMA_CPP_GPU_DEVICE_H__
 #include "absl/status/status.h"
+#include <map>
 #include <stddef.h>
 #include <string>
+#include <utility>
+#include <vector>
 
 namespace vkllama
 {
@@ -37,6 +40,17 @@ public:
   size_t total_memory () const { return total_mem_; }
   const std::string &name () const { return name_; }
 
+  // Pooled memory for tensors (the job VMA does in the reference,
+  // src/core/allocator.cpp): freed blocks are kept by size class and handed
+  // out again, so that the operator chain does not pay a driver allocation
+  // and release per intermediate tensor and pass.  All work runs on the one
+  // in-order stream, so a block reused by a later launch cannot be written
+  // before earlier launches have finished reading it.
+  int alloc (void **p, size_t bytes, bool host_visible);
+  void release (void *p, size_t bytes, bool host_visible);
+  // returns pooled blocks to the driver
+  void trim ();
+
 private:
   const int dev_;
   void *stream_;
@@ -45,6 +59,8 @@ private:
   size_t total_mem_;
   bool timing_;
   std::string name_;
+  std::map<std::pair<size_t, bool>, std::vector<void *>> pool_;
+  size_t pooled_bytes_ = 0;
 };
 }
 #endif

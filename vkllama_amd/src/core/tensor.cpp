@@ -1,4 +1,5 @@
 #include "src/core/tensor.h"
+#include "src/core/gpu_device.h"
 #include "absl/strings/str_format.h"
 #include "src/core/quants.h"
 #include "vkl_hip.h"
@@ -81,12 +82,7 @@ Tensor::release_ ()
   if (status_ && status_->ref_.fetch_sub (1) == 1)
     {
       if (data_)
-        {
-          if (visable_)
-            vkl_host_free_h (data_);
-          else
-            vkl_free (data_);
-        }
+        dev_->release (data_, status_->bytes_, visable_);
       delete status_;
     }
   status_ = nullptr;
@@ -135,13 +131,14 @@ Tensor::create ()
   update_strides_ ();
   const size_t n = bytes ();
   void *p = nullptr;
-  const int e = visable_ ? vkl_host_malloc_h (&p, n) : vkl_malloc (&p, n);
+  const int e = dev_->alloc (&p, n, visable_);
   if (e)
     return absl::InternalError (absl::StrFormat (
         "failed at allocating %zu bytes: %s", n, vkl_error_string (e)));
   data_ = p;
   status_ = new __TensorStatus ();
   status_->ref_.store (1);
+  status_->bytes_ = n;
   return absl::OkStatus ();
 }
 

@@ -75,6 +75,7 @@ private:
   struct __TensorStatus
   {
     std::atomic<int> ref_;
+    size_t bytes_ = 0; // size the block was requested with
   };
   __TensorStatus *status_;
 };
