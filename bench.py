@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llama2 token loop on one MI355X.
 
-A step is one batch-1 greedy decode token.  The default workload is BASELINE
+A step is one batch-1 greedy decode token.  The default workload is benchmark
 config 3: Llama-2-7B shape (dim 4096, 32 layers, 32 heads, FFN 11008, vocab
 32000, context 4096), random-init N(0, 0.02) weights quantised to Q8_0, fp16
 activations and KV cache, a 32-token random-id prompt, then K greedy decode
@@ -31,12 +31,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 WORKLOADS = {
-    # BASELINE configs 2, 3, 5 (config 4, FP16 weights, runs on the operator chain)
+    # the four model-level benchmark configurations
     "llama2-tiny-q8_0": dict(dim=512, n_layers=8, n_heads=8, ffn=1376, vocab=32000, maxlen=512, eps=1e-5, wtype=8,
                              prompt=16, prefill_kv=0),
     "llama2-7b-q8_0": dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5,
                            wtype=8, prompt=32, prefill_kv=0),
-    # BASELINE config 4: FP16 weights, 2048-token prompt
+    # FP16 weights, 2048-token prompt
     "llama2-7b-f16": dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5,
                           wtype=1, prompt=2048, prefill_kv=0),
     "llama2-13b-q8_0-ctx3968": dict(dim=5120, n_layers=40, n_heads=40, ffn=13824, vocab=32000, maxlen=4096,
@@ -80,8 +80,8 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (batch-1 decode is a single dependency chain; "
-                 "see DESIGN.md for how it would shard); got --gpus %d" % args.gpus)
+        sys.exit("bench.py: this build runs on ONE GPU (batch-1 decode is a single dependency chain and "
+                 "would shard by tensor parallelism, which is not built); got --gpus %d" % args.gpus)
 
     from vkllama_amd import capi, model as M
 

@@ -20,7 +20,7 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 SMALL = dict(dim=256, n_layers=3, n_heads=4, ffn=704, vocab=1024, maxlen=64, eps=1e-5, wtype=8)
 SMALL128 = dict(dim=256, n_layers=2, n_heads=2, ffn=352, vocab=640, maxlen=48, eps=1e-5, wtype=8)
-# BASELINE config 2
+# the tiny-llama benchmark configuration
 TINY = dict(dim=512, n_layers=8, n_heads=8, ffn=1376, vocab=32000, maxlen=512, eps=1e-5, wtype=8)
 
 
@@ -91,7 +91,7 @@ def test_greedy_ids_identical_to_oracle_small(cfg, seed, fused):
 
 
 def test_tiny_llama_config2_greedy_128_tokens():
-    """BASELINE config 2: prompt of 16 ids in [3, 32000), greedy 128 tokens;
+    """Tiny-llama benchmark configuration: prompt of 16 ids in [3, 32000), greedy 128 tokens;
     the first 32 must equal the oracle's (here: all of them are compared and
     the fixture pins the oracle's own sequence)."""
     w = M.synth_weights(TINY, seed=1234)

@@ -1,6 +1,6 @@
 """Parity of every HIP operator kernel with the CPU oracle, through the C ABI.
 
-Bars (BASELINE north star): bit-exact for Q8_0 repacking, embedding gather,
+Bars: bit-exact for Q8_0 repacking, embedding gather,
 KV-cache writes, arg-max ids and plain copies; fp16 outputs within 1e-2
 relative of the oracle (measured against max(|ref|, 1e-2 max|ref|)).
 """

@@ -4,7 +4,7 @@ import numpy as np
 
 def q8_weights(rng, N, K, lo=0.001, hi=0.01):
     """Random Q8_0 matrix as GGUF blocks (uint8 [N, K/32*34]) the way
-    BASELINE config 1 describes it: int8 uniform in [-127,127], fp16 scale
+    the single-GEMV benchmark configuration describes it: int8 uniform in [-127,127], fp16 scale
     uniform in (lo, hi).  Returns (raw, dequantised float64 [N, nb*32])."""
     nb = (K + 31) // 32
     q = rng.integers(-127, 128, size=(N, nb, 32), dtype=np.int8)
