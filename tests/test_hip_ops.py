@@ -239,7 +239,8 @@ def test_matmul_f16_tb(dev, rng, C, M, N, K):
     assert rel_err(f16(dy, (C, M, N)), O.matmul_f16_tb(a, b, scale=0.125)) < F16_REL_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512)])
+@pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512),
+                                   (512, 12800, 64), (600, 13000, 96)])
 def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     """FP16 weights, many token rows: the matrix-core path."""
     a = rng.standard_normal((1, M, K)).astype(np.float16)
