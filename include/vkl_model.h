@@ -45,6 +45,11 @@ typedef struct
 int vkl_model_create (int dev, const vkl_model_hparams *hp,
                       const vkl_tensor_desc *tensors, size_t n_tensors,
                       vkl_model **out);
+/* The same from a GGUF file, the way app/llama2_infer.cpp:46-75,120-121 of
+ * the reference loads a model: the file is mapped, its keys and tensors are
+ * collected into the maps Model::init takes, the weights are uploaded, and
+ * the mapping is released before this returns. */
+int vkl_model_load_gguf (int dev, const char *path_h, vkl_model **out);
 void vkl_model_destroy (vkl_model *m);
 const char *vkl_model_last_error (const vkl_model *m);
 size_t vkl_model_vocab (const vkl_model *m);

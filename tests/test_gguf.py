@@ -1,0 +1,111 @@
+"""GGUF files: the writer's output is read back by the reader with the
+gguf-tools calling interface (CPU), malformed files are refused, and a model
+loaded from a file behaves like the one created from the same weights (GPU)."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+from vkllama_amd import capi, gguf, model as M
+
+CFG = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=48, eps=1e-5, wtype=8)
+
+
+@pytest.fixture(scope="module")
+def model_file(tmp_path_factory):
+    w = M.synth_weights(CFG, seed=9)
+    path = str(tmp_path_factory.mktemp("gguf") / "tiny.gguf")
+    gguf.write_gguf(path, CFG, w, tokens=["<unk>", "<s>", "</s>", "a", "bc"])
+    return path, w
+
+
+def test_reader_returns_what_the_writer_wrote(model_file):
+    path, w = model_file
+    g = gguf.read_gguf(path)
+    assert g["version"] == 3
+    k = g["keys"]
+    assert k["llama.attention.head_count"] == (4, CFG["n_heads"])
+    assert k["llama.block_count"] == (4, CFG["n_layers"])
+    assert k["llama.context_length"] == (4, CFG["maxlen"])
+    assert k["llama.attention.layer_norm_rms_epsilon"][0] == 6
+    assert abs(k["llama.attention.layer_norm_rms_epsilon"][1] - CFG["eps"]) < 1e-12
+    assert k["general.architecture"] == (8, "llama")
+    assert k["tokenizer.ggml.tokens"][0] == 9           # arrays are skipped over, not decoded
+    assert list(g["tensors"]) == M.tensor_names(CFG["n_layers"])     # file order
+    for name, t in g["tensors"].items():
+        a = np.ascontiguousarray(w[name])
+        assert t["bsize"] == a.nbytes, name
+        assert np.array_equal(t["data"], a.view(np.uint8).ravel()), name
+        if name.endswith("norm.weight"):
+            assert t["type"] == 0 and t["dims"] == [CFG["dim"]]
+        else:
+            rows, K = M.matrix_shape(CFG, name)
+            assert t["type"] == 8 and t["dims"] == [K, rows]
+
+
+def test_malformed_files_are_refused(model_file, tmp_path):
+    path, _ = model_file
+    raw = open(path, "rb").read()
+    cases = {
+        "magic": b"GGUX" + raw[4:],
+        "version": raw[:4] + struct.pack("<I", 7) + raw[8:],
+        "truncated_header": raw[:200],
+        "truncated_data": raw[:len(raw) - 4096],
+        "huge_key_count": raw[:16] + struct.pack("<Q", 1 << 40) + raw[24:],
+        "empty": b"",
+    }
+    for name, data in cases.items():
+        p = str(tmp_path / (name + ".gguf"))
+        open(p, "wb").write(data)
+        with pytest.raises(OSError):
+            gguf.read_gguf(p)
+    with pytest.raises(OSError):
+        gguf.read_gguf(str(tmp_path / "missing.gguf"))
+
+
+@pytest.mark.gpu
+def test_model_from_gguf_equals_model_from_weights(model_file):
+    path, w = model_file
+    prompt = np.array([5, 17, 99, 3], np.uint32)
+    a = M.Llama2(CFG, w)
+    b = M.Llama2.from_gguf(path)
+    assert np.array_equal(a.forward(prompt, 0), b.forward(prompt, 0))
+    ia, _, _ = a.generate_greedy(prompt, 16)
+    ib, _, _ = b.generate_greedy(prompt, 16)
+    assert list(ia) == list(ib)
+    a.close(), b.close()
+    with pytest.raises(capi.VklError, match=r"\(5\)"):          # NotFound
+        M.Llama2.from_gguf(path + ".nope")
+
+
+@pytest.mark.gpu
+def test_infer_cli_on_a_gguf_file(model_file, capsys):
+    from vkllama_amd import infer
+    path, w = model_file
+    assert infer.main([path, "6", "--ids", "5", "17", "99"]) == 0
+    out = capsys.readouterr().out
+    ids = [int(t) for t in out.split("ids:")[1].split()]
+    m = M.Llama2(CFG, w)
+    want, _, _ = m.generate_greedy(np.array([5, 17, 99], np.uint32), 6)
+    m.close()
+    assert ids == [int(t) for t in want]
+
+
+@pytest.mark.gpu
+def test_cpp_llama2_infer_program(model_file):
+    """The C++ command-line program (the reference's app/llama2_infer.cpp flow
+    on the drop-in classes) prints the same greedy ids."""
+    import subprocess
+    path, w = model_file
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "vkllama_amd", "lib",
+                       "llama2_infer")
+    r = subprocess.run([exe, path, "6", "5", "17", "99"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-1500:]
+    ids = [int(t) for t in r.stdout.split()]
+    m = M.Llama2(CFG, w)
+    want, _, _ = m.generate_greedy(np.array([5, 17, 99], np.uint32), 6)
+    m.close()
+    assert ids == [int(t) for t in want]
+    bad = subprocess.run([exe, path + ".nope", "2", "1"], capture_output=True, text=True, timeout=60)
+    assert bad.returncode == 1 and "GGUF" in bad.stderr

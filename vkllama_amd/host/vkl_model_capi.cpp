@@ -1,6 +1,7 @@
 // extern "C" wrappers around vkllama::Model and the synthetic-weight helpers
 // (include/vkl_model.h).
 #include "vkl_model.h"
+#include "models/gguflib.h"
 #include "models/llama2.h"
 #include "vkl_decode.h"
 #include "vkl_hip.h"
@@ -86,6 +87,38 @@ vkl_model_create (int dev, const vkl_model_hparams *hp,
       return fail (m, absl::InternalError (e.what ()));
     }
   return 0;
+}
+
+extern "C" int
+vkl_model_load_gguf (int dev, const char *path, vkl_model **out)
+{
+  if (!path || !out)
+    return (int)absl::StatusCode::kInvalidArgument;
+  auto *m = new vkl_model ();
+  *out = m;
+  gguf_ctx *g = gguf_open (path);
+  if (!g)
+    return fail (m, absl::NotFoundError (std::string ("not a readable GGUF file: ") + path));
+  std::map<std::string, gguf_key> kv;
+  std::map<std::string, gguf_tensor> ts;
+  gguf_key key;
+  while (gguf_get_key (g, &key))
+    kv[std::string (key.name, key.namelen)] = key;
+  gguf_tensor t;
+  while (gguf_get_tensor (g, &t))
+    ts[std::string (t.name, t.namelen)] = t;
+  m->model = new vkllama::Model (dev);
+  absl::Status s = absl::OkStatus ();
+  try
+    {
+      s = m->model->init (kv, ts);
+    }
+  catch (const std::exception &e)
+    {
+      s = absl::InternalError (e.what ());
+    }
+  gguf_close (g); // every weight has been copied to the device by now
+  return s.ok () ? 0 : fail (m, s);
 }
 
 extern "C" void

@@ -23,6 +23,7 @@ class HParams(C.Structure):
 
 SIGNATURES = {
     "vkl_model_create": (i32, [i32, C.POINTER(HParams), C.POINTER(TensorDesc), sz, C.POINTER(vp)]),
+    "vkl_model_load_gguf": (i32, [i32, C.c_char_p, C.POINTER(vp)]),
     "vkl_model_destroy": (None, [vp]),
     "vkl_model_last_error": (C.c_char_p, [vp]),
     "vkl_model_vocab": (sz, [vp]),
@@ -123,6 +124,22 @@ class Llama2:
         self._h = h
         if rc:
             raise capi.VklError("vkl_model_create failed (%d): %s" % (rc, self._err()))
+
+    @classmethod
+    def from_gguf(cls, path, dev=0):
+        """Loads a GGUF file the way app/llama2_infer.cpp of the reference does
+        (keys and tensors through the gguf reader, then Model::init)."""
+        self = cls.__new__(cls)
+        self._h = None
+        h = vp()
+        rc = lib().vkl_model_load_gguf(dev, path.encode(), C.byref(h))
+        self._h = h
+        if rc:
+            msg = self._err()
+            self.close()
+            raise capi.VklError("vkl_model_load_gguf failed (%d): %s" % (rc, msg))
+        self.cfg = {"vocab": int(lib().vkl_model_vocab(self._h))}
+        return self
 
     def _err(self):
         m = lib().vkl_model_last_error(self._h)

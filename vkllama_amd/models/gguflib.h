@@ -60,5 +60,49 @@ typedef struct
   uint64_t num_weights;
   uint8_t *weights_data;
 } gguf_tensor;
+
+/* GGUF metadata value types (the file format's numbering) */
+enum gguf_value_type
+{
+  GGUF_VALUE_TYPE_UINT8 = 0,
+  GGUF_VALUE_TYPE_INT8 = 1,
+  GGUF_VALUE_TYPE_UINT16 = 2,
+  GGUF_VALUE_TYPE_INT16 = 3,
+  GGUF_VALUE_TYPE_UINT32 = 4,
+  GGUF_VALUE_TYPE_INT32 = 5,
+  GGUF_VALUE_TYPE_FLOAT32 = 6,
+  GGUF_VALUE_TYPE_BOOL = 7,
+  GGUF_VALUE_TYPE_STRING = 8,
+  GGUF_VALUE_TYPE_ARRAY = 9,
+  GGUF_VALUE_TYPE_UINT64 = 10,
+  GGUF_VALUE_TYPE_INT64 = 11,
+  GGUF_VALUE_TYPE_FLOAT64 = 12,
+};
+
+/* The part of gguf-tools' reader interface that app/llama2_infer.cpp:46-75 of
+ * the reference uses, implemented in models/gguf_reader.cpp from the GGUF
+ * file format (versions 2 and 3, little endian): the file is mapped read-only
+ * and keys / tensors are handed out in file order; names and values point
+ * into the mapping and stay valid until gguf_close. */
+typedef struct gguf_ctx gguf_ctx;
+#ifdef __cplusplus
+extern "C" {
+#endif
+gguf_ctx *gguf_open (const char *filename);
+void gguf_close (gguf_ctx *ctx);
+void gguf_rewind (gguf_ctx *ctx);
+/* 1 and *key filled while keys remain, then 0 */
+int gguf_get_key (gguf_ctx *ctx, gguf_key *key);
+/* 1 and *tensor filled while tensors remain, then 0; all keys are skipped
+ * first if the caller has not read them */
+int gguf_get_tensor (gguf_ctx *ctx, gguf_tensor *tensor);
+const char *gguf_get_value_type_name (uint32_t type);
+const char *gguf_get_tensor_type_name (uint32_t type);
+uint32_t gguf_version (const gguf_ctx *ctx);
+uint64_t gguf_tensor_count (const gguf_ctx *ctx);
+uint64_t gguf_key_count (const gguf_ctx *ctx);
+#ifdef __cplusplus
+}
+#endif
 #endif
 #endif
