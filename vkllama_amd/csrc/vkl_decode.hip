@@ -332,12 +332,13 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         {
+          const bool in = (threadIdx.x + j * kDecThreads) * 8 < K;
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             {
-              const float a = h2f ((uint16_t)(w[i] & 0xffff));
-              const float b = h2f ((uint16_t)(w[i] >> 16));
+              const float a = in ? h2f ((uint16_t)(w[i] & 0xffff)) : 0.f;
+              const float b = in ? h2f ((uint16_t)(w[i] >> 16)) : 0.f;
               s += a * a;
               s += b * b;
             }
@@ -538,22 +539,27 @@ template <bool COH, int WT = 8> struct Gemv
     const uint8_t *q[R];
     const uint16_t *d[R];
     rows_of (ps, u, q, d);
-    // the residual pair of the unit travels with the item, so the epilogue
-    // does not start a dependent trip to memory at the end of the row
-    b.res = 0;
-    if (ps.residual && 2 * u + 1 < ps.N)
-      b.res = ld_u32<COH> ((const uint32_t *)(ps.residual + 2 * u));
+    // Every load below is unconditional, from a clamped (always valid)
+    // address; what lies outside the row is ignored when the item is
+    // consumed.  A branch around a load would keep the compiler from counting
+    // the loads in flight, and the wait for one item would then wait for
+    // the next one as well.
+    //
+    // The residual pair of the unit travels with the item, so the epilogue
+    // does not start a dependent trip to memory at the end of the row.
+    const uint16_t *rp = ps.residual ? ps.residual : (const uint16_t *)ps.m0.q;
+    b.res = ld_u32<COH> ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
 #pragma unroll
     for (int s = 0; s < S; ++s)
       {
         const int kk = c * CHUNK + s * (VKL_WAVE * 16) + ps.lane * 16;
-        const bool ok = kk < ps.Kp;
+        const int kc = kk < ps.Kp ? kk : 0;
 #pragma unroll
         for (int r = 0; r < R; ++r)
           {
-            b.w[r * S + s] = ok ? ldg4 (q[r] + kk) : make_uint4 (0, 0, 0, 0);
+            b.w[r * S + s] = ldg4 (q[r] + kc);
             if (WT == 8)
-              b.d[r * S + s] = ok ? ldg (d[r] + (kk >> 5)) : (uint16_t)0;
+              b.d[r * S + s] = ldg (d[r] + (kc >> 5));
           }
       }
   }
