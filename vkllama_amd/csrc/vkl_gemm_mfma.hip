@@ -27,8 +27,19 @@ namespace
 typedef _Float16 half8 __attribute__ ((ext_vector_type (8)));
 typedef float float16v __attribute__ ((ext_vector_type (16)));
 
-constexpr int BN = 128, BK = 32;
-constexpr int LDK = BK + 8; // LDS row stride in halves (80 B: conflict-free b128 reads)
+constexpr int BN = 128;
+// k extent of a step.  Q8_0: one block, so that the block scale applies to a
+// whole step.  fp16 weights: 64, so that the eight 16-byte chunks of a tile
+// row are one full 128-byte cache line (with 32, every request is half a
+// line and the L2 delivers half the bytes per cycle).
+template <int WT> struct Geo
+{
+  static constexpr int BK = WT == 8 ? 32 : 64;
+  static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
+  static constexpr int LDK = BK + 8;  // LDS row stride in halves: 80 or 144
+                                      // bytes, conflict-free 16-byte accesses
+  static constexpr int NB = WT == 8 ? 1 : BN * CPR / 256; // weight chunks per thread
+};
 constexpr int kGemmThreads = 256;
 // k-tiles in flight in registers: more for the small-M configuration, where
 // few workgroups run and each has to hide the memory latency alone
@@ -51,14 +62,16 @@ keep_if (bool c, const uint4 v)
   return make_uint4 (c ? v.x : 0u, c ? v.y : 0u, c ? v.z : 0u, c ? v.w : 0u);
 }
 
+__device__ __align__ (16) const uint32_t g_zero_chunk[4] = { 0, 0, 0, 0 };
+
 template <int BM, int WT>
 struct TileLoads
 {
-  static constexpr int ACH = BM * 4 / kGemmThreads; // 16-byte chunks of x per thread
+  static constexpr int ACH = BM * Geo<WT>::CPR / kGemmThreads; // 16-byte chunks of x per thread
+  static constexpr int NB = Geo<WT>::NB;
   uint4 a[ACH];
-  uint4 b[2];  // fp16: two chunks; Q8_0: b[0] = 16 quants
+  uint4 b[NB]; // fp16: weight chunks; Q8_0: b[0] = 16 quants
   uint16_t bd; // Q8_0 block scale
-  uint32_t ok; // validity bits: x chunks from bit 0, weight chunks from bit 8
 };
 
 // Per-thread source addresses of the tile loads.  They depend on k only
@@ -70,13 +83,14 @@ struct TileLoads
 template <int BM, int WT>
 struct TileAddr
 {
-  static constexpr int ACH = BM * 4 / kGemmThreads;
+  static constexpr int ACH = BM * Geo<WT>::CPR / kGemmThreads;
+  static constexpr int NB = Geo<WT>::NB;
   const uint16_t *a[ACH]; // x chunk at k = 0, or null beyond M
   int ak[ACH];            // its column offset within a k-step
   const uint8_t *bq;      // Q8_0: quants of this thread's row at k = 0
   const uint16_t *bd;     // Q8_0: its scales
-  const uint16_t *b[2];   // fp16: chunk pointers at k = 0
-  int bk[2];              // fp16 [N, K]: column offset; [K, N]: row offset
+  const uint16_t *b[NB];  // fp16: chunk pointers at k = 0
+  int bk[NB];             // fp16 [N, K]: column offset; [K, N]: row offset
 };
 
 __device__ __forceinline__ const void *
@@ -91,17 +105,19 @@ tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
                 int n0, TileAddr<BM, WT> &ta)
 {
   const int tid = threadIdx.x;
+  constexpr int CPR = Geo<WT>::CPR, NB = Geo<WT>::NB;
 #pragma unroll
   for (int i = 0; i < TileAddr<BM, WT>::ACH; ++i)
     {
       const int c = tid + i * kGemmThreads;
-      const int m = m0 + (c >> 2);
-      ta.ak[i] = (c & 3) * 8;
+      const int m = m0 + c / CPR;
+      ta.ak[i] = (c % CPR) * 8;
       ta.a[i] = m < a.M ? a.x + xoff + (size_t)m * a.xs + ta.ak[i] : nullptr;
     }
   ta.bq = nullptr, ta.bd = nullptr;
-  ta.b[0] = ta.b[1] = nullptr;
-  ta.bk[0] = ta.bk[1] = 0;
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+    ta.b[i] = nullptr, ta.bk[i] = 0;
   if (WT == 8)
     {
       const int v = tid >> 1, seg = tid & 1;
@@ -118,7 +134,7 @@ tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
   else if (WT == 2)
     {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
         {
           const int c = tid + i * kGemmThreads;
           const int n = n0 + (c & 15) * 8;
@@ -131,13 +147,13 @@ tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
   else
     {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
         {
           const int c = tid + i * kGemmThreads;
-          const int v = c >> 2;
+          const int v = c / CPR;
           const int mat = a.upgate ? (v >> 6) : zmat;
           const int n = a.upgate ? n0 + (v & 63) : n0 + v;
-          ta.bk[i] = (c & 3) * 8;
+          ta.bk[i] = (c % CPR) * 8;
           if (n < a.N)
             ta.b[i] = (const uint16_t *)pick3 (a.wh[0], a.wh[1], a.wh[2], mat)
                       + woff + (size_t)n * a.ws + ta.bk[i];
@@ -145,47 +161,42 @@ tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
     }
 }
 
-// Every load is issued unconditionally (from a clamped, always valid address)
-// and masked to zero when the tile is stored: with no branch around a load
-// the compiler can count the loads in flight and wait for exactly the tile it
-// needs instead of for all of them.
+// Every load is issued unconditionally: with no branch around a load the
+// compiler can count the loads in flight and wait for exactly the tile it
+// needs instead of for all of them.  A chunk outside the matrices (rows
+// beyond M or N, columns beyond K) is read from a block of zeros instead, so
+// nothing has to be masked after the load: a select on loaded data would be
+// scheduled early and wait for the newest tile, which leaves one k-step of
+// look-ahead whatever the depth.
 template <int BM, int WT>
 __device__ __forceinline__ void
 issue_tile (const GemmArgs &a, const TileAddr<BM, WT> &ta, int k0,
             TileLoads<BM, WT> &t)
 {
-  uint32_t ok = 0;
+  const void *zeros = g_zero_chunk;
 #pragma unroll
   for (int i = 0; i < TileLoads<BM, WT>::ACH; ++i)
     {
       const bool v = ta.a[i] != nullptr && k0 + ta.ak[i] < a.K;
-      const uint16_t *p = v ? ta.a[i] + k0 : a.x;
-      t.a[i] = ldg16 (p);
-      ok |= (v ? 1u : 0u) << i;
+      t.a[i] = ldg16 (v ? (const void *)(ta.a[i] + k0) : zeros);
     }
   if (WT == 8)
     {
+      // rows beyond N: zero quants and a zero scale
       const bool v = ta.bq != nullptr;
-      const uint8_t *pq = v ? ta.bq + k0 : a.wq[0];
-      const uint16_t *pd = v ? ta.bd + (k0 >> 5) : a.wd[0];
-      t.b[0] = ldg16 (pq);
-      t.bd = ldg (pd);
-      ok |= (v ? 1u : 0u) << 8;
+      t.b[0] = ldg16 (v ? (const void *)(ta.bq + k0) : zeros);
+      t.bd = ldg (v ? ta.bd + (k0 >> 5) : (const uint16_t *)zeros);
     }
   else
     {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < Geo<WT>::NB; ++i)
         {
           const bool v = ta.b[i] != nullptr && k0 + ta.bk[i] < a.K;
-          const uint16_t *p
-              = v ? ta.b[i] + (WT == 2 ? (size_t)k0 * a.ws : (size_t)k0)
-                  : a.wh[0];
-          t.b[i] = ldg16 (p);
-          ok |= (v ? 1u : 0u) << (8 + i);
+          t.b[i] = ldg16 (v ? (const void *)(ta.b[i] + (WT == 2 ? (size_t)k0 * a.ws : (size_t)k0))
+                            : zeros);
         }
     }
-  t.ok = ok;
 }
 
 template <int BM, int WT>
@@ -194,20 +205,19 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
             uint16_t *Ds)
 {
   const int tid = threadIdx.x;
+  constexpr int CPR = Geo<WT>::CPR, LDK = Geo<WT>::LDK, NB = Geo<WT>::NB;
 #pragma unroll
   for (int i = 0; i < TileLoads<BM, WT>::ACH; ++i)
     {
       const int c = tid + i * kGemmThreads;
-      const int row = c >> 2, seg = c & 3;
-      *(uint4 *)(As + row * LDK + seg * 8) = keep_if ((t.ok >> i) & 1, t.a[i]);
+      const int row = c / CPR, seg = c % CPR;
+      *(uint4 *)(As + row * LDK + seg * 8) = t.a[i];
     }
   if (WT == 8)
     {
       const int v = tid >> 1, seg = tid & 1;
-      const bool okb = (t.ok >> 8) & 1;
       if (seg == 0)
-        Ds[v] = okb ? t.bd : (uint16_t)0;
-      // quants of rows beyond N need no masking: their scale is zero
+        Ds[v] = t.bd;
       const uint32_t w[4] = { t.b[0].x, t.b[0].y, t.b[0].z, t.b[0].w };
       uint32_t o[8];
 #pragma unroll
@@ -226,13 +236,11 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
     {
       // transpose on the way in: LDS holds the tile as [column][k]
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
         {
           const int c = tid + i * kGemmThreads;
           const int kr = c >> 4, v = (c & 15) * 8;
-          const bool okb = (t.ok >> (8 + i)) & 1;
-          const uint32_t w[4] = { okb ? t.b[i].x : 0u, okb ? t.b[i].y : 0u,
-                                  okb ? t.b[i].z : 0u, okb ? t.b[i].w : 0u };
+          const uint32_t w[4] = { t.b[i].x, t.b[i].y, t.b[i].z, t.b[i].w };
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             {
@@ -244,11 +252,11 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
   else
     {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
         {
           const int c = tid + i * kGemmThreads;
-          const int v = c >> 2, seg = c & 3;
-          *(uint4 *)(Bs + v * LDK + seg * 8) = keep_if ((t.ok >> (8 + i)) & 1, t.b[i]);
+          const int v = c / CPR, seg = c % CPR;
+          *(uint4 *)(Bs + v * LDK + seg * 8) = t.b[i];
         }
     }
 }
@@ -262,10 +270,11 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
 {
   constexpr int TM = BM / 64;
   constexpr int D = GemmDepth<BM>::value;
+  constexpr int BK = Geo<WT>::BK, LDK = Geo<WT>::LDK, KS = BK / 16;
   const int lane = threadIdx.x & 63;
-  half8 af[2][TM], bf[2][2];
+  half8 af[KS][TM], bf[KS][2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
+  for (int ks = 0; ks < KS; ++ks)
     {
       const int kof = ks * 16 + (lane >> 5) * 8;
 #pragma unroll
@@ -296,7 +305,7 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
   else
     {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+      for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
@@ -320,6 +329,7 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
   const size_t bi = a.batch > 1 ? blockIdx.y : 0;
   const size_t xoff = bi * a.xbs, woff = bi * a.wbs, yoff = bi * a.ybs;
   constexpr int TM = BM / 64; // 32-row accumulators per wave along M
+  constexpr int BK = Geo<WT>::BK, LDK = Geo<WT>::LDK;
   __shared__ __align__ (16) uint16_t As[2][BM * LDK];
   __shared__ __align__ (16) uint16_t Bs[2][BN * LDK];
   __shared__ uint16_t Ds[2][BN]; // Q8_0 block scales of the tile rows
