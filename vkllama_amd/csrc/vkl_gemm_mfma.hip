@@ -320,7 +320,7 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
 }
 
 template <int BM, int WT>
-__global__ __launch_bounds__ (kGemmThreads) void
+__global__ __launch_bounds__ (kGemmThreads, 2) void
 gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
 {
   // element offsets of this problem of the batch (the argument block itself
