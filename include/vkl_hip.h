@@ -139,6 +139,21 @@ int vkl_kv_update_f16 (void *cache, const void *kv, int C, int HO, int H,
 /* src/ops/softmax.cpp:52-92, src/shaders/softmax_fp16.comp */
 int vkl_softmax_f16 (const void *x, int C, int H, int W, int seq_mask,
                      uint32_t offset, void *out, void *stream);
+/* The attention core of src/ops/multiheadattention_v2.cpp:290-309 in one
+ * launch for many query rows: matmul_b0_tb_fp16_v2.comp (scores = fp16(scale
+ * q.k)), softmax_fp16.comp with seq_mask (key l is masked iff l > s + (L - S))
+ * and matmul_broadcast0_fp16_v2.comp (P V), with the same fp16 rounding points
+ * and neither scores nor probabilities stored.  q [H,S,hd] with strides (qcs,
+ * qhs); k, v [H,L,hd] views with strides (kcs, khs), (vcs, vhs), e.g. the
+ * first L rows of a [H,maxlen,hd] cache; out[s*ors + h*ohs + d] (ors = H*hd,
+ * ohs = hd gives the [S, H*hd] layout the output projection reads; ors = hd,
+ * ohs = S*hd gives [H,S,hd]).  hd 64 or 128; strides in elements. */
+int vkl_attn_prefill_causal_f16 (const void *q, const void *k, const void *v,
+                                 int H, int S, int L, int hd, size_t qcs,
+                                 size_t qhs, size_t kcs, size_t khs,
+                                 size_t vcs, size_t vhs, float scale,
+                                 void *out, size_t ors, size_t ohs,
+                                 void *stream);
 /* src/ops/elementwise.cpp:60-101, src/shaders/element_wise_fp16.comp:
  * y = fp16(x op y), in place into y; op 0..3 = add, sub, mul, div */
 int vkl_elementwise_f16 (const void *x, void *y, size_t n, int op,

@@ -289,6 +289,38 @@ def test_attention_products_many_rows(dev, rng, H, S, Lk, hd, maxlen):
     assert rel_err(f16(do, (H, S, hd)), want_o) < F16_REL_TOL
 
 
+@pytest.mark.parametrize("H,S,Lk,hd,maxlen,flat", [
+    (8, 40, 40, 64, 64, True), (3, 130, 200, 128, 256, False), (2, 9, 77, 64, 128, True),
+    (8, 300, 300, 128, 320, True), (16, 1, 150, 128, 160, True), (8, 257, 385, 64, 512, False)])
+def test_attn_prefill_causal(dev, rng, H, S, Lk, hd, maxlen, flat):
+    """One-launch prompt attention against the three separate operators of the
+    oracle (scores with fp16 rounding, masked softmax, P V).  A score whose
+    fp32 value lies next to an fp16 rounding boundary rounds either way
+    depending on the summation order of the dot product, which moves one
+    probability by 2^-11 relative; the tolerance is therefore 1e-2 relative to
+    max(|o|, 0.1 * sum_l p[l] |v[l]|), the size of the terms summed, not to a
+    possibly cancelled |o| alone."""
+    q = rng.standard_normal((H, S, hd)).astype(np.float16)
+    kc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    vc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    kc[:, Lk:] = np.float16(np.nan)   # rows past L must not be touched
+    vc[:, Lk:] = np.float16(np.nan)
+    dq, dk, dv = dev.upload(q), dev.upload(kc), dev.upload(vc)
+    do = dev.alloc(H * S * hd * 2)
+    sc = 1.0 / np.sqrt(hd)
+    ors, ohs = (H * hd, hd) if flat else (hd, S * hd)
+    capi.check(L().vkl_attn_prefill_causal_f16(dq.ptr, dk.ptr, dv.ptr, H, S, Lk, hd, S * hd, hd, maxlen * hd, hd,
+                                               maxlen * hd, hd, sc, do.ptr, ors, ohs, dev.stream))
+    scores = O.matmul_f16_tb(q, np.ascontiguousarray(kc[:, :Lk]), scale=sc)
+    p = O.softmax(scores, True, Lk - S)
+    want = O.matmul_f16_nn(p, np.ascontiguousarray(vc[:, :Lk]))
+    got = f16(do, (S, H, hd)).transpose(1, 0, 2) if flat else f16(do, (H, S, hd))
+    assert np.isfinite(got.astype(np.float32)).all()
+    terms = np.einsum("hsl,hld->hsd", p.astype(np.float64), np.abs(vc[:, :Lk].astype(np.float64)))
+    denom = np.maximum(np.abs(want.astype(np.float64)), 0.1 * terms)
+    assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)) / denom)) < F16_REL_TOL
+
+
 def test_matmul_f16_tb_reads_cache_view(dev, rng):
     """scores = Q K^T over the first L rows of a [H, maxlen, hd] cache."""
     H, maxlen, hd, Lk, S = 4, 64, 64, 37, 3

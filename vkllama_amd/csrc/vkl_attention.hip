@@ -1,0 +1,358 @@
+// Attention of many query rows over the K/V rows of a prompt, one kernel per
+// call: scores, masked softmax and the product with V without the [H, S, L]
+// score and probability tensors ever reaching memory.
+//
+// The values rounded to fp16 are the ones the separate operators round:
+// score = fp16(scale * q.k), probability = fp16(exp(score - max) / sum), the
+// output sum_l p[l] v[l] in fp32 and rounded once.  To know max and sum before
+// the first probability is formed, the keys are walked twice: pass 1 computes
+// the scores and keeps a running maximum and a running sum of exponentials per
+// query, pass 2 computes the scores again, turns them into probabilities and
+// accumulates P V.  (The maximum is taken over the keys a query may see; it
+// cancels in the quotient, so taking it over masked keys as well, as the
+// separate softmax operator does, changes the result by fp32 rounding only.)
+//
+// Workgroup = 4 waves = 128 query rows of one head, 32 per wave; the keys come
+// through LDS in tiles of 64.  Both products run on v_mfma_f32_32x32x16_f16 in
+// the transposed form, so that a lane's accumulator registers belong to ONE
+// query:
+//   S^T[key, q] = sum_d K[key, d] Q[q, d]      A = K tile (LDS), B = Q (regs)
+//   O^T[d, q]   = sum_key V^T[d, key] P^T[key, q]   A = V^T tile (LDS), B = P^T
+// Lane l of a wave owns query l % 32.  Of a 32-key block its 16 accumulator
+// registers hold the keys 8*(r/4) + 4*(l/32) + r%4, so maximum and sum over
+// keys are sums over a lane's own registers (the two lane halves are merged
+// once, after pass 1), and the probabilities it forms are, as they lie, the B
+// operand of the second product: registers 8t .. 8t+7 are the eight k values
+// of lane half l/32 in k-step t.  The V tile is written to LDS transposed and
+// with its keys permuted to that same order (slot 16t + 8h + j holds key
+// 16t + 8*(j/4) + 4h + j%4 of the block), so the A operand of the second
+// product is one 16-byte LDS read.
+#include "../../include/vkl_hip.h"
+#include "vkl_common.h"
+
+namespace
+{
+typedef _Float16 half8 __attribute__ ((ext_vector_type (8)));
+typedef float float16v __attribute__ ((ext_vector_type (16)));
+typedef uint32_t u32x2 __attribute__ ((ext_vector_type (2)));
+
+constexpr int kBQ = 128;      // query rows per workgroup
+constexpr int kBKey = 64;     // keys per tile
+constexpr int kThreads = 256;
+constexpr float kNeg = -1.0e30f; // "no key seen yet": finite, so that kNeg - kNeg = 0
+
+struct AttnArgs
+{
+  const uint16_t *q, *k, *v;
+  uint16_t *out;
+  int H, S, L, ntq;
+  size_t qcs, qhs, kcs, khs, vcs, vhs, ors, ohs;
+  float scale;
+};
+
+__device__ __align__ (16) const uint32_t g_zero16[4] = { 0, 0, 0, 0 };
+
+__device__ __forceinline__ float
+fast_exp (float x)
+{
+  return __builtin_amdgcn_exp2f (x * 1.44269504088896340736f);
+}
+
+__device__ __forceinline__ half8
+as_half8 (const uint4 v)
+{
+  return __builtin_bit_cast (half8, v);
+}
+
+template <int HD> struct Tile
+{
+  static constexpr int CPR = HD / 8;                       // 16-byte chunks per row
+  static constexpr int KCH = kBKey * CPR / kThreads;       // K chunks per thread
+  static constexpr int VIT = (kBKey / 2) * CPR / kThreads; // (key pair, chunk) items per thread
+  uint4 k[KCH];
+  uint4 v[VIT][2];
+};
+
+// K rows [t*64, t*64+64) of the head, as they lie; rows beyond L read zeros
+template <int HD>
+__device__ __forceinline__ void
+load_k (const AttnArgs &a, const uint16_t *kb, int t, Tile<HD> &r)
+{
+  constexpr int CPR = Tile<HD>::CPR;
+  const void *zeros = g_zero16;
+#pragma unroll
+  for (int i = 0; i < Tile<HD>::KCH; ++i)
+    {
+      const int c = threadIdx.x + i * kThreads;
+      const int row = t * kBKey + c / CPR;
+      r.k[i] = vkl::ldg4 (row < a.L ? (const void *)(kb + (size_t)row * a.khs + (c % CPR) * 8)
+                                    : zeros);
+    }
+}
+
+// key of slot s (0..63) of a tile
+__device__ __forceinline__ int
+slot_key (int s)
+{
+  const int blk = s >> 5, t = (s >> 4) & 1, h = (s >> 3) & 1, j = s & 7;
+  return 32 * blk + 16 * t + 8 * (j >> 2) + 4 * h + (j & 3);
+}
+
+template <int HD>
+__device__ __forceinline__ void
+load_v (const AttnArgs &a, const uint16_t *vb, int t, Tile<HD> &r)
+{
+  const void *zeros = g_zero16;
+#pragma unroll
+  for (int i = 0; i < Tile<HD>::VIT; ++i)
+    {
+      const int it = threadIdx.x + i * kThreads;
+      const int pair = it & 31, dc = it >> 5;
+      // slots 2*pair and 2*pair+1 hold two adjacent keys
+      const int row = t * kBKey + slot_key (2 * pair);
+      r.v[i][0] = vkl::ldg4 (row < a.L ? (const void *)(vb + (size_t)row * a.vhs + dc * 8) : zeros);
+      r.v[i][1] = vkl::ldg4 (row + 1 < a.L ? (const void *)(vb + (size_t)(row + 1) * a.vhs + dc * 8)
+                                           : zeros);
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void
+store_k (const Tile<HD> &r, uint16_t *Ks)
+{
+  constexpr int CPR = Tile<HD>::CPR, LDK = HD + 8;
+#pragma unroll
+  for (int i = 0; i < Tile<HD>::KCH; ++i)
+    {
+      const int c = threadIdx.x + i * kThreads;
+      *(uint4 *)(Ks + (c / CPR) * LDK + (c % CPR) * 8) = r.k[i];
+    }
+}
+
+// V^T: row = d, column = slot; a thread writes the two keys of its pair as one
+// 32-bit word per d
+template <int HD>
+__device__ __forceinline__ void
+store_v (const Tile<HD> &r, uint16_t *Vt)
+{
+  constexpr int LDV = kBKey + 8;
+#pragma unroll
+  for (int i = 0; i < Tile<HD>::VIT; ++i)
+    {
+      const int it = threadIdx.x + i * kThreads;
+      const int pair = it & 31, dc = it >> 5;
+      const uint32_t va[4] = { r.v[i][0].x, r.v[i][0].y, r.v[i][0].z, r.v[i][0].w };
+      const uint32_t vb[4] = { r.v[i][1].x, r.v[i][1].y, r.v[i][1].z, r.v[i][1].w };
+      uint32_t *dst = (uint32_t *)(Vt + (size_t)(dc * 8) * LDV + 2 * pair);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        {
+          dst[(2 * e) * (LDV / 2)] = (va[e] & 0xffffu) | (vb[e] << 16);
+          dst[(2 * e + 1) * (LDV / 2)] = (va[e] >> 16) | (vb[e] & 0xffff0000u);
+        }
+    }
+}
+
+// S^T of one 32-key block: rows = keys 32*blk .. +31 of the tile in LDS
+template <int HD>
+__device__ __forceinline__ float16v
+score_block (const uint16_t *Ks, int blk, const half8 (&qf)[HD / 16], int lane)
+{
+  constexpr int LDK = HD + 8;
+  float16v acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+  const uint16_t *kp = Ks + (32 * blk + (lane & 31)) * LDK + (lane >> 5) * 8;
+#pragma unroll
+  for (int kt = 0; kt < HD / 16; ++kt)
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16 (*(const half8 *)(kp + kt * 16), qf[kt], acc,
+                                                  0, 0, 0);
+  return acc;
+}
+
+template <int HD>
+__global__ __launch_bounds__ (kThreads, 2) void
+attn_prefill_kernel (const AttnArgs a)
+{
+  constexpr int KT = HD / 16, DB = HD / 32;
+  constexpr int LDK = HD + 8, LDV = kBKey + 8;
+  __shared__ __align__ (16) uint16_t Ks[kBKey * LDK];
+  __shared__ __align__ (16) uint16_t Vt[HD * LDV];
+
+  // Heavy query tiles (the last ones: most keys) first.  With a head count
+  // that is a multiple of 8 the workgroups of one head share id % 8, which
+  // keeps the head's K and V in the L2 of one XCD.
+  const int b = blockIdx.x;
+  int head, qt;
+  if ((a.H & 7) == 0)
+    {
+      const int j = b >> 3;
+      head = (b & 7) + 8 * (j / a.ntq);
+      qt = a.ntq - 1 - (j % a.ntq);
+    }
+  else
+    {
+      head = b / a.ntq;
+      qt = a.ntq - 1 - (b % a.ntq);
+    }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lq = lane & 31, hh = lane >> 5;
+  const int q0 = qt * kBQ;
+  const int qrow = q0 + wave * 32 + lq; // this lane's query
+  const int shift = a.L - a.S;          // key l is visible iff l <= qrow + shift
+  const int kmax = min (a.L, q0 + kBQ + shift);
+  const int ntile = (kmax + kBKey - 1) / kBKey;
+  const int wave_last = q0 + wave * 32 + 31 + shift; // last key any query of the wave sees
+  const uint16_t *kb = a.k + (size_t)head * a.kcs;
+  const uint16_t *vb = a.v + (size_t)head * a.vcs;
+
+  half8 qf[KT];
+  {
+    const uint16_t *qp = a.q + (size_t)head * a.qcs + (size_t)min (qrow, a.S - 1) * a.qhs + hh * 8;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+      qf[kt] = as_half8 (vkl::ldg4 (qp + kt * 16));
+  }
+
+  Tile<HD> tl;
+  // ---- pass 1: maximum and sum of exponentials per query ---------------------
+  float m = kNeg, sum = 0.f;
+  load_k<HD> (a, kb, 0, tl);
+  for (int t = 0; t < ntile; ++t)
+    {
+      __syncthreads ();
+      store_k<HD> (tl, Ks);
+      __syncthreads ();
+      if (t + 1 < ntile)
+        load_k<HD> (a, kb, t + 1, tl);
+      if (t * kBKey > wave_last)
+        continue;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+        {
+          const float16v acc = score_block<HD> (Ks, blk, qf, lane);
+          const int key0 = t * kBKey + 32 * blk + 4 * hh;
+          float sv[16];
+          float bm = kNeg;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            {
+              const int key = key0 + 8 * (r >> 2) + (r & 3);
+              const float s = vkl::h2f (vkl::f2h (acc[r] * a.scale));
+              sv[r] = key <= qrow + shift ? s : kNeg;
+              bm = fmaxf (bm, sv[r]);
+            }
+          const float mn = fmaxf (m, bm);
+          float add = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            add += sv[r] > 0.5f * kNeg ? fast_exp (sv[r] - mn) : 0.f;
+          sum = sum * fast_exp (m - mn) + add;
+          m = mn;
+        }
+    }
+  // the other half of the lanes holds the other keys of the same query
+  {
+    const float mo = __shfl_xor (m, 32, 64), so = __shfl_xor (sum, 32, 64);
+    const float M = fmaxf (m, mo);
+    sum = sum * fast_exp (m - M) + so * fast_exp (mo - M);
+    m = M;
+  }
+
+  // ---- pass 2: probabilities and P V -----------------------------------------
+  float16v oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      oacc[db][r] = 0.f;
+  load_k<HD> (a, kb, 0, tl);
+  load_v<HD> (a, vb, 0, tl);
+  for (int t = 0; t < ntile; ++t)
+    {
+      __syncthreads ();
+      store_k<HD> (tl, Ks);
+      store_v<HD> (tl, Vt);
+      __syncthreads ();
+      if (t + 1 < ntile)
+        {
+          load_k<HD> (a, kb, t + 1, tl);
+          load_v<HD> (a, vb, t + 1, tl);
+        }
+      if (t * kBKey > wave_last)
+        continue;
+      half8 pf[2][2];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+        {
+          const float16v acc = score_block<HD> (Ks, blk, qf, lane);
+          const int key0 = t * kBKey + 32 * blk + 4 * hh;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            {
+              const int key = key0 + 8 * (r >> 2) + (r & 3);
+              const float s = vkl::h2f (vkl::f2h (acc[r] * a.scale));
+              const float p = key <= qrow + shift ? fast_exp (s - m) / sum : 0.f;
+              pf[blk][r >> 3][r & 7] = (_Float16)p;
+            }
+        }
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        {
+          const uint16_t *vp = Vt + (size_t)(32 * db + lq) * LDV + 8 * hh;
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+              oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (
+                  *(const half8 *)(vp + 32 * blk + 16 * t2), pf[blk][t2], oacc[db], 0, 0, 0);
+        }
+    }
+
+  if (qrow >= a.S)
+    return;
+  uint16_t *op = a.out + (size_t)qrow * a.ors + (size_t)head * a.ohs;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      {
+        const int d = 32 * db + 8 * g + 4 * hh;
+        u32x2 w;
+        w.x = (uint32_t)vkl::f2h (oacc[db][4 * g]) | ((uint32_t)vkl::f2h (oacc[db][4 * g + 1]) << 16);
+        w.y = (uint32_t)vkl::f2h (oacc[db][4 * g + 2])
+              | ((uint32_t)vkl::f2h (oacc[db][4 * g + 3]) << 16);
+        *(VKL_GLOBAL u32x2 *)(op + d) = w;
+      }
+}
+} // namespace
+
+extern "C" int
+vkl_attn_prefill_causal_f16 (const void *q, const void *k, const void *v,
+                             int H, int S, int L, int hd, size_t qcs,
+                             size_t qhs, size_t kcs, size_t khs, size_t vcs,
+                             size_t vhs, float scale, void *out, size_t ors,
+                             size_t ohs, void *stream)
+{
+  VKL_CHECK_ARG (q && k && v && out);
+  VKL_CHECK_ARG (H > 0 && S > 0 && L >= S);
+  VKL_CHECK_ARG (hd == 64 || hd == 128);
+  // 16-byte vector loads, 8-byte stores
+  VKL_CHECK_ARG (((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0
+                 && ((uintptr_t)out % 8) == 0);
+  VKL_CHECK_ARG ((qcs % 8) == 0 && (qhs % 8) == 0 && (kcs % 8) == 0 && (khs % 8) == 0
+                 && (vcs % 8) == 0 && (vhs % 8) == 0 && (ors % 4) == 0 && (ohs % 4) == 0);
+  AttnArgs a;
+  a.q = (const uint16_t *)q, a.k = (const uint16_t *)k, a.v = (const uint16_t *)v;
+  a.out = (uint16_t *)out;
+  a.H = H, a.S = S, a.L = L, a.ntq = (S + kBQ - 1) / kBQ;
+  a.qcs = qcs, a.qhs = qhs, a.kcs = kcs, a.khs = khs, a.vcs = vcs, a.vhs = vhs;
+  a.ors = ors, a.ohs = ohs, a.scale = scale;
+  const dim3 grid ((unsigned)(a.ntq * H));
+  if (hd == 128)
+    attn_prefill_kernel<128><<<grid, dim3 (kThreads), 0, (hipStream_t)stream>>> (a);
+  else
+    attn_prefill_kernel<64><<<grid, dim3 (kThreads), 0, (hipStream_t)stream>>> (a);
+  return vkl_launch_status ();
+}

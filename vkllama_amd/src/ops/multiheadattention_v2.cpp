@@ -225,6 +225,34 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
           = vcache_.view (vcache_.channels (), read_len, vcache_.width ());
     }
 
+  // scores, masked softmax and P V in one launch, written as [seqlen,
+  // heads*dim]: same rounding points as the three operators below, without
+  // the [heads, seqlen, read_len] tensors in memory
+  attn_fused_last_ = false;
+  if (dtype_ == FP16 && (dim_ == 64 || dim_ == 128) && roped_q->dtype () == FP16
+      && roped_k->dtype () == FP16 && transposed_v->dtype () == FP16)
+    {
+      const size_t Sq = roped_q->height (), Lk = roped_k->height ();
+      if (!(attn_out_.channels () == 1 && attn_out_.height () == Sq
+            && attn_out_.width () == heads * (size_t)dim_))
+        {
+          attn_out_ = Tensor (1, Sq, heads * dim_, dev_, FP16, false);
+          VKLLAMA_STATUS_OK (attn_out_.create ());
+        }
+      attn_timer_.start (dev_);
+      const int err = vkl_attn_prefill_causal_f16 (
+          roped_q->data (), roped_k->data (), transposed_v->data (),
+          (int)heads, (int)Sq, (int)Lk, dim_, roped_q->cs () / 2,
+          roped_q->hs () / 2, roped_k->cs () / 2, roped_k->hs () / 2,
+          transposed_v->cs () / 2, transposed_v->hs () / 2,
+          1.0f / std::sqrt ((float)dim_), attn_out_.data (),
+          heads * (size_t)dim_, (size_t)dim_, dev_->stream ());
+      attn_timer_.stop (dev_);
+      VKLLAMA_STATUS_OK (launch_status ("attention", err));
+      attn_fused_last_ = true;
+      return (*matmul_o_) (attn_out_);
+    }
+
   // [heads, seqlen, read_len]
   auto attn_scores = (*matmul_qk_) (*roped_q, *roped_k);
   VKLLAMA_STATUS_OK (attn_scores);
@@ -253,9 +281,12 @@ MultiHeadAttentionV2::time () noexcept
                    transpose_v_->time () });
   if (use_kvcache_)
     t += std::max (update_kcache_op_->time (), update_vcache_op_->time ());
-  t += rope_q_->time () + matmul_qk_->time () + softmax_->time ()
-       + matmul_weighted_->time () + transpose_heads_->time ()
-       + matmul_o_->time ();
+  t += rope_q_->time () + matmul_o_->time ();
+  if (attn_fused_last_)
+    t += attn_timer_.micros ();
+  else
+    t += matmul_qk_->time () + softmax_->time () + matmul_weighted_->time ()
+         + transpose_heads_->time ();
   return t;
 }
 }

@@ -71,6 +71,9 @@ private:
   std::unique_ptr<UpdateKVCache> update_vcache_op_;
   std::unique_ptr<Slice> clip_output_op_;
   Tensor k_, q_, v_;
+  Tensor attn_out_;     // [1, S, heads*dim] of the one-launch attention
+  OpTimer attn_timer_;
+  bool attn_fused_last_ = false;
 };
 }
 #endif
