@@ -261,6 +261,9 @@ attn_prefill_kernel (const AttnArgs a)
   }
 
   // ---- pass 2: probabilities and P V -----------------------------------------
+  // exp(s - max) * (1 / sum) instead of a division per key: the two differ by
+  // one rounding of an fp32 value that is rounded to fp16 next
+  const float inv = 1.0f / sum;
   float16v oacc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -293,7 +296,7 @@ attn_prefill_kernel (const AttnArgs a)
             {
               const int key = key0 + 8 * (r >> 2) + (r & 3);
               const float s = vkl::h2f (vkl::f2h (acc[r] * a.scale));
-              const float p = key <= qrow + shift ? fast_exp (s - m) / sum : 0.f;
+              const float p = key <= qrow + shift ? fast_exp (s - m) * inv : 0.f;
               pf[blk][r >> 3][r & 7] = (_Float16)p;
             }
         }
