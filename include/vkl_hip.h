@@ -139,6 +139,19 @@ int vkl_kv_update_f16 (void *cache, const void *kv, int C, int HO, int H,
 /* src/ops/softmax.cpp:52-92, src/shaders/softmax_fp16.comp */
 int vkl_softmax_f16 (const void *x, int C, int H, int W, int seq_mask,
                      uint32_t offset, void *out, void *stream);
+/* src/ops/multiheadattention_v2.cpp:205-287 in one launch, on the [S, H*hd]
+ * outputs of the K/Q/V projections (row stride row_stride): the reshape and
+ * Transpose of K, Q, V become index arithmetic, Rope (rope_fp16.comp) rotates
+ * q rows [q_row0, q_row0 + q_rows) in place at positions q_pos0 + i and every
+ * k row s at position k_pos0 + s, and UpdateKVCache (update_kvcache_fp16.comp)
+ * writes the rotated k and v to rows (k_pos0 + s) % maxlen of [H, maxlen, hd]
+ * caches.  freqc / freqs: fp32 [table_rows, hd/2]. */
+int vkl_rope_kvwrite_f16 (void *q, const void *k, const void *v, int S, int H,
+                          int hd, size_t row_stride, int q_row0, int q_rows,
+                          uint32_t q_pos0, uint32_t k_pos0,
+                          const float *freqc, const float *freqs,
+                          int table_rows, void *kcache, void *vcache,
+                          int maxlen, void *stream);
 /* The attention core of src/ops/multiheadattention_v2.cpp:290-309 in one
  * launch for many query rows: matmul_b0_tb_fp16_v2.comp (scores = fp16(scale
  * q.k)), softmax_fp16.comp with seq_mask (key l is masked iff l > s + (L - S))

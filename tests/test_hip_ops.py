@@ -368,6 +368,35 @@ def test_rope_bit_exact(dev, rng, C, H, W, off):
     assert np.array_equal(f16(dx, x.shape).view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("S,H,hd,maxlen,off,clip,qpos", [
+    (16, 8, 64, 64, 0, False, 0), (5, 3, 128, 256, 100, False, 100), (7, 4, 128, 128, 121, True, 121),
+    (7, 4, 64, 128, 9, True, 15)])
+def test_rope_kvwrite_bit_exact(dev, rng, S, H, hd, maxlen, off, clip, qpos):
+    """RoPE of Q and K plus the cache write on [S, H*hd] projection outputs equals
+    Transpose -> Rope -> UpdateKVCache of the oracle bit for bit; with clip only
+    the last q row is rotated (at position qpos)."""
+    fc, fs = O.rope_tables(maxlen, hd)
+    q, k, v = (rng.standard_normal((S, H, hd)).astype(np.float16) for _ in range(3))
+    kc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    vc = rng.standard_normal((H, maxlen, hd)).astype(np.float16)
+    dq, dk, dv, dkc, dvc = (dev.upload(a) for a in (q, k, v, kc, vc))
+    dfc, dfs = dev.upload(fc), dev.upload(fs)
+    q_row0, q_rows = (S - 1, 1) if clip else (0, S)
+    capi.check(L().vkl_rope_kvwrite_f16(dq.ptr, dk.ptr, dv.ptr, S, H, hd, H * hd, q_row0, q_rows, qpos, off,
+                                        dfc.ptr, dfs.ptr, maxlen, dkc.ptr, dvc.ptr, maxlen, dev.stream))
+    kt, vt, qt = O.transpose102(k), O.transpose102(v), O.transpose102(q)       # [H, S, hd]
+    want_k = O.update_kvcache(kc, O.rope(kt, fc, fs, off), off)
+    want_v = O.update_kvcache(vc, vt, off)
+    assert np.array_equal(f16(dkc, kc.shape).view(np.uint16), want_k.view(np.uint16))
+    assert np.array_equal(f16(dvc, vc.shape).view(np.uint16), want_v.view(np.uint16))
+    got_q = f16(dq, q.shape)
+    want_q = q.copy()
+    rot = O.rope(np.ascontiguousarray(qt[:, q_row0:q_row0 + q_rows]), fc, fs, qpos)  # [H, rows, hd]
+    want_q[q_row0:q_row0 + q_rows] = rot.transpose(1, 0, 2)
+    assert np.array_equal(got_q.view(np.uint16), want_q.view(np.uint16))
+    assert np.array_equal(f16(dk, k.shape), k) and np.array_equal(f16(dv, v.shape), v)
+
+
 @pytest.mark.parametrize("off", [0, 1022, 500])
 def test_kv_update_bit_exact(dev, rng, off):
     C, HO, H, W = 8, 1024, 5, 64

@@ -27,6 +27,9 @@
 // with its keys permuted to that same order (slot 16t + 8h + j holds key
 // 16t + 8*(j/4) + 4h + j%4 of the block), so the A operand of the second
 // product is one 16-byte LDS read.
+//
+// A second, small kernel in this file prepares the inputs of the first from
+// the projection outputs: RoPE of Q (in place) and K, and the K/V cache write.
 #include "../../include/vkl_hip.h"
 #include "vkl_common.h"
 
@@ -329,7 +332,103 @@ attn_prefill_kernel (const AttnArgs a)
         *(VKL_GLOBAL u32x2 *)(op + d) = w;
       }
 }
+// ---------------------------------------------------------------------------
+// RoPE of Q and K and the K/V cache write, straight from the [S, H*hd]
+// outputs of the projections: one thread per 8 consecutive elements of a
+// (row, head).  Q is rotated in place (the attention kernel reads it with a
+// row stride of H*hd), the rotated K and V go to cache rows (k_pos0 + s) %
+// maxlen of their head.  Arithmetic of one pair as in the RoPE operator:
+// (a, b) -> (fp16(a c - b s), fp16(a s + b c)) with fp32 tables.
+// ---------------------------------------------------------------------------
+struct RopeKvArgs
+{
+  uint16_t *q;
+  const uint16_t *k, *v;
+  uint16_t *kcache, *vcache;
+  const float *fc, *fs;
+  int S, H, hd, maxlen;
+  int q_row0, q_rows;       // rows of q that are rotated, and their positions
+  uint32_t q_pos0, k_pos0;  // q row q_row0 + i is at q_pos0 + i; k row s at k_pos0 + s
+  size_t rs;                // row stride of q, k, v (elements)
+};
+
+__device__ __forceinline__ uint4
+rotate8 (const uint4 x, const float *fc, const float *fs)
+{
+  const uint4 c4 = vkl::ldg4 (fc), s4 = vkl::ldg4 (fs);
+  const float c[4] = { __uint_as_float (c4.x), __uint_as_float (c4.y), __uint_as_float (c4.z),
+                       __uint_as_float (c4.w) };
+  const float sn[4] = { __uint_as_float (s4.x), __uint_as_float (s4.y), __uint_as_float (s4.z),
+                        __uint_as_float (s4.w) };
+  const uint32_t w[4] = { x.x, x.y, x.z, x.w };
+  uint32_t o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const float a = vkl::h2f ((uint16_t)(w[j] & 0xffff)), b = vkl::h2f ((uint16_t)(w[j] >> 16));
+      const float r0 = a * c[j] - b * sn[j];
+      const float r1 = a * sn[j] + b * c[j];
+      o[j] = (uint32_t)vkl::f2h (r0) | ((uint32_t)vkl::f2h (r1) << 16);
+    }
+  return make_uint4 (o[0], o[1], o[2], o[3]);
+}
+
+__global__ __launch_bounds__ (256) void
+rope_kvwrite_kernel (const RopeKvArgs a, size_t total)
+{
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= total)
+    return;
+  const int cpr = a.hd / 8;
+  const int c = (int)(t % cpr);
+  const int h = (int)((t / cpr) % a.H);
+  const int s = (int)(t / ((size_t)cpr * a.H));
+  const size_t src = (size_t)s * a.rs + (size_t)h * a.hd + c * 8;
+  const int half = a.hd / 2;
+  const uint32_t kpos = a.k_pos0 + (uint32_t)s;
+  const size_t dst = ((size_t)h * a.maxlen + kpos % (uint32_t)a.maxlen) * a.hd + c * 8;
+  const uint4 kr = rotate8 (vkl::ldg4 (a.k + src), a.fc + (size_t)kpos * half + c * 4,
+                            a.fs + (size_t)kpos * half + c * 4);
+  *(uint4 *)(a.kcache + dst) = kr;
+  *(uint4 *)(a.vcache + dst) = vkl::ldg4 (a.v + src);
+  if (s >= a.q_row0 && s < a.q_row0 + a.q_rows)
+    {
+      const uint32_t qpos = a.q_pos0 + (uint32_t)(s - a.q_row0);
+      *(uint4 *)(a.q + src) = rotate8 (vkl::ldg4 (a.q + src), a.fc + (size_t)qpos * half + c * 4,
+                                       a.fs + (size_t)qpos * half + c * 4);
+    }
+}
 } // namespace
+
+extern "C" int
+vkl_rope_kvwrite_f16 (void *q, const void *k, const void *v, int S, int H,
+                      int hd, size_t row_stride, int q_row0, int q_rows,
+                      uint32_t q_pos0, uint32_t k_pos0, const float *freqc,
+                      const float *freqs, int table_rows, void *kcache,
+                      void *vcache, int maxlen, void *stream)
+{
+  VKL_CHECK_ARG (q && k && v && freqc && freqs && kcache && vcache);
+  VKL_CHECK_ARG (S > 0 && H > 0 && hd > 0 && (hd % 8) == 0 && maxlen > 0 && S <= maxlen);
+  VKL_CHECK_ARG (q_row0 >= 0 && q_rows >= 0 && q_row0 + q_rows <= S);
+  // every position must have a row in the cos / sin tables
+  VKL_CHECK_ARG ((size_t)k_pos0 + S <= (size_t)table_rows
+                 && (size_t)q_pos0 + q_rows <= (size_t)table_rows);
+  VKL_CHECK_ARG ((row_stride % 8) == 0 && row_stride >= (size_t)H * hd);
+  VKL_CHECK_ARG (((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0
+                 && ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0
+                 && ((uintptr_t)freqc % 16) == 0 && ((uintptr_t)freqs % 16) == 0);
+  RopeKvArgs a;
+  a.q = (uint16_t *)q, a.k = (const uint16_t *)k, a.v = (const uint16_t *)v;
+  a.kcache = (uint16_t *)kcache, a.vcache = (uint16_t *)vcache;
+  a.fc = freqc, a.fs = freqs;
+  a.S = S, a.H = H, a.hd = hd, a.maxlen = maxlen;
+  a.q_row0 = q_row0, a.q_rows = q_rows, a.q_pos0 = q_pos0, a.k_pos0 = k_pos0;
+  a.rs = row_stride;
+  const size_t total = (size_t)S * H * (hd / 8);
+  rope_kvwrite_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, (hipStream_t)stream>>> (
+      a, total);
+  return vkl_launch_status ();
+}
 
 extern "C" int
 vkl_attn_prefill_causal_f16 (const void *q, const void *k, const void *v,

@@ -180,6 +180,47 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
       k = *rk, q = *rq, v = *rv;
     }
 
+  // With a cache and fp16 activations the rest of the operator is two
+  // launches on the projection outputs as they lie ([S, heads*dim]): RoPE of
+  // Q and K + cache write, then scores / masked softmax / P V.  Reshapes,
+  // transposes, the clip of Q to its last row and the cache views of the
+  // operator-by-operator form below become index arithmetic; the values and
+  // their fp16 rounding points are the same.
+  attn_fused_last_ = false;
+  if (use_kvcache_ && dtype_ == FP16 && (dim_ == 64 || dim_ == 128)
+      && k.dtype () == FP16 && q.dtype () == FP16 && v.dtype () == FP16)
+    {
+      const int q_row0 = clip_output_ ? (int)S - 1 : 0;
+      const int q_rows = clip_output_ ? 1 : (int)S;
+      const size_t q_pos0
+          = clip_output_ && !rope_quirk_ ? offset + S - 1 : offset;
+      if (!(attn_out_.channels () == 1 && attn_out_.height () == (size_t)q_rows
+            && attn_out_.width () == N))
+        {
+          attn_out_ = Tensor (1, q_rows, N, dev_, FP16, false);
+          VKLLAMA_STATUS_OK (attn_out_.create ());
+        }
+      attn_timer_.start (dev_);
+      int err = vkl_rope_kvwrite_f16 (
+          q.data (), k.data (), v.data (), (int)S, (int)heads, dim_, N, q_row0,
+          q_rows, (uint32_t)q_pos0, (uint32_t)offset,
+          (const float *)rope_q_->freqc ().data (),
+          (const float *)rope_q_->freqs ().data (), maxlen_, kcache_.data (),
+          vcache_.data (), maxlen_, dev_->stream ());
+      if (err == 0)
+        err = vkl_attn_prefill_causal_f16 (
+            (const uint16_t *)q.data () + (size_t)q_row0 * N, kcache_.data (),
+            vcache_.data (), (int)heads, q_rows, (int)(offset + S), dim_,
+            (size_t)dim_, N, (size_t)maxlen_ * dim_, (size_t)dim_,
+            (size_t)maxlen_ * dim_, (size_t)dim_,
+            1.0f / std::sqrt ((float)dim_), attn_out_.data (), N,
+            (size_t)dim_, dev_->stream ());
+      attn_timer_.stop (dev_);
+      VKLLAMA_STATUS_OK (launch_status ("attention", err));
+      attn_fused_last_ = true;
+      return (*matmul_o_) (attn_out_);
+    }
+
   // [seqlen, heads, dim]
   VKLLAMA_STATUS_OK (k.reshape (S, heads, dim_));
   VKLLAMA_STATUS_OK (q.reshape (S, heads, dim_));
@@ -228,7 +269,6 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
   // scores, masked softmax and P V in one launch, written as [seqlen,
   // heads*dim]: same rounding points as the three operators below, without
   // the [heads, seqlen, read_len] tensors in memory
-  attn_fused_last_ = false;
   if (dtype_ == FP16 && (dim_ == 64 || dim_ == 128) && roped_q->dtype () == FP16
       && roped_k->dtype () == FP16 && transposed_v->dtype () == FP16)
     {
@@ -277,6 +317,8 @@ uint64_t
 MultiHeadAttentionV2::time () noexcept
 {
   uint64_t t = timer_.micros ();
+  if (attn_fused_last_ && use_kvcache_)
+    return t + attn_timer_.micros () + matmul_o_->time ();
   t += std::max ({ transpose_k_->time (), transpose_q_->time (),
                    transpose_v_->time () });
   if (use_kvcache_)
