@@ -90,6 +90,20 @@ void vkl_synth_normal_f16 (uint64_t seed, size_t n, float std,
 void vkl_synth_normal_q8_0 (uint64_t seed, size_t rows, size_t K, float std,
                             uint8_t *out_h);
 
+/* ---- host samplers (models/samplers.h:8-43) ------------------------------
+ * kind 0: TopkSampler (param = k), kind 1: TopPSampler (param = p).  seeded:
+ * 0 seeds from std::random_device as the reference does, else from `seed`. */
+typedef struct vkl_sampler vkl_sampler;
+int vkl_sampler_create (int kind, float param, int seeded, uint64_t seed,
+                        vkl_sampler **out);
+void vkl_sampler_destroy (vkl_sampler *s);
+/* a token id drawn for one row of n logits (host memory); -1 if n == 0 */
+int vkl_sampler_sample (vkl_sampler *s, const float *logits_h, size_t n);
+/* candidates of the last draw, most likely first: up to cap (id, probability)
+ * pairs are written; returns how many candidates there were */
+size_t vkl_sampler_candidates (const vkl_sampler *s, int32_t *ids_h,
+                               float *probs_h, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,12 +1,16 @@
-// Command-line greedy generation from a GGUF file with the drop-in classes:
-// the flow of the reference's app/llama2_infer.cpp (open the file, collect
-// keys and tensors, Model::init, prompt pass, then one token per step with a
-// top-1 pick on the host) without the sentencepiece tokenizer, which is not
-// available to C++ in this image: the prompt is given as token ids.
+// Command-line generation from a GGUF file with the drop-in classes: the flow
+// of the reference's app/llama2_infer.cpp (open the file, collect keys and
+// tensors, Model::init, prompt pass, then one token per step picked on the
+// host by a TopkSampler(1), line 138 there) without the sentencepiece
+// tokenizer, which is not available to C++ in this image: the prompt is given
+// as token ids.
 //
-//   llama2_infer MODEL.gguf N_TOKENS ID [ID ...]
+//   llama2_infer [--topk K | --topp P] [--seed S] MODEL.gguf N_TOKENS ID [ID ...]
 #include "models/gguflib.h"
 #include "models/llama2.h"
+#include "models/samplers.h"
+#include <cstring>
+#include <memory>
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
@@ -18,11 +22,34 @@
 int
 main (int argc, char **argv)
 {
-  if (argc < 4)
+  size_t topk = 1;
+  float topp = -1.f;
+  bool seeded = false;
+  uint64_t seed = 0;
+  while (argc > 2 && argv[1][0] == '-' && argv[1][1] == '-')
     {
-      fprintf (stderr, "usage: %s <model.gguf> <predict tokens> <prompt id> [id ...]\n", argv[0]);
+      if (!strcmp (argv[1], "--topk"))
+        topk = (size_t)strtoul (argv[2], nullptr, 10);
+      else if (!strcmp (argv[1], "--topp"))
+        topp = strtof (argv[2], nullptr);
+      else if (!strcmp (argv[1], "--seed"))
+        seeded = true, seed = strtoull (argv[2], nullptr, 10);
+      else
+        break;
+      argv += 2, argc -= 2;
+    }
+  if (argc < 4 || topk < 1)
+    {
+      fprintf (stderr,
+               "usage: llama2_infer [--topk K | --topp P] [--seed S] <model.gguf> <predict tokens> "
+               "<prompt id> [id ...]\n");
       return 2;
     }
+  std::unique_ptr<Sampler> sampler;
+  if (topp >= 0.f)
+    sampler.reset (seeded ? new TopPSampler (topp, seed) : new TopPSampler (topp));
+  else
+    sampler.reset (seeded ? new TopkSampler (topk, seed) : new TopkSampler (topk));
   gguf_ctx *gguf = gguf_open (argv[1]);
   if (!gguf)
     {
@@ -72,10 +99,11 @@ main (int argc, char **argv)
         }
       if (i == 0)
         t1 = clock::now ();
-      // top-1 over the last row of logits; the lowest index wins ties
+      // the sampler sees the last row of logits (top-1 by default; the
+      // lowest index wins ties)
       const size_t V = model.vocab_size ();
       const float *row = logits->data () + (logits->size () - V);
-      const uint32_t next = (uint32_t)(std::max_element (row, row + V) - row);
+      const uint32_t next = (uint32_t)sampler->sample (row, V);
       printf ("%u%c", next, i + 1 == predict ? '\n' : ' ');
       offset += toks.size ();
       toks = { next };

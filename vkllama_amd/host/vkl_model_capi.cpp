@@ -333,3 +333,61 @@ vkl_synth_normal_q8_0 (uint64_t seed, size_t rows, size_t K, float std,
       }
   }
 }
+
+// ---- host samplers -----------------------------------------------------------
+#include "models/samplers.h"
+#include <memory>
+
+struct vkl_sampler
+{
+  std::unique_ptr<Sampler> impl;
+};
+
+extern "C" int
+vkl_sampler_create (int kind, float param, int seeded, uint64_t seed,
+                    vkl_sampler **out)
+{
+  if (!out || (kind != 0 && kind != 1))
+    return 1;
+  if (kind == 0 && !(param >= 1.0f))
+    return 1;
+  auto *s = new vkl_sampler;
+  if (kind == 0)
+    s->impl.reset (seeded ? new TopkSampler ((size_t)param, seed)
+                          : new TopkSampler ((size_t)param));
+  else
+    s->impl.reset (seeded ? new TopPSampler (param, seed) : new TopPSampler (param));
+  *out = s;
+  return 0;
+}
+
+extern "C" void
+vkl_sampler_destroy (vkl_sampler *s)
+{
+  delete s;
+}
+
+extern "C" int
+vkl_sampler_sample (vkl_sampler *s, const float *logits, size_t n)
+{
+  if (!s || !logits)
+    return -1;
+  return s->impl->sample (logits, n);
+}
+
+extern "C" size_t
+vkl_sampler_candidates (const vkl_sampler *s, int32_t *ids, float *probs,
+                        size_t cap)
+{
+  if (!s)
+    return 0;
+  const auto &c = s->impl->candidates ();
+  for (size_t i = 0; i < c.size () && i < cap; ++i)
+    {
+      if (ids)
+        ids[i] = c[i].second;
+      if (probs)
+        probs[i] = c[i].first;
+    }
+  return c.size ();
+}

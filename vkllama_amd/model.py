@@ -38,6 +38,10 @@ SIGNATURES = {
     "vkl_synth_normal_f32": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_f16": (None, [u64, sz, C.c_float, vp]),
     "vkl_synth_normal_q8_0": (None, [u64, sz, sz, C.c_float, vp]),
+    "vkl_sampler_create": (i32, [i32, C.c_float, i32, u64, C.POINTER(vp)]),
+    "vkl_sampler_destroy": (None, [vp]),
+    "vkl_sampler_sample": (i32, [vp, vp, sz]),
+    "vkl_sampler_candidates": (sz, [vp, vp, vp, sz]),
 }
 
 _lib = None
@@ -91,6 +95,42 @@ def synth_weights(cfg, seed=1234, std=0.02, norm_value=1.0):
             out = out.view(np.float16)
         w[name] = out
     return w
+
+
+class Sampler:
+    """Host sampler over a row of logits (TopkSampler / TopPSampler of the
+    reference's models/samplers.h).  kind "topk" with k, or "topp" with p;
+    seed=None seeds from the system's random device as the reference does."""
+
+    def __init__(self, kind, param, seed=None):
+        h = vp()
+        err = lib().vkl_sampler_create({"topk": 0, "topp": 1}[kind], float(param), int(seed is not None),
+                                       int(seed or 0), C.byref(h))
+        if err:
+            raise ValueError("bad sampler parameters: %s %r" % (kind, param))
+        self._h = h
+
+    def sample(self, logits):
+        logits = np.ascontiguousarray(logits, np.float32).reshape(-1)
+        return int(lib().vkl_sampler_sample(self._h, logits.ctypes.data, logits.size))
+
+    def candidates(self):
+        """(ids, probabilities) of the last draw's candidate set, most likely first"""
+        n = lib().vkl_sampler_candidates(self._h, None, None, 0)
+        ids, probs = np.empty(n, np.int32), np.empty(n, np.float32)
+        lib().vkl_sampler_candidates(self._h, ids.ctypes.data, probs.ctypes.data, n)
+        return ids, probs
+
+    def close(self):
+        if self._h:
+            lib().vkl_sampler_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Llama2:
