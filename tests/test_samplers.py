@@ -70,7 +70,7 @@ def test_topp_candidates_and_probabilities(logits, p):
     n_hi = max(int(np.sum(mass_before < p + 1e-4)), 1)
     n = ids.size
     assert n_lo <= n <= n_hi and np.array_equal(ids, order[:n])
-    assert np.allclose(probs, softmax32(logits[order[:n]]), rtol=1e-5, atol=1e-9)
+    assert np.allclose(probs, softmax32(logits[order[:n]]), rtol=1e-4, atol=1e-9)  # fp32 sum over up to 32000 terms
     assert tok in ids
 
 
