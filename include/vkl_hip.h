@@ -185,6 +185,23 @@ int vkl_argop_f16 (const void *x, int rows, int W, int op, uint32_t *out,
 /* src/ops/slice.cpp:30-77, src/shaders/slice_fp16.comp */
 int vkl_slice_f16 (const void *x, int C, int H, int W, int c0, int h0, int w0,
                    int CE, int HE, int WE, void *out, void *stream);
+/* src/ops/concat.cpp:68-188, src/shaders/concat_fp16.comp: one input of a
+ * Concat copied into the output: out[c*ocs + y*ohs + x + out_offset] =
+ * x[c*xcs + y*xhs + x] (element strides; the operator gives each input the
+ * offset of its position along the concatenation axis). */
+int vkl_concat_part_f16 (const void *x, int C, int H, int W, size_t xcs,
+                         size_t xhs, void *out, size_t ocs, size_t ohs,
+                         size_t out_offset, void *stream);
+/* src/ops/read_kvcache_op.cpp:31-70, src/shaders/read_kvcache_fp16.comp:
+ * out[c, y, :] = cache[c, (y + offset) % H, :] for y < len; cache [C,H,W]. */
+int vkl_read_kvcache_f16 (const void *cache, int C, int H, int W,
+                          uint32_t offset, uint32_t len, void *out,
+                          void *stream);
+/* src/ops/reduce.h:17-120, src/shaders/reduce_fp16.comp: over the last axis of
+ * [C,H,W], op 0 sum, 1 max, 2 min, 3 mean (sum * (1/W)); fp32 accumulation,
+ * out [C,H] fp16. */
+int vkl_reduce_f16 (const void *x, int C, int H, int W, int op, void *out,
+                    void *stream);
 /* src/ops/transpose.cpp:36-80 type 0, transpose_type0_fp16.comp:
  * [C,H,W] -> [H,C,W] */
 int vkl_transpose102_f16 (const void *x, int C, int H, int W, void *out,

@@ -24,6 +24,9 @@
 #include "src/ops/rms_norm.h"
 #include "src/ops/rope.h"
 #include "src/ops/slice.h"
+#include "src/ops/concat.h"
+#include "src/ops/reduce.h"
+#include "src/ops/read_kvcache_op.h"
 #include "src/ops/softmax.h"
 #include "src/ops/transpose.h"
 #include "src/ops/update_kv_cache.h"
@@ -745,6 +748,100 @@ test_attention (Ctx &c, int S, bool clip)
 }
 
 void
+test_concat_reduce_readkv (Ctx &c)
+{
+  g_test = "Concat/Reduce/ReadKVCache";
+  // tests/test_concat.cpp of the reference joins two tensors along each axis
+  for (int axis = 0; axis < 3; ++axis)
+    {
+      const int C = 3, H = 5, W = 16;
+      int d1[3] = { C, H, W };
+      d1[axis] += 2 + axis;
+      vec a = randn ((size_t)C * H * W), b = randn ((size_t)d1[0] * d1[1] * d1[2]);
+      auto ta = half_tensor (c, a, C, H, W);
+      auto tb = half_tensor (c, b, d1[0], d1[1], d1[2]);
+      CHECK_OK (ta.status ());
+      CHECK_OK (tb.status ());
+      Concat cat (&c.dev, &c.cmd, 2, axis, FP16);
+      CHECK_OK (cat.init ());
+      auto out = cat ({ *ta, *tb });
+      CHECK_OK (out.status ());
+      const int OC = axis == 0 ? C + d1[0] : C, OH = axis == 1 ? H + d1[1] : H,
+                OW = axis == 2 ? W + d1[2] : W;
+      CHECK (out->channels () == (size_t)OC && out->height () == (size_t)OH
+             && out->width () == (size_t)OW);
+      auto g = fetch_half (c, *out);
+      CHECK_OK (g.status ());
+      for (int ch = 0; ch < OC; ++ch)
+        for (int h = 0; h < OH; ++h)
+          for (int w = 0; w < OW; ++w)
+            {
+              const bool in_a = ch < C && h < H && w < W;
+              const float want
+                  = in_a ? a[((size_t)ch * H + h) * W + w]
+                         : b[((size_t)(ch - (axis == 0 ? C : 0)) * d1[1] + (h - (axis == 1 ? H : 0)))
+                                 * d1[2]
+                             + (w - (axis == 2 ? W : 0))];
+              CHECK ((*g)[((size_t)ch * OH + h) * OW + w] == want);
+            }
+      Concat bad (&c.dev, &c.cmd, 3, axis, FP16);
+      CHECK_OK (bad.init ());
+      CHECK (bad ({ *ta, *tb }).status ().code () == absl::StatusCode::kInvalidArgument);
+    }
+  {
+    // tests/test_reduce.cpp: sum / max / min / mean over the last axis, 1e-2
+    const int C = 3, H = 7, W = 300;
+    vec x = randn ((size_t)C * H * W);
+    auto tx = half_tensor (c, x, C, H, W);
+    CHECK_OK (tx.status ());
+    for (int op = 0; op < 4; ++op)
+      {
+        Reduce red (&c.dev, &c.cmd, op, FP16);
+        CHECK_OK (red.init ());
+        auto out = red (*tx);
+        CHECK_OK (out.status ());
+        CHECK (out->channels () == (size_t)C && out->height () == (size_t)H && out->width () == 1);
+        auto g = fetch_half (c, *out);
+        CHECK_OK (g.status ());
+        for (int r = 0; r < C * H; ++r)
+          {
+            double v = op == 0 || op == 3 ? 0.0 : x[(size_t)r * W];
+            for (int w = 0; w < W; ++w)
+              {
+                const double e = x[(size_t)r * W + w];
+                v = op == 0 || op == 3 ? v + e : (op == 1 ? std::max (v, e) : std::min (v, e));
+              }
+            if (op == 3)
+              v /= W;
+            if (op == 1 || op == 2)
+              CHECK ((*g)[r] == (float)v);
+            else
+              CHECK (fabs ((*g)[r] - v) <= 1e-2 * std::max (1.0, fabs (v)));
+          }
+      }
+  }
+  {
+    // ring read: rows (offset + y) % H
+    const int C = 4, H = 16, W = 8;
+    vec x = randn ((size_t)C * H * W);
+    auto tx = half_tensor (c, x, C, H, W);
+    CHECK_OK (tx.status ());
+    ReadKVCache rd (&c.dev, &c.cmd);
+    CHECK_OK (rd.init ());
+    auto out = rd (*tx, 13, 6);
+    CHECK_OK (out.status ());
+    CHECK (out->channels () == (size_t)C && out->height () == 6 && out->width () == (size_t)W);
+    auto g = fetch_half (c, *out);
+    CHECK_OK (g.status ());
+    for (int ch = 0; ch < C; ++ch)
+      for (int y = 0; y < 6; ++y)
+        for (int w = 0; w < W; ++w)
+          CHECK ((*g)[((size_t)ch * 6 + y) * W + w] == x[((size_t)ch * H + (y + 13) % H) * W + w]);
+    CHECK (rd (*tx, 0, 17).status ().code () == absl::StatusCode::kOutOfRange);
+  }
+}
+
+void
 run_gpu ()
 {
   Ctx c;
@@ -764,6 +861,7 @@ run_gpu ()
   test_embedding (c);
   test_rope_softmax_kv (c);
   test_slice_transpose (c);
+  test_concat_reduce_readkv (c);
   test_feed_forward (c, 1);
   test_feed_forward (c, 20);
   test_attention (c, 6, false);

@@ -475,3 +475,51 @@ def test_invalid_arguments_are_rejected_before_launch(dev):
     assert L().vkl_matmul_q8_0(buf.ptr, buf.ptr, 1, 4, 32, 16, 4, 1.0, 0.0, 0, None, buf.ptr, None,
                                dev.stream) == 1                                              # row stride < K
     dev.sync()
+
+
+# ------------------------------------------------- Concat / ReadKVCache / Reduce
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_concat_parts_bit_exact(dev, rng, axis):
+    """tests/test_concat.cpp of the reference: inputs joined along one axis."""
+    shapes = [[3, 5, 16], [3, 5, 16], [3, 5, 16]]
+    shapes[1][axis] += 4
+    shapes[2][axis] = 1
+    xs = [rng.standard_normal(sh).astype(np.float16) for sh in shapes]
+    want = np.concatenate(xs, axis=axis)
+    OC, OH, OW = want.shape
+    out = dev.alloc(want.nbytes)
+    off = 0
+    for x in xs:
+        Cc, H, W = x.shape
+        capi.check(L().vkl_concat_part_f16(dev.upload(x).ptr, Cc, H, W, H * W, W, out.ptr, OH * OW, OW, off, dev.stream))
+        off += (Cc * OH * OW, H * OW, W)[axis]
+    assert np.array_equal(f16(out, want.shape).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("off,n", [(0, 16), (13, 6), (31, 16), (5, 1)])
+def test_read_kvcache_bit_exact(dev, rng, off, n):
+    C_, H, W = 4, 16, 64
+    cache = rng.standard_normal((C_, H, W)).astype(np.float16)
+    out = dev.alloc(C_ * n * W * 2)
+    capi.check(L().vkl_read_kvcache_f16(dev.upload(cache).ptr, C_, H, W, off, n, out.ptr, dev.stream))
+    want = cache[:, (np.arange(n) + off) % H]
+    assert np.array_equal(f16(out, want.shape).view(np.uint16), want.view(np.uint16))
+    assert L().vkl_read_kvcache_f16(dev.upload(cache).ptr, C_, H, W, 0, H + 1, out.ptr, dev.stream) != 0
+
+
+@pytest.mark.parametrize("op", [0, 1, 2, 3])
+@pytest.mark.parametrize("shape", [(3, 7, 300), (1, 1, 5), (2, 64, 4096)])
+def test_reduce_last_axis(dev, rng, op, shape):
+    """tests/test_reduce.cpp of the reference (tolerance 1e-2); max and min are exact."""
+    x = rng.standard_normal(shape).astype(np.float16)
+    out = dev.alloc(shape[0] * shape[1] * 2)
+    capi.check(L().vkl_reduce_f16(dev.upload(x).ptr, *shape, op, out.ptr, dev.stream))
+    got = f16(out, shape[:2]).astype(np.float64)
+    x64 = x.astype(np.float64)
+    want = (x64.sum(-1), x64.max(-1), x64.min(-1), x64.mean(-1))[op]
+    if op in (1, 2):
+        assert np.array_equal(got, want)
+    else:
+        scale = np.abs(x64).sum(-1) / (shape[2] if op == 3 else 1)
+        assert np.all(np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 0.1 * scale) + 1e-3)
+

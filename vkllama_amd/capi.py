@@ -58,6 +58,9 @@ SIGNATURES = {
     "vkl_kqv_q8_0": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp]),
     "vkl_ffn_upgate_q8_0": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "vkl_rope_kvwrite_f16": (i32, [vp, vp, vp, i32, i32, i32, sz, i32, i32, u32, u32, vp, vp, i32, vp, vp, i32, vp]),
+    "vkl_concat_part_f16": (i32, [vp, i32, i32, i32, sz, sz, vp, sz, sz, sz, vp]),
+    "vkl_read_kvcache_f16": (i32, [vp, i32, i32, i32, u32, u32, vp, vp]),
+    "vkl_reduce_f16": (i32, [vp, i32, i32, i32, i32, vp, vp]),
     "vkl_attn_prefill_causal_f16": (i32, [vp, vp, vp, i32, i32, i32, i32, sz, sz, sz, sz, sz, sz, f32, vp, sz, sz, vp]),
     "vkl_matmul_f16_tb": (i32, [vp, vp, i32, i32, i32, i32, sz, sz, sz, sz, sz, sz, f32, f32, i32, vp, vp, vp, vp]),
     "vkl_matmul_f16_nn": (i32, [vp, vp, i32, i32, i32, i32, sz, sz, sz, sz, sz, sz, f32, f32, i32, vp, vp]),

@@ -244,6 +244,51 @@ transpose102_kernel (const uint16_t *__restrict__ x, int C, int H, int W,
   out[((size_t)h * C + c) * W + xw] = x[t];
 }
 
+// ---- strided copy of a [C, H, W] box (Concat, ReadKVCache) --------------------
+// out[c*dcs + y*dhs + x + doff] = in[c*scs + ((y + h0) % HM)*shs + x]
+__global__ void
+copy_box_kernel (const uint16_t *__restrict__ in, int H, int W, size_t scs,
+                 size_t shs, int h0, int HM, uint16_t *__restrict__ out,
+                 size_t dcs, size_t dhs, size_t doff, size_t total)
+{
+  const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= total)
+    return;
+  const int xw = (int)(t % W);
+  const size_t r = t / W;
+  const int y = (int)(r % H);
+  const size_t c = r / H;
+  const size_t ys = (size_t)(((uint32_t)y + (uint32_t)h0) % (uint32_t)HM);
+  out[c * dcs + (size_t)y * dhs + xw + doff] = in[c * scs + ys * shs + xw];
+}
+
+// ---- Reduce over the last axis: one wave per row ------------------------------
+// op 0 sum, 1 max, 2 min; out = fp16(r * scale)
+__global__ __launch_bounds__ (256) void
+reduce_rows_kernel (const uint16_t *__restrict__ x, int W, int op, float scale,
+                    uint16_t *__restrict__ out, size_t rows)
+{
+  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows)
+    return;
+  const int lane = threadIdx.x & 63;
+  const uint16_t *r = x + row * (size_t)W;
+  float v = op == 0 ? 0.f : vkl::h2f (r[0]);
+  for (int i = lane; i < W; i += 64)
+    {
+      const float e = vkl::h2f (r[i]);
+      v = op == 0 ? v + e : (op == 1 ? fmaxf (v, e) : fminf (v, e));
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    {
+      const float e = __shfl_xor (v, o, 64);
+      v = op == 0 ? v + e : (op == 1 ? fmaxf (v, e) : fminf (v, e));
+    }
+  if (lane == 0)
+    out[row] = vkl::f2h (v * scale);
+}
+
 inline unsigned
 blocks_for (size_t n, int threads)
 {
@@ -371,6 +416,48 @@ vkl_slice_f16 (const void *x, int C, int H, int W, int c0, int h0, int w0,
   slice_kernel<<<dim3 (blocks_for (total, 256)), dim3 (256), 0,
                  (hipStream_t)stream>>> ((const uint16_t *)x, H, W, c0, h0,
                                          w0, HE, WE, (uint16_t *)out, total);
+  return vkl_launch_status ();
+}
+
+int
+vkl_concat_part_f16 (const void *x, int C, int H, int W, size_t xcs,
+                     size_t xhs, void *out, size_t ocs, size_t ohs,
+                     size_t out_offset, void *stream)
+{
+  VKL_CHECK_ARG (x && out && C > 0 && H > 0 && W > 0);
+  const size_t total = (size_t)C * H * W;
+  copy_box_kernel<<<dim3 (blocks_for (total, 256)), dim3 (256), 0,
+                    (hipStream_t)stream>>> ((const uint16_t *)x, H, W, xcs,
+                                            xhs, 0, H, (uint16_t *)out, ocs,
+                                            ohs, out_offset, total);
+  return vkl_launch_status ();
+}
+
+int
+vkl_read_kvcache_f16 (const void *cache, int C, int H, int W, uint32_t offset,
+                      uint32_t len, void *out, void *stream)
+{
+  VKL_CHECK_ARG (cache && out && C > 0 && H > 0 && W > 0 && len > 0);
+  VKL_CHECK_ARG (len <= (uint32_t)H);
+  const size_t total = (size_t)C * len * W;
+  copy_box_kernel<<<dim3 (blocks_for (total, 256)), dim3 (256), 0,
+                    (hipStream_t)stream>>> (
+      (const uint16_t *)cache, (int)len, W, (size_t)H * W, (size_t)W,
+      (int)(offset % (uint32_t)H), H, (uint16_t *)out, (size_t)len * W,
+      (size_t)W, 0, total);
+  return vkl_launch_status ();
+}
+
+int
+vkl_reduce_f16 (const void *x, int C, int H, int W, int op, void *out,
+                void *stream)
+{
+  VKL_CHECK_ARG (x && out && C > 0 && H > 0 && W > 0 && op >= 0 && op <= 3);
+  const size_t rows = (size_t)C * H;
+  reduce_rows_kernel<<<dim3 (blocks_for (rows, 4)), dim3 (256), 0,
+                       (hipStream_t)stream>>> (
+      (const uint16_t *)x, W, op == 3 ? 0 : op,
+      op == 3 ? 1.0f / (float)W : 1.0f, (uint16_t *)out, rows);
   return vkl_launch_status ();
 }
 
