@@ -185,6 +185,20 @@ int vkl_argop_f16 (const void *x, int rows, int W, int op, uint32_t *out,
 /* src/ops/slice.cpp:30-77, src/shaders/slice_fp16.comp */
 int vkl_slice_f16 (const void *x, int C, int H, int W, int c0, int h0, int w0,
                    int CE, int HE, int WE, void *out, void *stream);
+/* models/samplers.cpp:37-101 on the device: the next token drawn from one row
+ * of V fp32 logits without the logits leaving device memory.  p < 0: the k
+ * largest logits (TopkSampler; k = 1 is the arg-max); p in [0, 1]: the most
+ * likely tokens until their mass reaches p (TopPSampler; at most 1024
+ * candidates).  Candidates rank by logit, ties toward the lower id; their
+ * probabilities are the softmax of the kept logits.  The draw inverts the
+ * cumulative distribution at one uniform number per (seed, counter +
+ * *counter_dev); counter_dev (device, optional) lets a position that lives
+ * on the device advance the generator.  tok: device; cand_ids / cand_probs /
+ * cand_n (device, optional, 1024 entries) receive the candidate set. */
+int vkl_sample_f32 (const float *logits, int V, int k, float p, uint64_t seed,
+                    uint32_t counter, const uint32_t *counter_dev,
+                    uint32_t *tok, uint32_t *cand_ids, float *cand_probs,
+                    uint32_t *cand_n, void *stream);
 /* src/ops/concat.cpp:68-188, src/shaders/concat_fp16.comp: one input of a
  * Concat copied into the output: out[c*ocs + y*ohs + x + out_offset] =
  * x[c*xcs + y*xhs + x] (element strides; the operator gives each input the

@@ -63,6 +63,14 @@ int vkl_model_generate_greedy (vkl_model *m, const uint32_t *prompt_h,
                                size_t n_prompt, size_t n_gen,
                                uint32_t *out_ids_h, double *prefill_ms,
                                double *decode_ms);
+/* the same loop with every token drawn on the device (vkl_sample_f32) from
+ * the topk largest logits (topp < 0) or the top-p set; position pos uses the
+ * uniform number of (seed, pos), so a seed reproduces the sequence */
+int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
+                                size_t n_prompt, size_t n_gen, int topk,
+                                float topp, uint64_t seed,
+                                uint32_t *out_ids_h, double *prefill_ms,
+                                double *decode_ms);
 /* options: fused one-token decode on/off, decode launch mode (0 = one launch
  * per phase, 1 = persistent, 2 = overlapped launches), the reference's last-block RoPE position quirk */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);

@@ -229,3 +229,37 @@ def test_graph_replayed_loop_equals_stepwise_and_oracle(n_prompt, n_gen):
         # eager work between replays: a plain forward pass
         m.forward(prompt[:3], 0)
     m.close()
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+def test_sampled_generation_on_the_device(small, fused):
+    """generate_sampled: k = 1 is the greedy sequence; a seed reproduces a top-k
+    sequence; every drawn token is one of the k most likely tokens of the
+    oracle's logits for the sequence so far (the candidate rule of
+    models/samplers.cpp:37-64), and top-p stays inside its candidate set."""
+    cfg, w = small
+    prompt = np.array([5, 17, 99, 3], np.uint32)
+    m = M.Llama2(cfg, w)
+    m.set_option("fused_decode", fused)
+    greedy, _, _ = m.generate_greedy(prompt, 12)
+    top1, _, _ = m.generate_sampled(prompt, 12, topk=1, seed=3)
+    assert list(top1) == list(greedy)
+    a, _, _ = m.generate_sampled(prompt, 16, topk=8, seed=7)
+    b, _, _ = m.generate_sampled(prompt, 16, topk=8, seed=7)
+    c, _, _ = m.generate_sampled(prompt, 16, topk=8, seed=8)
+    assert list(a) == list(b) and list(a) != list(c) and list(a) != list(greedy[:1]) * 16
+    om = O.OracleModel(cfg, w)
+    logits = om.forward(prompt, 0)
+    pos = len(prompt)
+    for t in a:
+        order = np.lexsort((np.arange(logits.size), -logits.astype(np.float64)))
+        # a logit within fp16 rounding of the k-th may swap places with it
+        assert int(t) in order[:8] or logits[t] >= logits[order[7]] - 2e-2 * abs(logits[order[7]])
+        logits = om.forward([int(t)], pos)
+        pos += 1
+    om.close()
+    d, _, _ = m.generate_sampled(prompt, 8, topp=0.0, seed=1)     # p = 0 keeps the top token only
+    assert list(d) == list(greedy[:8])
+    with pytest.raises(RuntimeError):
+        m.generate_sampled(prompt, 4, topk=0)
+    m.close()

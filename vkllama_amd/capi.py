@@ -14,6 +14,7 @@ HIP_LIB_PATH = os.path.join(_PKG, "lib", "libvkllama_hip.so")
 vp = C.c_void_p
 sz = C.c_size_t
 u32 = C.c_uint32
+u64 = C.c_uint64
 f32 = C.c_float
 i32 = C.c_int
 
@@ -58,6 +59,7 @@ SIGNATURES = {
     "vkl_kqv_q8_0": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp]),
     "vkl_ffn_upgate_q8_0": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "vkl_rope_kvwrite_f16": (i32, [vp, vp, vp, i32, i32, i32, sz, i32, i32, u32, u32, vp, vp, i32, vp, vp, i32, vp]),
+    "vkl_sample_f32": (i32, [vp, i32, i32, f32, u64, u32, vp, vp, vp, vp, vp, vp]),
     "vkl_concat_part_f16": (i32, [vp, i32, i32, i32, sz, sz, vp, sz, sz, sz, vp]),
     "vkl_read_kvcache_f16": (i32, [vp, i32, i32, i32, u32, u32, vp, vp]),
     "vkl_reduce_f16": (i32, [vp, i32, i32, i32, i32, vp, vp]),

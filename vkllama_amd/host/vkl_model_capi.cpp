@@ -188,6 +188,30 @@ vkl_model_generate_greedy (vkl_model *m, const uint32_t *prompt,
 }
 
 extern "C" int
+vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt,
+                            size_t n_prompt, size_t n_gen, int topk,
+                            float topp, uint64_t seed, uint32_t *out_ids,
+                            double *prefill_ms, double *decode_ms)
+{
+  if (!m || !m->model || !prompt || !out_ids)
+    return (int)absl::StatusCode::kInvalidArgument;
+  try
+    {
+      std::vector<uint32_t> p (prompt, prompt + n_prompt), out;
+      auto s = m->model->generate_sampled (p, n_gen, topk, topp, seed, out,
+                                           prefill_ms, decode_ms);
+      if (!s.ok ())
+        return fail (m, s);
+      std::copy (out.begin (), out.end (), out_ids);
+    }
+  catch (const std::exception &e)
+    {
+      return fail (m, absl::InternalError (e.what ()));
+    }
+  return 0;
+}
+
+extern "C" int
 vkl_model_set_option (vkl_model *m, const char *name, int value)
 {
   if (!m || !m->model || !name)

@@ -51,6 +51,8 @@ def main(argv=None):
     ap.add_argument("--topk", type=int, help="draw from the K most likely tokens (1 = greedy)")
     ap.add_argument("--topp", type=float, help="draw from the smallest set of tokens with probability mass P")
     ap.add_argument("--seed", type=int, help="seed of the sampler (default: random device)")
+    ap.add_argument("--device-sampler", action="store_true",
+                    help="draw on the device (no logits download per token); needs --seed or uses seed 0")
     args = ap.parse_args(argv)
 
     sp = None
@@ -69,7 +71,11 @@ def main(argv=None):
 
     from . import model as M
     m = M.Llama2.from_gguf(args.model, args.device)
-    if args.topp is not None or (args.topk or 1) > 1:
+    sampled = args.topp is not None or (args.topk or 1) > 1
+    if sampled and args.device_sampler:
+        out, prefill_ms, decode_ms = m.generate_sampled(np.array(ids, np.uint32), args.n_tokens, args.topk or 40,
+                                                        args.topp, args.seed or 0)
+    elif sampled:
         out, prefill_ms, decode_ms = generate_sampled(m, ids, args.n_tokens, args.topk, args.topp, args.seed)
     else:
         out, prefill_ms, decode_ms = m.generate_greedy(np.array(ids, np.uint32), args.n_tokens)

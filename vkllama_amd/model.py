@@ -29,6 +29,8 @@ SIGNATURES = {
     "vkl_model_vocab": (sz, [vp]),
     "vkl_model_forward": (i32, [vp, vp, sz, sz, vp]),
     "vkl_model_generate_greedy": (i32, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "vkl_model_generate_sampled": (i32, [vp, vp, sz, sz, i32, C.c_float, u64, vp, C.POINTER(C.c_double),
+                                         C.POINTER(C.c_double)]),
     "vkl_model_set_option": (i32, [vp, C.c_char_p, i32]),
     "vkl_model_read_kv_cache": (i32, [vp, sz, i32, vp, sz]),
     "vkl_model_decode_step_bytes": (sz, [vp, sz]),
@@ -217,6 +219,18 @@ class Llama2:
         self._check(lib().vkl_model_generate_greedy(self._h, prompt.ctypes.data, prompt.size, n_gen,
                                                     ids.ctypes.data, C.byref(t_pre), C.byref(t_dec)),
                     "vkl_model_generate_greedy")
+        return ids, t_pre.value, t_dec.value
+
+    def generate_sampled(self, prompt, n_gen, topk=40, topp=None, seed=0):
+        """Generation with the token drawn on the device: from the topk largest
+        logits, or (topp given) from the top-p set; seed fixes the sequence."""
+        prompt = np.ascontiguousarray(prompt, np.uint32)
+        ids = np.empty(n_gen, np.uint32)
+        t_pre, t_dec = C.c_double(0), C.c_double(0)
+        self._check(lib().vkl_model_generate_sampled(self._h, prompt.ctypes.data, prompt.size, n_gen, int(topk),
+                                                     -1.0 if topp is None else float(topp), int(seed),
+                                                     ids.ctypes.data, C.byref(t_pre), C.byref(t_dec)),
+                    "vkl_model_generate_sampled")
         return ids, t_pre.value, t_dec.value
 
     def read_kv_cache(self, layer, value):

@@ -184,4 +184,16 @@ DecodePlan::argmax_logits (uint32_t *dst)
   return hip_status ("argmax", vkl_argmax_f32 (p, (int)vocab_, dst,
                                                gpu_->stream ()));
 }
+
+absl::Status
+DecodePlan::sample_logits (uint32_t *dst, int topk, float topp, uint64_t seed,
+                           uint32_t counter)
+{
+  const Tensor &src = adopted_valid_ ? adopted_ : logits32_;
+  const float *p = (const float *)src.data () + (src.size () - vocab_);
+  return hip_status ("sample",
+                     vkl_sample_f32 (p, (int)vocab_, topk, topp, seed, counter,
+                                     nullptr, dst, nullptr, nullptr, nullptr,
+                                     gpu_->stream ()));
+}
 }

@@ -42,6 +42,10 @@ struct DecodePlan
   absl::Status adopt_logits (Tensor logits32);
   // arg-max of the current logits into device-visible memory
   absl::Status argmax_logits (uint32_t *dst);
+  // a token drawn from the current logits on the device (vkl_sample_f32):
+  // topp < 0 keeps the topk largest logits, else the top-p set
+  absl::Status sample_logits (uint32_t *dst, int topk, float topp,
+                              uint64_t seed, uint32_t counter);
 
 private:
   GPUDevice *gpu_;

@@ -455,6 +455,33 @@ Model::operator() (std::vector<uint32_t> const &toks, const size_t offset)
   return buf_logits;
 }
 
+// the next token from the logits of the last pass: arg-max, or a draw from
+// the top-k / top-p candidates with the uniform number of (seed, position)
+absl::Status
+Model::pick_token_ (uint32_t *dst, size_t position)
+{
+  if (!samp_on_)
+    return plan_->argmax_logits (dst);
+  return plan_->sample_logits (dst, samp_k_, samp_p_, samp_seed_,
+                               (uint32_t)position);
+}
+
+absl::Status
+Model::generate_sampled (std::vector<uint32_t> const &prompt, size_t n_gen,
+                         int topk, float topp, uint64_t seed,
+                         std::vector<uint32_t> &out, double *prefill_ms,
+                         double *decode_ms)
+{
+  if (topp < 0.f && topk < 1)
+    return absl::InvalidArgumentError ("top-k sampling needs k >= 1");
+  if (topp > 1.f)
+    return absl::InvalidArgumentError ("top-p sampling needs p in [0, 1]");
+  samp_on_ = true, samp_k_ = topk, samp_p_ = topp, samp_seed_ = seed;
+  auto s = generate_greedy (prompt, n_gen, out, prefill_ms, decode_ms);
+  samp_on_ = false;
+  return s;
+}
+
 absl::Status
 Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
                         std::vector<uint32_t> &out, double *prefill_ms,
@@ -495,14 +522,14 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
       VKLLAMA_STATUS_OK (logits32);
       VKLLAMA_STATUS_OK (plan_->adopt_logits (*logits32));
     }
-  VKLLAMA_STATUS_OK (plan_->argmax_logits (ids + 0));
+  VKLLAMA_STATUS_OK (pick_token_ (ids + 0, prompt.size ()));
   if (int e = vkl_stream_sync (s))
     return absl::InternalError (vkl_error_string (e));
   const auto t1 = clock::now ();
   size_t n_toks = prompt.size () + 1;
   size_t i0 = 1;
   if (fused_decode_ && plan_->usable () && decode_graph_ && plan_->mode () == 0
-      && n_gen > 1)
+      && n_gen > 1 && !samp_on_)
     {
       // ids[0] is at position prompt.size (); each replay appends one id
       VKLLAMA_STATUS_OK (plan_->loop (ids, prompt.size (), n_gen - 1));
@@ -513,8 +540,10 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
       if (fused_decode_ && plan_->usable ())
         {
           // the step's last launch reduces the arg-max partials into ids[i]
-          VKLLAMA_STATUS_OK (
-              plan_->step_device_token (ids + (i - 1), n_toks - 1, ids + i));
+          VKLLAMA_STATUS_OK (plan_->step_device_token (
+              ids + (i - 1), n_toks - 1, samp_on_ ? nullptr : ids + i));
+          if (samp_on_)
+            VKLLAMA_STATUS_OK (pick_token_ (ids + i, n_toks));
           continue;
         }
       else
@@ -528,7 +557,7 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
           VKLLAMA_STATUS_OK (logits32);
           VKLLAMA_STATUS_OK (plan_->adopt_logits (*logits32));
         }
-      VKLLAMA_STATUS_OK (plan_->argmax_logits (ids + i));
+      VKLLAMA_STATUS_OK (pick_token_ (ids + i, n_toks));
     }
   if (int e = vkl_stream_sync (s))
     return absl::InternalError (vkl_error_string (e));

@@ -169,6 +169,15 @@ public:
                                 size_t n_gen, std::vector<uint32_t> &out,
                                 double *prefill_ms = nullptr,
                                 double *decode_ms = nullptr);
+  // The same loop with the token drawn on the device from the top-k
+  // (topp < 0) or top-p candidates of every step's logits
+  // (models/samplers.cpp:37-101 as a kernel): logits never leave the device.
+  // The draw at position pos uses the uniform number of (seed, pos).
+  absl::Status generate_sampled (std::vector<uint32_t> const &prompt,
+                                 size_t n_gen, int topk, float topp,
+                                 uint64_t seed, std::vector<uint32_t> &out,
+                                 double *prefill_ms = nullptr,
+                                 double *decode_ms = nullptr);
   // copies one layer's K or V cache, [heads, maxlen, head_dim] fp16 bits
   absl::Status read_kv_cache (size_t layer, bool value,
                               std::vector<uint16_t> &out);
@@ -202,6 +211,12 @@ private:
   std::unique_ptr<ArgMax> argmax_;
   DecodePlan *plan_;
   bool decode_graph_ = true;
+  // sampling on the device during generate_*(): off = arg-max
+  bool samp_on_ = false;
+  int samp_k_ = 1;
+  float samp_p_ = -1.f;
+  uint64_t samp_seed_ = 0;
+  absl::Status pick_token_ (uint32_t *dst, size_t position);
 };
 
 }
