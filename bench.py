@@ -46,7 +46,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of a kernel from hardware counters (FETCH_SIZE +
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
-TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96258458}
+TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96227865}
 
 
 def cpu_baseline(cfg, weights, n_tokens):
@@ -73,6 +73,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS))
     ap.add_argument("--decode-mode", type=int, default=0)
+    ap.add_argument("--decode-graph", type=int, default=1, choices=(0, 1),
+                    help="1: the decode loop is replayed from a captured HIP graph; 0: the same launches step by step "
+                         "(for runs under a kernel tracer, which does not survive graph launches here)")
     ap.add_argument("--cpu-tokens", type=int, default=-1, help="decode tokens of the CPU baseline (0 = skip)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="before the timed region, launch the library's copy kernel N times on 1 GiB "
@@ -101,6 +104,7 @@ def main():
     t0 = time.perf_counter()
     m = M.Llama2(cfg, weights)
     m.set_option("decode_mode", args.decode_mode)
+    m.set_option("decode_graph", args.decode_graph)
     t_load = time.perf_counter() - t0
 
     if args.copy_calibration > 0:
@@ -132,7 +136,7 @@ def main():
     m.phase_times()
     m.generate_greedy(prompt, steps + 1)
     m.set_option("phase_timing", 0)
-    m.set_option("decode_graph", 1)
+    m.set_option("decode_graph", args.decode_graph)
     phases = m.phase_times()
     L_mid = int(ctx[len(ctx) // 2])
     per_phase = {}
@@ -183,8 +187,8 @@ def main():
         "data": "synthetic: random-init N(0,0.02) weights" + (" quantised to Q8_0" if cfg["wtype"] == 8 else " in FP16")
                 + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
-                   "decode_mode": ("launch-per-phase, replayed from a HIP graph", "persistent",
-                                   "overlapped-launches")[args.decode_mode],
+                   "decode_mode": ("launch-per-phase" + (", replayed from a HIP graph" if args.decode_graph else ""),
+                                   "persistent", "overlapped-launches")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "decode_tokens_per_second_host_interface": round(host_tok_s, 1),
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
@@ -205,6 +209,7 @@ def main():
     cpu_tokens = args.cpu_tokens
     if cpu_tokens < 0:
         cpu_tokens = 128 if cfg["dim"] >= 4096 else 1024
+    cpu_tokens = min(cpu_tokens, cfg["maxlen"] - 8)     # 4-token prompt, then one position per token
     if cpu_tokens > 0:
         v, dt = cpu_baseline(cfg, weights, cpu_tokens)
         result["cpu_baseline"] = {
