@@ -49,6 +49,7 @@ struct Scratch
 
 constexpr int kAttnChunks = 32;      // upper bound on chunks per head
 constexpr int kAttnSplitMinLen = 768; // shorter contexts use one workgroup per head
+constexpr int kAttnSweeps = 8;        // sweeps of cache rows a chunk kernel keeps in flight
 
 __host__ __device__ inline size_t
 align256 (size_t v)
@@ -1234,7 +1235,7 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
 {
   constexpr int LPR = HD / 8;             // lanes per cache row
   constexpr int RPS = kAttnThreads / LPR; // rows per sweep
-  constexpr int UN = 4;                   // sweeps in flight
+  constexpr int UN = kAttnSweeps;         // sweeps in flight
   extern __shared__ __align__ (16) uint8_t lds[];
   uint16_t *qk = (uint16_t *)lds;         // [2*HD]: rotated q, rotated k
   float *red = (float *)(lds + 1024);     // [8]
@@ -1248,6 +1249,25 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
   uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
   uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
   const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
+  if (l0 >= L)
+    {
+      // an empty chunk reports -inf / 0 and drops out of the sums
+      if (tid == 0)
+        {
+          stg (p.s.part_max + head * kAttnChunks + c, -INFINITY);
+          stg (p.s.part_sum + head * kAttnChunks + c, 0.f);
+        }
+      return;
+    }
+  // The first sweeps of K are requested before anything else, so that they
+  // travel while q is rotated: unconditional loads from clamped rows (a load
+  // under a branch would make every later wait a wait for all loads); rows
+  // past the chunk are ignored below, the row of the new position, which this
+  // kernel is writing at the same time, is replaced by the rotated k.
+  uint4 kv[UN];
+#pragma unroll
+  for (int j = 0; j < UN; ++j)
+    kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPS + grp, l1 - 1) * HD + sub * 8);
 
   if (tid < HD && (tid < HD / 2 || has_new))
     {
@@ -1275,23 +1295,21 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
   const float scale = 1.0f / sqrtf ((float)HD);
   const uint4 qv = ((const uint4 *)qk)[sub];
   float mx = -INFINITY;
+  const uint4 knew = ((const uint4 *)(qk + HD))[sub];
   for (int lb = l0; lb < l1; lb += UN * RPS)
     {
-      uint4 kv[UN];
-#pragma unroll
-      for (int j = 0; j < UN; ++j)
+      if (lb > l0)
         {
-          const int l = lb + j * RPS + grp;
-          kv[j] = make_uint4 (0, 0, 0, 0);
-          if (l < l1)
-            kv[j] = l == pos ? ((const uint4 *)(qk + HD))[sub]
-                             : ldg4 (kc + (size_t)l * HD + sub * 8);
+#pragma unroll
+          for (int j = 0; j < UN; ++j)
+            kv[j] = ldg4 (kc + (size_t)min (lb + j * RPS + grp, l1 - 1) * HD + sub * 8);
         }
 #pragma unroll
       for (int j = 0; j < UN; ++j)
         {
           const int l = lb + j * RPS + grp;
-          float sv = dot8_f16 (qv, kv[j], 0.f);
+          const uint4 kr = l == pos ? knew : kv[j];
+          float sv = dot8_f16 (qv, kr, 0.f);
 #pragma unroll
           for (int o = LPR >> 1; o > 0; o >>= 1)
             sv += __shfl_xor (sv, o, 64);
@@ -1319,7 +1337,6 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
   __syncthreads ();
   if (tid == 0)
     {
-      // an empty chunk (l0 >= L) reports -inf / 0 and drops out of the sums
       stg (p.s.part_max + head * kAttnChunks + c, mx);
       stg (p.s.part_sum + head * kAttnChunks + c,
            red[4] + red[5] + red[6] + red[7]);
@@ -1332,7 +1349,7 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
 {
   constexpr int LPR = HD / 8;
   constexpr int RPS = kAttnThreads / LPR;
-  constexpr int UN = 4;
+  constexpr int UN = kAttnSweeps;
   __shared__ float part[RPS * HD];
   const int head = blockIdx.y, c = blockIdx.x;
   const int maxlen = p.m.maxlen;
@@ -1342,16 +1359,38 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
   const uint16_t *vc = (const uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
   const uint16_t *sc16 = p.s.sc16 + (size_t)head * maxlen;
   const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
-
-  float M = -INFINITY;
-  for (int i = 0; i < C; ++i)
-    M = fmaxf (M, ldg (p.s.part_max + head * kAttnChunks + i));
+  if (l0 >= L)
+    {
+      if (tid < HD)
+        stg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid, 0.f);
+      return;
+    }
+  // One lane per chunk fetches that chunk's maximum and sum; the V rows and
+  // scores of the first sweeps are requested right behind them (unconditional,
+  // clamped rows), and travel while M and S are formed.
+  const int ci = tid & 31; // kAttnChunks <= 32
+  const float mi = ldg (p.s.part_max + head * kAttnChunks + min (ci, C - 1));
+  const float si = ldg (p.s.part_sum + head * kAttnChunks + min (ci, C - 1));
+  uint4 vv[UN];
+  uint16_t sh[UN];
+#pragma unroll
+  for (int j = 0; j < UN; ++j)
+    {
+      const int lc = min (l0 + j * RPS + grp, l1 - 1);
+      vv[j] = ldg4 (vc + (size_t)lc * HD + sub * 8);
+      sh[j] = ldg (sc16 + lc);
+    }
+  float M = ci < C ? mi : -INFINITY;
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1)
+    M = fmaxf (M, __shfl_xor (M, o, 64));
+  // chunks in index order, as a sequential loop would add them
   float S = 0.f;
   for (int i = 0; i < C; ++i)
     {
-      const float mi = ldg (p.s.part_max + head * kAttnChunks + i);
-      if (mi > -INFINITY)
-        S += ldg (p.s.part_sum + head * kAttnChunks + i) * expf (mi - M);
+      const float m_i = __shfl (mi, i, 64), s_i = __shfl (si, i, 64);
+      if (m_i > -INFINITY)
+        S += s_i * expf (m_i - M);
     }
 
   float acc[8];
@@ -1360,18 +1399,14 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
     acc[j] = 0.f;
   for (int lb = l0; lb < l1; lb += UN * RPS)
     {
-      uint4 vv[UN];
-      uint16_t sh[UN];
-#pragma unroll
-      for (int j = 0; j < UN; ++j)
+      if (lb > l0)
         {
-          const int l = lb + j * RPS + grp;
-          vv[j] = make_uint4 (0, 0, 0, 0);
-          sh[j] = 0;
-          if (l < l1)
+#pragma unroll
+          for (int j = 0; j < UN; ++j)
             {
-              vv[j] = ldg4 (vc + (size_t)l * HD + sub * 8);
-              sh[j] = ldg (sc16 + l);
+              const int lc = min (lb + j * RPS + grp, l1 - 1);
+              vv[j] = ldg4 (vc + (size_t)lc * HD + sub * 8);
+              sh[j] = ldg (sc16 + lc);
             }
         }
 #pragma unroll
@@ -1816,7 +1851,11 @@ launch_attention (const Params &p, const vkl_decode_model *m,
   const int L = (int)p.pos + 1;
   if (L < kAttnSplitMinLen)
     return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
+  // enough chunks to occupy the GPU, and, up to the bound, so many that a
+  // chunk's rows are all in flight at once (kAttnSweeps sweeps of 256 lanes)
   int C = (2 * n_cu + m->n_heads - 1) / m->n_heads;
+  const int rows_in_flight = kAttnSweeps * kAttnThreads / (m->head_dim / 8);
+  C = std::max (C, (L + rows_in_flight - 1) / rows_in_flight);
   C = C < 1 ? 1 : (C > kAttnChunks ? kAttnChunks : C);
   const int R = (L + C - 1) / C;
   const size_t lds_a = 1024 + 64 + (size_t)R * 4;
