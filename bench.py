@@ -66,12 +66,83 @@ def cpu_baseline(cfg, weights, n_tokens):
     return n_tokens / dt, dt
 
 
+def bench_single_matmul(args):
+    """Benchmark configuration 1: y[1,4096] = x[1,4096] W[4096,4096]^T with W in Q8_0 (int8 uniform in
+    [-127,127], fp16 scales U(0.001,0.01)), x ~ N(0,1) fp16, through vkl_matmul_q8_0.  A step is one call.  The
+    HBM figure cycles through a ring of 32 distinct matrices (571 MB, more than every cache); the same call on
+    one matrix over and over is reported beside it as the cache-resident figure."""
+    import ctypes as C
+    from vkllama_amd import capi
+    from oracle import oracle as O
+    N = K = 4096
+    ring, steps, warmup = 32, args.steps, args.warmup
+    rng = np.random.default_rng(args.seed)
+    dev = capi.Device(0)
+    L = capi.lib()
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    dx, dy = dev.upload(x), dev.alloc(N * 2)
+    raws, mats = [], []
+    for i in range(ring):
+        raw = np.zeros((N, K // 32, 34), np.uint8)
+        raw[:, :, 2:] = rng.integers(-127, 128, (N, K // 32, 32)).astype(np.int8).view(np.uint8)
+        raw[:, :, 0:2] = rng.uniform(0.001, 0.01, (N, K // 32)).astype(np.float16).view(np.uint8).reshape(N, K // 32, 2)
+        if i == 0:
+            raws.append(raw)
+        mats.append(dev.upload_q8_0(raw, N, K))
+
+    def run(n, same):
+        for i in range(n):
+            w = mats[0 if same else i % ring]
+            capi.check(L.vkl_matmul_q8_0(dx.ptr, w.ptr, 1, N, K, K, N, C.c_float(1.0), C.c_float(0.0), 0, None,
+                                         dy.ptr, None, dev.stream), "vkl_matmul_q8_0")
+
+    def timed(n, same):
+        run(warmup, same)
+        dev.sync()
+        e0, e1 = dev.event(), dev.event()
+        dev.record(e0)
+        run(n, same)
+        dev.record(e1)
+        return dev.elapsed_ms(e0, e1) / n
+
+    ms = timed(steps, False)
+    ms_hot = timed(steps, True)
+    run(1, True)
+    got = dy.read(np.float16, (1, N))
+    want = O.matmul_q8_0(x, raws[0].reshape(N, -1), K)
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))
+                       / np.maximum(np.abs(want.astype(np.float64)), 1e-2 * np.abs(want).max())))
+    nbytes = N * (K // 32) * 34 + K * 2 + N * 2           # 17,842,176
+    t0 = time.perf_counter()
+    n_cpu = 200
+    for _ in range(n_cpu):
+        O.matmul_q8_0(x, raws[0].reshape(N, -1), K)
+    cpu_calls = n_cpu / (time.perf_counter() - t0)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "q8_0_matmul_4096x4096_bs1_calls_per_second", "value": round(1e3 / ms, 1), "unit": "calls/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "q8_0 weights x f16 activations, f32 accumulate",
+        "data": "synthetic: int8 U[-127,127], fp16 scales U(0.001,0.01), x N(0,1); ring of %d matrices" % ring,
+        "config": {"workload": args.workload, "M": 1, "N": N, "K": K, "ring": ring},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "decode_phase_kernel<gemv> (the decode step's weight-streaming kernel, stand-alone)",
+                     "avg_launch_us": round(ms * 1e3, 3), "launches_timed": steps, "bytes_per_launch": nbytes,
+                     "cache_resident_avg_launch_us": round(ms_hot * 1e3, 3),
+                     "cache_resident_gbs": round(nbytes / (ms_hot * 1e-3) / 1e9, 1)},
+        "max_rel_err_vs_oracle": err,
+        "cpu_baseline": {"value": round(cpu_calls, 1), "unit": "calls/s",
+                         "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count())), "kind": "port",
+                         "sample": "%d calls of the oracle's matmul on the first matrix" % n_cpu}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS) + ["matmul-q8_0-4096"])
     ap.add_argument("--decode-mode", type=int, default=0)
     ap.add_argument("--decode-graph", type=int, default=1, choices=(0, 1),
                     help="1: the decode loop is replayed from a captured HIP graph; 0: the same launches step by step "
@@ -85,6 +156,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (batch-1 decode is a single dependency chain and "
                  "would shard by tensor parallelism, which is not built); got --gpus %d" % args.gpus)
+
+    if args.workload == "matmul-q8_0-4096":
+        return bench_single_matmul(args)
 
     from vkllama_amd import capi, model as M
 

@@ -93,6 +93,7 @@ struct Params
   // memory so that every step is the same sequence of launches
   const uint32_t *loop; // {index into ids, position}, or null
   uint32_t *ids;        // loop: input token ids[index], result to ids[index + 1]
+  const uint16_t *gemv_res; // stand-alone product (PH_GEMV): residual operand or null
 #ifdef VKL_TRACE
   unsigned long long *trace; // [phase slot][wg][8] wall-clock stamps
 #endif
@@ -902,7 +903,8 @@ enum Phase
   PH_UPGATE,
   PH_DOWN,
   PH_HEAD,
-  PH_ARGMAX
+  PH_ARGMAX,
+  PH_GEMV // a stand-alone y = W x (+ residual) on the down projection's path
 };
 
 template <bool COH>
@@ -1016,7 +1018,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
   uint16_t *xl = (uint16_t *)lds;
-  const int kstage = phase == PH_DOWN ? ffn : dim;
+  const int kstage = phase == PH_DOWN || phase == PH_GEMV ? ffn : dim;
   float *red = (float *)(lds + (size_t)kstage * 2); // 2*kDecWaves words
   uint8_t *nl = lds + (size_t)kstage * 2 + 256;     // parked norm weights
   Epilogue e = {};
@@ -1169,6 +1171,18 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
+        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        break;
+      }
+    case PH_GEMV:
+      {
+        // y[dim] = W[dim, ffn] x[ffn] (+ residual) for a caller's operands:
+        // x in s.t, y in s.x, W in w_down
+        const QMat w = wmat<WT> (lw.w_down, dim, ffn);
+        issue_x<COH> (p.s.t, ffn, x);
+        Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.gemv_res);
+        finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
+        e.y[0] = p.s.x, e.residual = p.gemv_res;
         Gemv<COH, WT>::run (ps, A, B, xl, e, red);
         break;
       }
@@ -2061,6 +2075,48 @@ launch_step (const Params &p, const vkl_decode_model *m, int n_cu, int G,
 
 }
 
+namespace vkl
+{
+// One token row times a matrix on the decode step's down-projection kernel:
+// y[N] = W[N, K] x[K] (+ residual), W planar Q8_0 (wtype 8) or dense fp16.
+bool
+decode_gemv_supported (int N, int K, int wtype)
+{
+  return (wtype == 8 || wtype == 1) && N > 0 && (N % 2) == 0 && K > 0
+         && (K % 32) == 0 && K <= 16384 && N <= (1 << 24)
+         && lds_bytes_needed (0, K, 1, 64) <= 160 * 1024;
+}
+
+int
+decode_gemv_launch (const void *x, const void *w, int wtype, int N, int K,
+                    const void *residual, void *y, hipStream_t s)
+{
+  if (!decode_gemv_supported (N, K, wtype))
+    return (int)hipErrorInvalidValue;
+  static int n_cu = 0;
+  if (n_cu == 0)
+    {
+      int dev = 0;
+      VKL_HIP (hipGetDevice (&dev));
+      VKL_HIP (hipDeviceGetAttribute (&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+  Params p = {};
+  p.m.dim = N, p.m.ffn = K, p.m.wtype = wtype;
+  p.s.t = (uint16_t *)x;
+  p.s.x = (uint16_t *)y;
+  p.gemv_res = (const uint16_t *)residual;
+  vkl_layer_weights lw = {};
+  lw.w_down = w;
+  const int G = n_cu * 2;
+  // staged activation row + reduction words (no norm weights are parked)
+  const size_t lds = (size_t)K * 2 + 256 + 64;
+  if (int e = wtype == 8 ? launch_phase_wt<PH_GEMV, 8> (p, lw, 0, G, G, lds, s)
+                         : launch_phase_wt<PH_GEMV, 1> (p, lw, 0, G, G, lds, s))
+    return e;
+  return vkl_launch_status ();
+}
+}
+
 extern "C" int
 vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
                  int mode, float *logits32, uint32_t *next_tok, void *stream)
@@ -2089,6 +2145,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.logits32 = logits32 ? logits32 : p.s.logits32;
   p.next_tok = next_tok;
   p.loop = nullptr, p.ids = nullptr;
+  p.gemv_res = nullptr;
 #ifdef VKL_TRACE
   p.trace = g_trace;
 #endif
@@ -2297,6 +2354,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.logits32 = p.s.logits32;
   p.next_tok = nullptr;
   p.loop = nullptr, p.ids = nullptr;
+  p.gemv_res = nullptr;
   p.wait_target = 0;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;

@@ -39,5 +39,12 @@ constexpr int kGemmMinRows = 9;
 // true if the shapes/alignments are ones the kernel covers
 bool gemm_mfma_supported (const GemmArgs &a);
 int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
+
+// One token row: y[N] = W[N, K] x[K] (+ residual) on the weight-streaming
+// kernel of the decode step (vkl_decode.hip); W planar Q8_0 (wtype 8) or
+// dense fp16 [N, K] (wtype 1).
+bool decode_gemv_supported (int N, int K, int wtype);
+int decode_gemv_launch (const void *x, const void *w, int wtype, int N, int K,
+                        const void *residual, void *y, hipStream_t s);
 }
 #endif

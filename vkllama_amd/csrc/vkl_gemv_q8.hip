@@ -258,6 +258,10 @@ vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
   a.act = act;
   a.residual = (const uint16_t *)residual;
   a.y32 = y32;
+  // one row, plain epilogue: the decode step's streaming kernel
+  if (M == 1 && scale == 1.0f && bias == 0.0f && act == 0 && !y32
+      && ((uintptr_t)x % 16) == 0 && vkl::decode_gemv_supported (N, K, 8))
+    return vkl::decode_gemv_launch (x, w_planar, 8, N, K, residual, y, (hipStream_t)stream);
   int err = 0;
   if (try_gemm (a, 1, 0, (hipStream_t)stream, err))
     return err;
