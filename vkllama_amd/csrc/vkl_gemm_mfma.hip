@@ -19,6 +19,9 @@
 // tile they share stays in that XCD's L2.
 #include "vkl_common.h"
 #include "vkl_gemm.h"
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace vkl
 {
@@ -652,10 +655,250 @@ gemm_skinny_kernel (const GemmArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------
+// few token rows (M <= 32), second form: K split over workgroups as well
+// ---------------------------------------------------------------------------
+// The form above keeps a wave's x fragments in registers next to its weight
+// fragments; an x fragment is twice the bytes of the Q8_0 weights it meets, so
+// few weight bytes are in flight per compute unit, in two dependent rounds, and
+// a matrix of 4096 rows occupies half the compute units.  Here a workgroup
+// owns 32 weight rows and a 1024-wide slice of K: its 32 x 1024 piece of x
+// goes to LDS once (64 KiB, so two workgroups share a compute unit and one
+// streams while the other reduces), each of the 8 waves requests ALL of its
+// weights (4 Q8_0 blocks of 32 rows) at the start, in one round, and reads
+// the x operand from LDS.  The slices' partial sums (fp32) go to a workspace and a
+// second small kernel adds them in slice order and applies the epilogue, so
+// the result does not depend on timing.
+constexpr int kSk2Waves = 8;
+constexpr int kSk2Slice = 1024;                // k extent of a workgroup
+constexpr int kSk2Ldx = kSk2Slice + 8;         // LDS row stride of x in halves
+constexpr size_t kSk2Workspace = 32u << 20;    // bytes, per stream
+
+template <int WT>
+__global__ __launch_bounds__ (kSk2Waves * 64) void
+gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
+{
+  constexpr int UN = kSk2Slice / 32 / kSk2Waves; // blocks per wave: 4
+  extern __shared__ __align__ (16) uint8_t lds[];
+  uint16_t *xs = (uint16_t *)lds; // [32][kSk2Ldx]
+  float *red = (float *)lds;      // after the products: [waves][32][33]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5;
+  const int n0 = blockIdx.x * 32, slice = blockIdx.y, mat = blockIdx.z;
+  const int k0 = slice * kSk2Slice;
+  const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
+  const void *zeros = g_zero_chunk;
+
+  // all weights of the wave, then the workgroup's piece of x
+  uint4 wv[UN][WT == 8 ? 1 : 2];
+  uint16_t dv[UN];
+  const int bw = k0 / 32 + wave * UN; // first block of the wave
+#pragma unroll
+  for (int u = 0; u < UN; ++u)
+    {
+      const int k = (bw + u) * 32 + g * 16;
+      if (WT == 8)
+        {
+          const bool v = k < a.Kp;
+          const uint8_t *wq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat) + (size_t)nrow * a.Kp;
+          const uint16_t *wd
+              = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat) + (size_t)nrow * (a.Kp >> 5);
+          wv[u][0] = ldg16 (v ? (const void *)(wq + k) : zeros);
+          dv[u] = ldg (v ? wd + (bw + u) : (const uint16_t *)zeros);
+        }
+      else
+        {
+          const bool v = k + 16 <= a.K;
+          const uint16_t *wh = (const uint16_t *)pick3 (a.wh[0], a.wh[1], a.wh[2], mat) + (size_t)nrow * a.ws;
+          wv[u][0] = ldg16 (v ? (const void *)(wh + k) : zeros);
+          wv[u][WT == 8 ? 0 : 1] = ldg16 (v ? (const void *)(wh + k + 8) : zeros);
+          dv[u] = 0;
+        }
+    }
+  {
+    constexpr int CPR = kSk2Slice / 8;                         // chunks per x row
+    constexpr int NCH = 32 * CPR / (kSk2Waves * 64);           // per thread: 8
+    uint4 xv[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+      {
+        const int c = tid + i * kSk2Waves * 64;
+        const int row = c / CPR, k = k0 + (c % CPR) * 8;
+        const bool v = row < a.M && k + 8 <= a.K;
+        xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
+      }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+      {
+        const int c = tid + i * kSk2Waves * 64;
+        *(uint4 *)(xs + (c / CPR) * kSk2Ldx + (c % CPR) * 8) = xv[i];
+      }
+  }
+  __syncthreads ();
+
+  float16v acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+  const uint16_t *xa = xs + (lane & 31) * kSk2Ldx + wave * UN * 32 + g * 16;
+#pragma unroll
+  for (int u = 0; u < UN; ++u)
+    {
+      // operands: A = x (rows = tokens), B = weights (columns = rows n); a
+      // lane's 16 consecutive k values feed two MFMAs
+      const half8 a0 = *(const half8 *)(xa + u * 32), a1 = *(const half8 *)(xa + u * 32 + 8);
+      half8 b0, b1;
+      if (WT == 8)
+        {
+          const uint32_t w[4] = { wv[u][0].x, wv[u][0].y, wv[u][0].z, wv[u][0].w };
+          uint32_t o[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              h16x2 lo, hi;
+              i8x4_to_h2x2 (w[j], lo, hi);
+              o[2 * j] = __builtin_bit_cast (uint32_t, lo);
+              o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
+            }
+          b0 = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
+          b1 = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
+          // Q8_0: block sum from a zero accumulator, times the block scale
+          float16v part;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            part[r] = 0.f;
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, part, 0, 0, 0);
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, part, 0, 0, 0);
+          const float sc = h2f (dv[u]);
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[r] += part[r] * sc;
+        }
+      else
+        {
+          b0 = __builtin_bit_cast (half8, wv[u][0]);
+          b1 = __builtin_bit_cast (half8, wv[u][WT == 8 ? 0 : 1]);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, acc, 0, 0, 0);
+        }
+    }
+
+  // add the waves' parts of the slice (x in LDS is no longer needed)
+  __syncthreads ();
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    red[(wave * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) * 33 + (lane & 31)] = acc[r];
+  __syncthreads ();
+  for (int i = tid; i < 32 * 32; i += kSk2Waves * 64)
+    {
+      const int m = i >> 5, nn = i & 31, n = n0 + nn;
+      if (m < a.M && n < a.N)
+        {
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < kSk2Waves; ++w)
+            v += red[(w * 32 + m) * 33 + nn];
+          ws[((size_t)(mat * S + slice) * 32 + m) * a.N + n] = v;
+        }
+    }
+}
+
+// sum over the slices in order, then the epilogue of the product
+__global__ __launch_bounds__ (256) void
+skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S)
+{
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)a.M * a.N)
+    return;
+  const int m = (int)(i / a.N), n = (int)(i % a.N);
+  const int nm = a.upgate ? 2 : a.nmat;
+  float v[3] = { 0.f, 0.f, 0.f };
+  for (int t = 0; t < nm; ++t)
+    for (int sl = 0; sl < S; ++sl)
+      v[t] += ldg (ws + ((size_t)(t * S + sl) * 32 + m) * a.N + n);
+  const size_t o = (size_t)m * a.ys + n;
+  if (a.upgate)
+    {
+      a.y[0][o] = f2h (silu (v[1]) * v[0]);
+      return;
+    }
+  if (a.nmat > 1)
+    {
+      for (int t = 0; t < a.nmat; ++t)
+        a.y[t][o] = f2h (v[t]);
+      return;
+    }
+  float r = v[0] * a.scale + a.bias;
+  if (a.act == 1)
+    r = silu (r);
+  uint16_t h = f2h (r);
+  if (a.residual)
+    h = f2h (h2f (h) + h2f (ldg (a.residual + o)));
+  a.y[0][o] = h;
+  if (a.y32)
+    a.y32[(size_t)m * a.N + n] = h2f (h);
+}
+
+// fp32 workspace of the split form, one per stream, kept for the life of the
+// process
+float *
+skinny2_workspace (hipStream_t s)
+{
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, float *> table;
+  std::lock_guard<std::mutex> lock (mu);
+  int dev = 0;
+  if (hipGetDevice (&dev) != hipSuccess)
+    return nullptr;
+  auto it = table.find ({ dev, s });
+  if (it != table.end ())
+    return it->second;
+  void *p = nullptr;
+  if (hipMalloc (&p, kSk2Workspace) != hipSuccess)
+    return nullptr;
+  table[{ dev, s }] = (float *)p;
+  return (float *)p;
+}
+
+template <int WT>
+bool
+launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
+{
+  if (a.M > 32 || a.batch > 1)
+    return false;
+  const int keff = WT == 8 ? a.Kp : a.K;
+  const int S = (keff + kSk2Slice - 1) / kSk2Slice;
+  const int nm = a.upgate ? 2 : a.nmat;
+  if ((size_t)nm * S * 32 * a.N * sizeof (float) > kSk2Workspace)
+    return false;
+  static bool lds_set = false;
+  const size_t lds = (size_t)32 * kSk2Ldx * 2;
+  if (!lds_set)
+    {
+      if (hipFuncSetAttribute ((const void *)gemm_skinny2_kernel<WT>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+          != hipSuccess)
+        return false;
+      lds_set = true;
+    }
+  float *ws = skinny2_workspace (s);
+  if (!ws)
+    return false;
+  gemm_skinny2_kernel<WT><<<dim3 ((unsigned)((a.N + 31) / 32), (unsigned)S, (unsigned)nm),
+                           dim3 (kSk2Waves * 64), lds, s>>> (a, ws, S);
+  const size_t total = (size_t)a.M * a.N;
+  skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S);
+  err = (int)hipGetLastError ();
+  return true;
+}
+
 template <int WT>
 int
 launch_skinny (const GemmArgs &a, hipStream_t s)
 {
+  int err = 0;
+  if (launch_skinny2<WT> (a, s, err))
+    return err;
   const dim3 grid ((unsigned)((a.N + 31) / 32), 1, (unsigned)(a.upgate ? 1 : a.nmat));
   // sixteen waves where their registers (128 each) and the reduction buffer allow
   if (a.upgate)
