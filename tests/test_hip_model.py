@@ -185,7 +185,7 @@ def test_other_decode_modes_match_oracle(cfg, seed, mode):
 
 @pytest.mark.parametrize("heads", [4, 2])
 def test_long_context_decode_uses_split_attention(heads):
-    """Past 768 positions the decode step splits each head's context over
+    """Past 544 positions the decode step splits each head's context over
     several workgroups (scores / values / combine launches); logits, greedy ids
     and the cache rows written on the way must still match the oracle."""
     cfg = dict(dim=256, n_layers=2, n_heads=heads, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
@@ -209,12 +209,12 @@ def test_long_context_decode_uses_split_attention(heads):
     m.close()
 
 
-@pytest.mark.parametrize("n_prompt,n_gen", [(4, 40), (760, 24)])
+@pytest.mark.parametrize("n_prompt,n_gen", [(4, 40), (536, 24), (760, 24)])
 def test_graph_replayed_loop_equals_stepwise_and_oracle(n_prompt, n_gen):
     """generate_greedy replays one captured step per token (token index and
     position advance in device memory); the ids must equal those of the
     step-by-step launches and the oracle's, also across the switch of the
-    attention phase to its split form at 768 positions, and on a second use
+    attention phase to its split form at 544 positions, and on a second use
     of the cached graphs."""
     cfg = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
     w = M.synth_weights(cfg, seed=33)

@@ -48,7 +48,8 @@ struct Scratch
 };
 
 constexpr int kAttnChunks = 32;      // upper bound on chunks per head
-constexpr int kAttnSplitMinLen = 768; // shorter contexts use one workgroup per head
+constexpr int kAttnSplitMinLen = 544; // shorter contexts use one workgroup per head (measured
+                                      // break-even of the two forms at 7B: 540 positions)
 constexpr int kAttnSweeps = 8;        // sweeps of cache rows a chunk kernel keeps in flight
 
 __host__ __device__ inline size_t
@@ -1457,9 +1458,16 @@ __global__ __launch_bounds__ (HD) void
 attn_combine_kernel (const Params p, int C)
 {
   const int head = blockIdx.x, tid = threadIdx.x;
+  // all parts are requested at once (a loop with a run-time bound would wait
+  // for each load before the next); they are added in chunk order
+  float part[kAttnChunks];
+#pragma unroll
+  for (int c = 0; c < kAttnChunks; ++c)
+    part[c] = ldg (p.s.part_out + ((size_t)head * kAttnChunks + min (c, C - 1)) * HD + tid);
   float o = 0.f;
-  for (int c = 0; c < C; ++c)
-    o += ldg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid);
+#pragma unroll
+  for (int c = 0; c < kAttnChunks; ++c)
+    o += c < C ? part[c] : 0.f;
   stg (p.s.att + head * HD + tid, f2h (o));
 }
 
