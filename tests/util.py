@@ -34,3 +34,15 @@ def ulp_diff_f16(a, b):
         u = np.ascontiguousarray(x, np.float16).view(np.uint16).astype(np.int32)
         return np.where(u & 0x8000, -(u & 0x7fff), u)
     return np.abs(key(a) - key(b))
+
+
+def within_one_ulp_or_cancelled(got, want, frac=1e-3):
+    """True where two fp16 results of the same sum agree to one ulp, or, for a
+    sum whose terms cancel to a value far below the row's scale, to `frac` of
+    the largest magnitude in `want`: fp32 partial sums taken in another order
+    differ by rounding noise of the TERMS, which can exceed one ulp of a tiny
+    result."""
+    g = np.asarray(got, np.float64)
+    w = np.asarray(want, np.float64)
+    return (ulp_diff_f16(got, want) <= 1) | (np.abs(g - w) <= frac * np.abs(w).max())
+

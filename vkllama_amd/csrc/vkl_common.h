@@ -64,23 +64,68 @@ ldg4 (const void *p)
   return make_uint4 (v.x, v.y, v.z, v.w);
 }
 
-// sum over the 64 lanes of a wave; every lane gets the total.
+// Cross-lane data movement by DPP (a modifier of a VALU instruction, a few
+// cycles) instead of ds_bpermute (a trip through the LDS crossbar that also
+// counts against the LDS counter): v of the lane chosen by CTRL within the
+// lane's row of 16.  0xB1 / 0x4E swap neighbours / pairs inside a quad, 0x141
+// mirrors a half row (8 lanes), 0x140 a row.
+template <int CTRL>
+__device__ __forceinline__ float
+dpp_get (float v)
+{
+  return __builtin_bit_cast (
+      float, __builtin_amdgcn_update_dpp (0, __builtin_bit_cast (int, v), CTRL, 0xf, 0xf, false));
+}
+
+// sum / maximum over groups of LANES (4, 8 or 16) consecutive lanes; every
+// lane of a group gets the group's result
+template <int LANES>
+__device__ __forceinline__ float
+row_sum (float v)
+{
+  v += dpp_get<0xB1> (v);
+  v += dpp_get<0x4E> (v);
+  if (LANES >= 8)
+    v += dpp_get<0x141> (v);
+  if (LANES >= 16)
+    v += dpp_get<0x140> (v);
+  return v;
+}
+
+template <int LANES>
+__device__ __forceinline__ float
+row_max (float v)
+{
+  v = fmaxf (v, dpp_get<0xB1> (v));
+  v = fmaxf (v, dpp_get<0x4E> (v));
+  if (LANES >= 8)
+    v = fmaxf (v, dpp_get<0x141> (v));
+  if (LANES >= 16)
+    v = fmaxf (v, dpp_get<0x140> (v));
+  return v;
+}
+
+__device__ __forceinline__ float
+lane_value (float v, int lane)
+{
+  return __builtin_bit_cast (float, __builtin_amdgcn_readlane (__builtin_bit_cast (int, v), lane));
+}
+
+// sum over the 64 lanes of a wave; every lane gets the total: the four rows
+// of 16 by DPP, their results through scalar registers.
 __device__ __forceinline__ float
 wave_sum (float v)
 {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    v += __shfl_xor (v, o, 64);
-  return v;
+  v = row_sum<16> (v);
+  return (lane_value (v, 0) + lane_value (v, 16)) + (lane_value (v, 32) + lane_value (v, 48));
 }
 
 __device__ __forceinline__ float
 wave_max (float v)
 {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    v = fmaxf (v, __shfl_xor (v, o, 64));
-  return v;
+  v = row_max<16> (v);
+  return fmaxf (fmaxf (lane_value (v, 0), lane_value (v, 16)),
+                fmaxf (lane_value (v, 32), lane_value (v, 48)));
 }
 
 __device__ __forceinline__ float

@@ -734,7 +734,7 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
 {
   constexpr int LPR = HD / 8;            // lanes per cache row (16 B each)
   constexpr int RPB = kDecThreads / LPR; // cache rows per sweep
-  constexpr int PRE = 4;                 // sweeps prefetched up front
+  constexpr int PRE = 8;                 // sweeps prefetched up front
   const int dim = p.m.dim, maxlen = p.m.maxlen;
   const uint32_t pos = step_pos (p);
   const int L = (int)pos + 1;
@@ -794,9 +794,7 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   const uint4 qv = ((const uint4 *)qk)[sub];
   auto score_row = [&] (int l, const uint4 kv) {
     float s = l < L ? dot8_f16 (qv, kv, 0.f) : 0.f;
-#pragma unroll
-    for (int o = LPR >> 1; o > 0; o >>= 1)
-      s += __shfl_xor (s, o, 64);
+    s = row_sum<LPR> (s);
     if (l < L && sub == 0)
       sc[l] = h2f (f2h (s * scale + 0.f));
   };
@@ -807,14 +805,22 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
       if (j * RPB < L) // wave-uniform
         score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kpre[j]);
     }
-  for (int l0 = PRE * RPB; l0 < L; l0 += RPB)
+  // the rest of the context, PRE sweeps at a time: unconditional loads from
+  // clamped rows, all of a round in flight together (one load per iteration
+  // would cost a trip to memory per sweep)
+  for (int l0 = PRE * RPB; l0 < L; l0 += PRE * RPB)
     {
-      const int l = l0 + grp;
-      uint4 kv = make_uint4 (0, 0, 0, 0);
-      if (l < L)
-        kv = l == (int)pos ? ((const uint4 *)(qk + HD))[sub]
-                           : ldg4 (kc + (size_t)l * HD + sub * 8);
-      score_row (l, kv);
+      uint4 kv[PRE];
+#pragma unroll
+      for (int j = 0; j < PRE; ++j)
+        kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPB + grp, L - 1) * HD + sub * 8);
+#pragma unroll
+      for (int j = 0; j < PRE; ++j)
+        {
+          const int l = l0 + j * RPB + grp;
+          if (l0 + j * RPB < L) // uniform over the workgroup
+            score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kv[j]);
+        }
     }
   __syncthreads ();
 
@@ -861,9 +867,19 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
       const int l = grp + j * RPB;
       pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vpre[j]);
     }
-  for (int l = grp + PRE * RPB; l < L; l += RPB)
-    pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub]
-                             : ldg4 (vc + (size_t)l * HD + sub * 8));
+  for (int l0 = PRE * RPB; l0 < L; l0 += PRE * RPB)
+    {
+      uint4 vv[PRE];
+#pragma unroll
+      for (int j = 0; j < PRE; ++j)
+        vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPB + grp, L - 1) * HD + sub * 8);
+#pragma unroll
+      for (int j = 0; j < PRE; ++j)
+        {
+          const int l = l0 + j * RPB + grp;
+          pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vv[j]);
+        }
+    }
 #pragma unroll
   for (int j = 0; j < 8; ++j)
     part[grp * HD + sub * 8 + j] = acc[j];
@@ -1324,10 +1340,7 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
         {
           const int l = lb + j * RPS + grp;
           const uint4 kr = l == pos ? knew : kv[j];
-          float sv = dot8_f16 (qv, kr, 0.f);
-#pragma unroll
-          for (int o = LPR >> 1; o > 0; o >>= 1)
-            sv += __shfl_xor (sv, o, 64);
+          float sv = row_sum<LPR> (dot8_f16 (qv, kr, 0.f));
           if (l < l1 && sub == 0)
             {
               const uint16_t h = f2h (sv * scale + 0.f);
