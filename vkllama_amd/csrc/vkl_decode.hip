@@ -383,6 +383,103 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
   __syncthreads ();
 }
 
+// ---- the same without a branch -------------------------------------------------
+// The helpers above put every load under `if (idx * 8 < K)`.  With branches
+// between the first load and the first use of the row the compiler cannot
+// count the loads in flight, and the wait for the row becomes a wait for
+// everything requested so far: the first weight item, on its way from HBM,
+// stands between the row and its normalisation.  Here the number of
+// 4096-element chunks of the row is a compile-time constant XCH, every load is
+// unconditional from a clamped address, and a thread whose chunk lies past K
+// computes and stores a duplicate of the last chunk (same address, same value).
+template <int XCH>
+__device__ __forceinline__ void
+load_row (const uint16_t *src, int K, XRegs &x)
+{
+#pragma unroll
+  for (int j = 0; j < XCH; ++j)
+    {
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
+      x.v[j] = ldg4 (src + idx * 8);
+    }
+}
+
+template <int XCH>
+__device__ __forceinline__ void
+load_norm (const float *w, int K, NormRegs &n)
+{
+#pragma unroll
+  for (int j = 0; j < XCH; ++j)
+    {
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
+      n.w[j][0] = ldg4 (w + idx * 8);
+      n.w[j][1] = ldg4 (w + idx * 8 + 4);
+    }
+}
+
+template <bool NORM, int XCH>
+__device__ __forceinline__ void
+stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
+           float *red, unsigned long long *tr = nullptr)
+{
+  float alpha = 0.f;
+#ifdef VKL_TRACE
+  if (tr && threadIdx.x == 0)
+    {
+      asm volatile("" ::"v"(x.v[0].x), "v"(x.v[XCH - 1].w));
+      tr[1] = wall_clock64 ();
+    }
+#endif
+  if (NORM)
+    {
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < XCH; ++j)
+        {
+          const bool in = (threadIdx.x + j * kDecThreads) * 8 < K;
+          const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            {
+              const float a = in ? h2f ((uint16_t)(w[i] & 0xffff)) : 0.f;
+              const float b = in ? h2f ((uint16_t)(w[i] >> 16)) : 0.f;
+              s += a * a;
+              s += b * b;
+            }
+        }
+      const float total = block_sum (s, red);
+#ifdef VKL_TRACE
+      if (tr && threadIdx.x == 0)
+        tr[3] = wall_clock64 ();
+#endif
+      alpha = 1.0f / sqrtf (total / (float)K + eps);
+    }
+#pragma unroll
+  for (int j = 0; j < XCH; ++j)
+    {
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
+      uint4 o = x.v[j];
+      if (NORM)
+        {
+          const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
+          const uint4 g0 = n.w[j][0], g1 = n.w[j][1];
+          const uint32_t g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
+          uint32_t r[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            {
+              const float a = h2f ((uint16_t)(w[i] & 0xffff));
+              const float b = h2f ((uint16_t)(w[i] >> 16));
+              r[i] = (uint32_t)f2h (a * __uint_as_float (g[2 * i]) * alpha)
+                     | ((uint32_t)f2h (b * __uint_as_float (g[2 * i + 1]) * alpha) << 16);
+            }
+          o = make_uint4 (r[0], r[1], r[2], r[3]);
+        }
+      ((uint4 *)xl)[idx] = o;
+    }
+  __syncthreads ();
+}
+
 // ---------------------------------------------------------------------------
 // projections
 // ---------------------------------------------------------------------------
@@ -433,6 +530,7 @@ struct PipeState
   int mode, N, Kp, nb, nch;
   int lane, wave, wg;
   int u_lo, nit, primed;
+  int U; // units of the whole product
   float best_v;
   uint32_t best_i;
   const uint16_t *residual; // mode 0: fetched with each item, see issue ()
@@ -491,7 +589,7 @@ template <bool COH, int WT = 8> struct Gemv
   static __device__ __forceinline__ void
   begin (PipeState &ps, PipeBuf &A, PipeBuf &B, int mode, const QMat a,
          const QMat b, const QMat c, int N, int K, int wg, int G, int depth,
-         const uint16_t *residual = nullptr)
+         const uint16_t *residual = nullptr, bool always = false)
   {
     ps.mode = mode;
     ps.residual = residual;
@@ -510,12 +608,29 @@ template <bool COH, int WT = 8> struct Gemv
     const int lo = (int)((unsigned)U * (unsigned)wg / (unsigned)G);
     const int hi = (int)((unsigned)U * (unsigned)(wg + 1) / (unsigned)G);
     ps.u_lo = lo + ps.wave;
+    ps.U = U;
     const int nunits
         = ps.u_lo < hi ? (hi - ps.u_lo + kDecWaves - 1) / kDecWaves : 0;
     ps.nit = nunits * ps.nch;
     ps.best_v = -INFINITY, ps.best_i = 0xffffffffu;
     ps.primed = 0;
-    prime (ps, A, B, depth);
+    if (always)
+      {
+        // the first item without a condition around its loads: the waits
+        // that follow in the caller can then be counted exactly
+        if (depth >= 1)
+          {
+            issue (ps, A, 0);
+            ps.primed = 1;
+          }
+        if (depth >= 2)
+          {
+            issue (ps, B, 1);
+            ps.primed = 2;
+          }
+      }
+    else
+      prime (ps, A, B, depth);
   }
 
   // issues the first `depth` (<= 2) items if they are not in flight yet
@@ -538,7 +653,9 @@ template <bool COH, int WT = 8> struct Gemv
   issue (const PipeState &ps, PipeBuf &b, int it)
   {
     const int ui = it / ps.nch, c = it - ui * ps.nch;
-    const int u = ps.u_lo + ui * kDecWaves;
+    // (a wave without units still requests the last unit's first item when
+    // begin () is told to issue unconditionally; it is never consumed)
+    const int u = min (ps.u_lo + ui * kDecWaves, ps.U - 1);
     const uint8_t *q[R];
     const uint16_t *d[R];
     rows_of (ps, u, q, d);
@@ -552,11 +669,21 @@ template <bool COH, int WT = 8> struct Gemv
     // does not start a dependent trip to memory at the end of the row.
     const uint16_t *rp = ps.residual ? ps.residual : (const uint16_t *)ps.m0.q;
     b.res = ld_u32<COH> ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
+    // an item past the wave's last (requested all the same when begin ()
+    // issues unconditionally) reads one and the same KiB for every load, so
+    // that it adds nothing to the traffic
+    const bool none = it >= ps.nit;
+    if (none)
+      {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          q[r] = ps.m0.q, d[r] = ps.m0.d;
+      }
 #pragma unroll
     for (int s = 0; s < S; ++s)
       {
         const int kk = c * CHUNK + s * (VKL_WAVE * 16) + ps.lane * 16;
-        const int kc = kk < ps.Kp ? kk : 0;
+        const int kc = none ? ps.lane * 16 : (kk < ps.Kp ? kk : 0);
 #pragma unroll
         for (int r = 0; r < R; ++r)
           {
@@ -1244,6 +1371,118 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
 }
 
 // ---------------------------------------------------------------------------
+// the projection phases of the launch-per-phase mode, without a branch between
+// the first load and the staged row (see load_row): row, norm weights, first
+// weight item, then normalisation and staging, then the weight pipeline.
+// Layer 0's K/Q/V phase, which starts from the embedding table, keeps the
+// general form above.
+// ---------------------------------------------------------------------------
+template <int WT, int XCH>
+__device__ __forceinline__ void
+run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
+                  int phase, int wg, int G, uint8_t *lds)
+{
+  typedef Gemv<false, WT> GV;
+  const vkl_decode_model &m = p.m;
+  const int dim = m.dim, ffn = m.ffn;
+  uint16_t *xl = (uint16_t *)lds;
+  const int kstage = phase == PH_DOWN || phase == PH_GEMV ? ffn : dim;
+  float *red = (float *)(lds + (size_t)kstage * 2); // 2*kDecWaves words
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
+  VKL_TR (0);
+  switch (phase)
+    {
+    case PH_KQV:
+      {
+        const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
+                   wv = wmat<WT> (lw.wv, dim, dim);
+        load_row<XCH> (p.s.x, dim, x);
+        load_norm<XCH> (lw.attn_norm, dim, nw);
+        // keep the scheduler from moving the row / norm loads behind the weight
+        // loads: waiting for them would then wait for the weights as well
+        __builtin_amdgcn_sched_barrier (0);
+        GV::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1, nullptr, true);
+        stage_row<true, XCH> (x, dim, xl, nw, m.eps, red, VKL_TRP);
+        VKL_TR (2);
+        e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
+        break;
+      }
+    case PH_WO:
+      {
+        const QMat w = wmat<WT> (lw.wo, dim, dim);
+        load_row<XCH> (p.s.att, dim, x);
+        // keep the scheduler from moving the row / norm loads behind the weight
+        // loads: waiting for them would then wait for the weights as well
+        __builtin_amdgcn_sched_barrier (0);
+        GV::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x, true);
+        stage_row<false, XCH> (x, dim, xl, nw, 0.f, red, VKL_TRP);
+        VKL_TR (2);
+        e.y[0] = p.s.x, e.residual = p.s.x;
+        break;
+      }
+    case PH_UPGATE:
+      {
+        const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
+        load_row<XCH> (p.s.x, dim, x);
+        load_norm<XCH> (lw.ffn_norm, dim, nw);
+        // keep the scheduler from moving the row / norm loads behind the weight
+        // loads: waiting for them would then wait for the weights as well
+        __builtin_amdgcn_sched_barrier (0);
+        GV::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true);
+        stage_row<true, XCH> (x, dim, xl, nw, m.eps, red, VKL_TRP);
+        VKL_TR (2);
+        e.y[0] = p.s.t;
+        break;
+      }
+    case PH_DOWN:
+    case PH_GEMV:
+      {
+        const uint16_t *res = phase == PH_DOWN ? p.s.x : p.gemv_res;
+        const QMat w = wmat<WT> (lw.w_down, dim, ffn);
+        load_row<XCH> (p.s.t, ffn, x);
+        // keep the scheduler from moving the row / norm loads behind the weight
+        // loads: waiting for them would then wait for the weights as well
+        __builtin_amdgcn_sched_barrier (0);
+        GV::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, res, true);
+        stage_row<false, XCH> (x, ffn, xl, nw, 0.f, red, VKL_TRP);
+        VKL_TR (2);
+        e.y[0] = p.s.x, e.residual = res;
+        break;
+      }
+    default: // PH_HEAD
+      {
+        const QMat w = wmat<WT> (m.output, m.vocab, dim);
+        load_row<XCH> (p.s.x, dim, x);
+        load_norm<XCH> (m.output_norm, dim, nw);
+        // keep the scheduler from moving the row / norm loads behind the weight
+        // loads: waiting for them would then wait for the weights as well
+        __builtin_amdgcn_sched_barrier (0);
+        GV::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1, nullptr, true);
+        stage_row<true, XCH> (x, dim, xl, nw, m.final_eps, red, VKL_TRP);
+        VKL_TR (2);
+        e.y[0] = p.s.logits16, e.y32 = p.logits32;
+        e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
+        break;
+      }
+    }
+  GV::run (ps, A, B, xl, e, red);
+  VKL_TR (4);
+}
+
+template <int PHASE, int WT, int XCH>
+__global__ __launch_bounds__ (kDecThreads) void
+decode_phase_direct_kernel (const Params p, const vkl_layer_weights lw, int layer,
+                            int G)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  run_phase_direct<WT, XCH> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
+}
+
+// ---------------------------------------------------------------------------
 // long contexts: attention split over chunks of the context
 // ---------------------------------------------------------------------------
 // One workgroup per head walks the cache row by row, which at several thousand
@@ -1842,10 +2081,17 @@ timer_collect (hipStream_t s)
 }
 
 template <int PHASE, int WT>
+int launch_direct (const Params &p, const vkl_layer_weights &lw, int layer,
+                   int grid, int G, size_t lds, hipStream_t s);
+
+template <int PHASE, int WT>
 int
 launch_phase_wt (const Params &p, const vkl_layer_weights &lw, int layer,
                  int grid, int G, size_t lds, hipStream_t s)
 {
+  if (PHASE == PH_WO || PHASE == PH_UPGATE || PHASE == PH_DOWN || PHASE == PH_HEAD
+      || PHASE == PH_GEMV || (PHASE == PH_KQV && layer > 0))
+    return launch_direct<PHASE, WT> (p, lw, layer, grid, G, lds, s);
   static size_t lds_set = 0;
   if (lds > lds_set)
     {
@@ -1858,6 +2104,45 @@ launch_phase_wt (const Params &p, const vkl_layer_weights &lw, int layer,
       <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
                                                                  G);
   return 0;
+}
+
+// the branch-free form of a projection phase; XCH = 4096-element chunks of
+// the staged row
+template <int PHASE, int WT, int XCH>
+int
+launch_direct_xch (const Params &p, const vkl_layer_weights &lw, int layer,
+                   int grid, int G, size_t lds, hipStream_t s)
+{
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute (
+          (const void *)decode_phase_direct_kernel<PHASE, WT, XCH>,
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  decode_phase_direct_kernel<PHASE, WT, XCH>
+      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G);
+  return 0;
+}
+
+template <int PHASE, int WT>
+int
+launch_direct (const Params &p, const vkl_layer_weights &lw, int layer,
+               int grid, int G, size_t lds, hipStream_t s)
+{
+  const int kstage = PHASE == PH_DOWN || PHASE == PH_GEMV ? p.m.ffn : p.m.dim;
+  switch ((kstage + 4095) / 4096)
+    {
+    case 1:
+      return launch_direct_xch<PHASE, WT, 1> (p, lw, layer, grid, G, lds, s);
+    case 2:
+      return launch_direct_xch<PHASE, WT, 2> (p, lw, layer, grid, G, lds, s);
+    case 3:
+      return launch_direct_xch<PHASE, WT, 3> (p, lw, layer, grid, G, lds, s);
+    default:
+      return launch_direct_xch<PHASE, WT, 4> (p, lw, layer, grid, G, lds, s);
+    }
 }
 
 template <int PHASE>
