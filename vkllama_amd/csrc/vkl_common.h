@@ -64,6 +64,15 @@ ldg4 (const void *p)
   return make_uint4 (v.x, v.y, v.z, v.w);
 }
 
+// The same for data read once (a weight stream): the non-temporal hint keeps it
+// from displacing what the caches hold for re-use.
+__device__ __forceinline__ uint4
+ldg4_stream (const void *p)
+{
+  const vkl_u32x4 v = __builtin_nontemporal_load ((const VKL_GLOBAL vkl_u32x4 *)p);
+  return make_uint4 (v.x, v.y, v.z, v.w);
+}
+
 // Cross-lane data movement by DPP (a modifier of a VALU instruction, a few
 // cycles) instead of ds_bpermute (a trip through the LDS crossbar that also
 // counts against the LDS counter): v of the lane chosen by CTRL within the
