@@ -67,7 +67,7 @@ def test_embedding_f16_bit_exact(dev, rng):
 
 
 # ----------------------------------------------------------------- RMSNorm --
-@pytest.mark.parametrize("rows,W", [(1, 4096), (16, 512), (3, 1000), (2, 5120)])
+@pytest.mark.parametrize("rows,W", [(1, 4096), (16, 512), (3, 1000), (2, 5120), (33, 4096), (2, 1004), (3, 8200), (2, 8192)])
 def test_rmsnorm(dev, rng, rows, W):
     x = (rng.standard_normal((rows, W)) * 2).astype(np.float16)
     w = rng.uniform(0.5, 1.5, W).astype(np.float32)

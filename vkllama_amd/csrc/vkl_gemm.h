@@ -33,8 +33,12 @@ struct GemmArgs
   float *y32;               // dense [M, N] widened copy
 };
 
-// smallest M for which the GEMM beats re-streaming the weights per 4 rows
-constexpr int kGemmMinRows = 9;
+// smallest M for which the matrix-core kernels beat one weight-streaming pass
+// per token row (measured on the 7B shapes): Q8_0 weights, fp16 weights, and
+// batched fp16 products (one small matrix per head)
+constexpr int kGemmMinRows = 2;
+constexpr int kGemmMinRowsF16 = 3;
+constexpr int kGemmMinRowsBatched = 9;
 
 // true if the shapes/alignments are ones the kernel covers
 bool gemm_mfma_supported (const GemmArgs &a);

@@ -179,7 +179,7 @@ vkl_matmul_f16_tb (const void *a, const void *b, int C, int M, int N, int K,
   p.C = C, p.M = M, p.N = N, p.K = K;
   p.acs = acs, p.ahs = ahs, p.bcs = bcs, p.bhs = bhs, p.ycs = ycs, p.yhs = yhs;
   p.scale = scale, p.bias = bias, p.act = act;
-  if (M >= vkl::kGemmMinRows)
+  if (M >= (C > 1 ? vkl::kGemmMinRowsBatched : vkl::kGemmMinRowsF16))
     {
       // many rows (a projection, or the scores of a prompt pass): matrix cores
       vkl::GemmArgs g = {};
@@ -213,7 +213,7 @@ vkl_ffn_upgate_f16 (const void *x, const void *wup, const void *wgate, int M,
   p.acs = 0, p.ahs = (size_t)K, p.bcs = 0, p.bhs = (size_t)K;
   p.ycs = 0, p.yhs = (size_t)N;
   p.scale = 1.f, p.bias = 0.f, p.act = 0;
-  if (M >= vkl::kGemmMinRows)
+  if (M >= vkl::kGemmMinRowsF16)
     {
       vkl::GemmArgs g = {};
       g.x = p.a, g.xs = (size_t)K;
@@ -247,7 +247,7 @@ vkl_matmul_f16_nn (const void *a, const void *b, int C, int M, int N, int K,
   p.C = C, p.M = M, p.N = N, p.K = K;
   p.acs = acs, p.ahs = ahs, p.bcs = bcs, p.bhs = bhs, p.ycs = ycs, p.yhs = yhs;
   p.scale = scale, p.bias = bias, p.act = act;
-  if (M >= vkl::kGemmMinRows)
+  if (M >= (C > 1 ? vkl::kGemmMinRowsBatched : vkl::kGemmMinRowsF16))
     {
       vkl::GemmArgs g = {};
       g.batch = C, g.xbs = acs, g.wbs = bcs, g.ybs = ycs;

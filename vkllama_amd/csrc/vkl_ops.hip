@@ -8,9 +8,10 @@
 namespace
 {
 // ---- RMSNorm: one workgroup (256 threads) per row ---------------------------
+// general form: any row width, the row is read twice
 __global__ __launch_bounds__ (256) void
-rmsnorm_kernel (const uint16_t *__restrict__ x, const float *__restrict__ w,
-                int W, float eps, uint16_t *__restrict__ out)
+rmsnorm_generic_kernel (const uint16_t *__restrict__ x, const float *__restrict__ w,
+                        int W, float eps, uint16_t *__restrict__ out)
 {
   __shared__ float part[4];
   const uint16_t *xr = x + (size_t)blockIdx.x * W;
@@ -31,6 +32,69 @@ rmsnorm_kernel (const uint16_t *__restrict__ x, const float *__restrict__ w,
     {
       const float v = vkl::h2f (xr[i]);
       o[i] = vkl::f2h (v * w[i] * alpha);
+    }
+}
+
+// rows of W = 8 * n values, n <= 256 * VEC: the row stays in registers between
+// the sum of squares and the scaling, and row and weights are requested at
+// once (16-byte loads from clamped addresses, no branch around a load)
+template <int VEC>
+__global__ __launch_bounds__ (256) void
+rmsnorm_kernel (const uint16_t *__restrict__ x, const float *__restrict__ w,
+                int W, float eps, uint16_t *__restrict__ out)
+{
+  __shared__ float part[4];
+  const uint16_t *xr = x + (size_t)blockIdx.x * W;
+  uint16_t *o = out + (size_t)blockIdx.x * W;
+  const int nv = W >> 3;
+  uint4 v[VEC], g[VEC][2];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j)
+    v[j] = vkl::ldg4 (xr + (size_t)min ((int)threadIdx.x + j * 256, nv - 1) * 8);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j)
+    {
+      const float *wp = w + (size_t)min ((int)threadIdx.x + j * 256, nv - 1) * 8;
+      g[j][0] = vkl::ldg4 (wp), g[j][1] = vkl::ldg4 (wp + 4);
+    }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j)
+    {
+      const uint32_t h[4] = { v[j].x, v[j].y, v[j].z, v[j].w };
+      float t = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        {
+          const float a = vkl::h2f ((uint16_t)(h[i] & 0xffff)), b = vkl::h2f ((uint16_t)(h[i] >> 16));
+          t += a * a;
+          t += b * b;
+        }
+      s += (int)threadIdx.x + j * 256 < nv ? t : 0.f;
+    }
+  s = vkl::wave_sum (s);
+  if ((threadIdx.x & 63) == 0)
+    part[threadIdx.x >> 6] = s;
+  __syncthreads ();
+  const float total = (part[0] + part[1]) + (part[2] + part[3]);
+  const float alpha = 1.0f / sqrtf (total / (float)W + eps);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j)
+    {
+      const int idx = (int)threadIdx.x + j * 256;
+      const uint32_t h[4] = { v[j].x, v[j].y, v[j].z, v[j].w };
+      const uint32_t gw[8] = { g[j][0].x, g[j][0].y, g[j][0].z, g[j][0].w,
+                               g[j][1].x, g[j][1].y, g[j][1].z, g[j][1].w };
+      uint32_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        {
+          const float a = vkl::h2f ((uint16_t)(h[i] & 0xffff)), b = vkl::h2f ((uint16_t)(h[i] >> 16));
+          r[i] = (uint32_t)vkl::f2h (a * __uint_as_float (gw[2 * i]) * alpha)
+                 | ((uint32_t)vkl::f2h (b * __uint_as_float (gw[2 * i + 1]) * alpha) << 16);
+        }
+      if (idx < nv)
+        *(uint4 *)(o + (size_t)idx * 8) = make_uint4 (r[0], r[1], r[2], r[3]);
     }
 }
 
@@ -303,9 +367,19 @@ vkl_rmsnorm_f16 (const void *x, const float *w, int rows, int W, float eps,
                  void *out, void *stream)
 {
   VKL_CHECK_ARG (x && w && out && rows > 0 && W > 0);
-  rmsnorm_kernel<<<dim3 ((unsigned)rows), dim3 (256), 0,
-                   (hipStream_t)stream>>> ((const uint16_t *)x, w, W, eps,
-                                           (uint16_t *)out);
+  const hipStream_t s = (hipStream_t)stream;
+  const uint16_t *xp = (const uint16_t *)x;
+  uint16_t *op = (uint16_t *)out;
+  const bool aligned = (W % 8) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0
+                       && ((uintptr_t)w % 16) == 0;
+  if (aligned && W <= 2048)
+    rmsnorm_kernel<1><<<dim3 ((unsigned)rows), dim3 (256), 0, s>>> (xp, w, W, eps, op);
+  else if (aligned && W <= 4096)
+    rmsnorm_kernel<2><<<dim3 ((unsigned)rows), dim3 (256), 0, s>>> (xp, w, W, eps, op);
+  else if (aligned && W <= 8192)
+    rmsnorm_kernel<4><<<dim3 ((unsigned)rows), dim3 (256), 0, s>>> (xp, w, W, eps, op);
+  else
+    rmsnorm_generic_kernel<<<dim3 ((unsigned)rows), dim3 (256), 0, s>>> (xp, w, W, eps, op);
   return vkl_launch_status ();
 }
 
