@@ -127,7 +127,7 @@ def bench_single_matmul(args):
         "config": {"workload": args.workload, "M": 1, "N": N, "K": K, "ring": ring},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "decode_phase_kernel<gemv> (the decode step's weight-streaming kernel, stand-alone)",
+                     "kernel": "decode_phase_direct_kernel<7, 8, %d, false> (the decode step's weight-streaming kernel, stand-alone)" % min(4, (K + 4095) // 4096),
                      "avg_launch_us": round(ms * 1e3, 3), "launches_timed": steps, "bytes_per_launch": nbytes,
                      "cache_resident_avg_launch_us": round(ms_hot * 1e3, 3),
                      "cache_resident_gbs": round(nbytes / (ms_hot * 1e-3) / 1e9, 1)},
@@ -227,7 +227,22 @@ def main():
         m.phase_replay(dom, L_mid - 1, 1)
         dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
         dom_bytes = per_phase[dom]["bytes_per_launch"]
-        dom_kernel, dom_pair_us = "decode_phase_kernel<%s>" % dom, per_phase[dom]["avg_us"]
+        # the kernel's name as a profiler prints it: phase number, weight type,
+        # 4096-value chunks of the staged activation row
+        phase_no = {"kqv": 0, "attention": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5}[dom]
+        kstage = cfg["ffn"] if dom == "down" else cfg["dim"]
+        if dom == "attention":
+            dom_kernel = "decode_phase_kernel<1, %d> (attention)" % (8 if cfg["wtype"] == 8 else 1)
+        else:
+            # last argument: weights of a step beyond what the caches hold are
+            # requested with the non-temporal hint (same rule as the library's)
+            per = 34.0 / 32.0 if cfg["wtype"] == 8 else 2.0
+            wbytes = (cfg["n_layers"] * (4.0 * cfg["dim"] ** 2 + 3.0 * cfg["dim"] * cfg["ffn"])
+                      + cfg["vocab"] * cfg["dim"]) * per
+            dom_kernel = "decode_phase_direct_kernel<%d, %d, %d, %s> (%s)" % (
+                phase_no, 8 if cfg["wtype"] == 8 else 1, min(4, (kstage + 4095) // 4096),
+                "true" if wbytes > (288 << 20) else "false", dom)
+        dom_pair_us = per_phase[dom]["avg_us"]
     else:
         # persistent / overlapped modes: one launch (or one overlapped train of
         # launches) per token, priced as a whole

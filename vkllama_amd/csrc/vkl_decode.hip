@@ -95,6 +95,7 @@ struct Params
   const uint32_t *loop; // {index into ids, position}, or null
   uint32_t *ids;        // loop: input token ids[index], result to ids[index + 1]
   const uint16_t *gemv_res; // stand-alone product (PH_GEMV): residual operand or null
+  int stream_once; // the weights of a step exceed the caches: request them non-temporally
 #ifdef VKL_TRACE
   unsigned long long *trace; // [phase slot][wg][8] wall-clock stamps
 #endif
@@ -1378,15 +1379,17 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
 // Layer 0's K/Q/V phase, which starts from the embedding table, keeps the
 // general form above.
 // ---------------------------------------------------------------------------
-template <int PHASE, int WT, int XCH>
+template <int PHASE, int WT, int XCH, bool NT>
 __device__ __forceinline__ void
 run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
                   int wg, int G, uint8_t *lds)
 {
-  // The weights stream past once per token: read with the non-temporal hint
-  // they arrive about a tenth faster in the long phases.  The short Wo phase
-  // measured slower with it and keeps plain loads.
-  typedef Gemv<false, WT, PHASE != PH_WO> GV;
+  // NT: the weights stream past once per token and do not fit the caches.
+  // Read with the non-temporal hint they arrive about a tenth faster in the
+  // long phases (the short Wo phase measured slower with it and keeps plain
+  // loads).  Weights that fit the caches must not carry the hint: it would
+  // keep them from staying there for the next token.
+  typedef Gemv<false, WT, NT && PHASE != PH_WO> GV;
   constexpr int phase = PHASE;
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
@@ -1478,13 +1481,13 @@ run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
   VKL_TR (4);
 }
 
-template <int PHASE, int WT, int XCH>
+template <int PHASE, int WT, int XCH, bool NT>
 __global__ __launch_bounds__ (kDecThreads) void
 decode_phase_direct_kernel (const Params p, const vkl_layer_weights lw, int layer,
                             int G)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
-  run_phase_direct<PHASE, WT, XCH> (p, lw, layer, (int)blockIdx.x, G, lds);
+  run_phase_direct<PHASE, WT, XCH, NT> (p, lw, layer, (int)blockIdx.x, G, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -2113,22 +2116,32 @@ launch_phase_wt (const Params &p, const vkl_layer_weights &lw, int layer,
 
 // the branch-free form of a projection phase; XCH = 4096-element chunks of
 // the staged row
-template <int PHASE, int WT, int XCH>
+template <int PHASE, int WT, int XCH, bool NT>
 int
-launch_direct_xch (const Params &p, const vkl_layer_weights &lw, int layer,
-                   int grid, int G, size_t lds, hipStream_t s)
+launch_direct_nt (const Params &p, const vkl_layer_weights &lw, int layer,
+                  int grid, int G, size_t lds, hipStream_t s)
 {
   static size_t lds_set = 0;
   if (lds > lds_set)
     {
       VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_direct_kernel<PHASE, WT, XCH>,
+          (const void *)decode_phase_direct_kernel<PHASE, WT, XCH, NT>,
           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       lds_set = lds;
     }
-  decode_phase_direct_kernel<PHASE, WT, XCH>
+  decode_phase_direct_kernel<PHASE, WT, XCH, NT>
       <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G);
   return 0;
+}
+
+template <int PHASE, int WT, int XCH>
+int
+launch_direct_xch (const Params &p, const vkl_layer_weights &lw, int layer,
+                   int grid, int G, size_t lds, hipStream_t s)
+{
+  return p.stream_once
+             ? launch_direct_nt<PHASE, WT, XCH, true> (p, lw, layer, grid, G, lds, s)
+             : launch_direct_nt<PHASE, WT, XCH, false> (p, lw, layer, grid, G, lds, s);
 }
 
 template <int PHASE, int WT>
@@ -2149,6 +2162,19 @@ launch_direct (const Params &p, const vkl_layer_weights &lw, int layer,
       return launch_direct_xch<PHASE, WT, 4> (p, lw, layer, grid, G, lds, s);
     }
 }
+
+// bytes of weights one decode step reads
+size_t
+step_weight_bytes (const vkl_decode_model &m)
+{
+  const double per = m.wtype == 8 ? 34.0 / 32.0 : 2.0;
+  const double layer = 4.0 * m.dim * m.dim + 3.0 * (double)m.dim * m.ffn;
+  return (size_t)((m.n_layers * layer + (double)m.vocab * m.dim) * per);
+}
+
+// what the memory-side cache and the L2s hold together; a set of weights
+// below this stays resident from one token to the next
+constexpr size_t kCacheResidentBytes = (size_t)288 << 20;
 
 template <int PHASE>
 int
@@ -2416,6 +2442,9 @@ decode_gemv_launch (const void *x, const void *w, int wtype, int N, int K,
   p.s.t = (uint16_t *)x;
   p.s.x = (uint16_t *)y;
   p.gemv_res = (const uint16_t *)residual;
+  // one product cannot know whether its matrix is used again soon; a matrix
+  // that cannot stay cached anyway is streamed
+  p.stream_once = (double)N * K * (wtype == 8 ? 34.0 / 32.0 : 2.0) > (double)kCacheResidentBytes;
   vkl_layer_weights lw = {};
   lw.w_down = w;
   const int G = n_cu * 2;
@@ -2448,7 +2477,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
     }
   const size_t lds
       = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
-  Params p;
+  Params p = {};
   p.m = *m;
   p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
   p.tok = tok;
@@ -2457,6 +2486,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.next_tok = next_tok;
   p.loop = nullptr, p.ids = nullptr;
   p.gemv_res = nullptr;
+  p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
 #ifdef VKL_TRACE
   p.trace = g_trace;
 #endif
@@ -2546,7 +2576,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
                                   dev));
   const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
   hipStream_t s = (hipStream_t)stream;
-  Params p;
+  Params p = {};
   p.m = *m;
   p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
   p.tok = nullptr;
@@ -2555,6 +2585,8 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
   p.loop = p.s.sync + 16;
   p.ids = ids;
   p.wait_target = 0;
+  p.gemv_res = nullptr;
+  p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
 #ifdef VKL_TRACE
   p.trace = nullptr;
 #endif
@@ -2657,7 +2689,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   VKL_HIP (hipDeviceGetAttribute (&n_cu, hipDeviceAttributeMultiprocessorCount,
                                   dev));
   const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
-  Params p;
+  Params p = {};
   p.m = *m;
   p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
   p.tok = (const uint32_t *)p.s.amax_idx; // any device word: ids >= vocab read row 0
@@ -2666,6 +2698,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.next_tok = nullptr;
   p.loop = nullptr, p.ids = nullptr;
   p.gemv_res = nullptr;
+  p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
   p.wait_target = 0;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;
