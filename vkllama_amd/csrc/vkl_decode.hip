@@ -859,8 +859,15 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
 template <int HD, bool COH>
 __device__ __forceinline__ void
 attention_head (const Params &p, const vkl_layer_weights &lw, int head,
-                uint8_t *lds)
+                uint8_t *lds, unsigned long long *tr = nullptr)
 {
+#ifdef VKL_TRACE
+#define VKL_TRA(slot)                                                         \
+  if (tr && threadIdx.x == 0)                                                 \
+    tr[slot] = wall_clock64 ();
+#else
+#define VKL_TRA(slot)
+#endif
   constexpr int LPR = HD / 8;            // lanes per cache row (16 B each)
   constexpr int RPB = kDecThreads / LPR; // cache rows per sweep
   constexpr int PRE = 8;                 // sweeps prefetched up front
@@ -868,9 +875,9 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   const uint32_t pos = step_pos (p);
   const int L = (int)pos + 1;
   uint16_t *qk = (uint16_t *)lds;    // [3*HD]
-  float *sc = (float *)(lds + 1024); // [maxlen]
-  float *part = sc + maxlen;         // [RPB][HD]
-  float *red = part + RPB * HD;      // [2*kDecWaves]
+  float *sc = (float *)(lds + 1024);      // [maxlen]
+  float *part = sc + ((maxlen + 3) & ~3); // [RPB][HD], 16-byte aligned
+  float *red = part + RPB * HD;           // [2*kDecWaves]
   uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
   uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
   const uint16_t *kin = p.s.kqv + head * HD;
@@ -879,53 +886,59 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   const int tid = threadIdx.x;
   const int sub = tid % LPR, grp = tid / LPR;
 
-  // rows written by earlier steps do not depend on this token: fetch the
-  // first sweeps of K and V before anything else
+  // This token's q, k, v and its rotation factors are requested first and
+  // the first sweeps of cached K and V rows right behind them: loads return
+  // in order, so the few bytes the prologue needs are not queued behind the
+  // cache rows.  Every load is unconditional, from a clamped address (a branch
+  // around a load would make the wait below a wait for all of them): threads
+  // without a q/k/v pair repeat pair 0, cache rows past the context repeat the
+  // last row and are ignored where they would be used.
+  const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
+  const bool is_v = tid >= HD && tid < HD + HD / 2;
+  const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
+  const uint32_t inw
+      = ld_u32<COH> ((const uint32_t *)(is_k ? kin : (is_v ? vin : qin)) + pi);
+  const float fc = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
+  const float fs = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
+  // (the scheduler must not move the cache rows ahead of these)
+  __builtin_amdgcn_sched_barrier (0);
   uint4 kpre[PRE], vpre[PRE];
+  const int lastrow = max ((int)pos - 1, 0);
 #pragma unroll
   for (int j = 0; j < PRE; ++j)
-    {
-      const int l = grp + j * RPB;
-      kpre[j] = vpre[j] = make_uint4 (0, 0, 0, 0);
-      if (l < (int)pos)
-        {
-          kpre[j] = ldg4 (kc + (size_t)l * HD + sub * 8);
-          vpre[j] = ldg4 (vc + (size_t)l * HD + sub * 8);
-        }
-    }
+    kpre[j] = ldg4 (kc + (size_t)min (grp + j * RPB, lastrow) * HD + sub * 8);
+#pragma unroll
+  for (int j = 0; j < PRE; ++j)
+    vpre[j] = ldg4 (vc + (size_t)min (grp + j * RPB, lastrow) * HD + sub * 8);
+  __builtin_amdgcn_sched_barrier (0);
 
-  // RoPE on adjacent pairs at position pos; K and V rows go to the cache
-  if (tid < HD) // HD/2 pairs of q, HD/2 pairs of k
-    {
-      const bool is_k = tid >= HD / 2;
-      const int i = is_k ? tid - HD / 2 : tid;
-      const uint32_t v = ld_u32<COH> ((const uint32_t *)(is_k ? kin : qin) + i);
-      const float c = ldg (p.m.freqc + (size_t)pos * (HD / 2) + i);
-      const float s = ldg (p.m.freqs + (size_t)pos * (HD / 2) + i);
-      const float a = h2f ((uint16_t)(v & 0xffff)), b = h2f ((uint16_t)(v >> 16));
-      const uint32_t r = (uint32_t)f2h (a * c - b * s)
-                         | ((uint32_t)f2h (a * s + b * c) << 16);
-      ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + i] = r;
-      if (is_k)
-        stg ((uint32_t *)(kc + (size_t)pos * HD) + i, r);
-    }
-  else if (tid < HD + HD / 2)
-    {
-      const int i = tid - HD;
-      const uint32_t v = ld_u32<COH> ((const uint32_t *)vin + i);
-      stg ((uint32_t *)(vc + (size_t)pos * HD) + i, v);
-      ((uint32_t *)qk)[HD + i] = v;
-    }
+  // RoPE on adjacent pairs at position pos.  The new K and V rows are used
+  // from LDS here; they go to the cache at the end of the head (a store
+  // under a branch at this point would turn the counted waits for the cache
+  // rows into waits for everything in flight).
+  const float ra = h2f ((uint16_t)(inw & 0xffff)), rb = h2f ((uint16_t)(inw >> 16));
+  const uint32_t rot = (uint32_t)f2h (ra * fc - rb * fs)
+                       | ((uint32_t)f2h (ra * fs + rb * fc) << 16);
+  if (is_q || is_k)
+    ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + pi] = rot;
+  if (is_v)
+    ((uint32_t *)qk)[HD + pi] = inw;
   __syncthreads ();
+  VKL_TRA (1);
 
   // scores[l] = fp16(dot(q, K[l]) / sqrt(HD)); LPR lanes share one cache row
   const float scale = 1.0f / sqrtf ((float)HD);
   const uint4 qv = ((const uint4 *)qk)[sub];
+  float mx = -INFINITY; // of the scores this lane has written
   auto score_row = [&] (int l, const uint4 kv) {
     float s = l < L ? dot8_f16 (qv, kv, 0.f) : 0.f;
     s = row_sum<LPR> (s);
     if (l < L && sub == 0)
-      sc[l] = h2f (f2h (s * scale + 0.f));
+      {
+        const float r = h2f (f2h (s * scale + 0.f));
+        sc[l] = r;
+        mx = fmaxf (mx, r);
+      }
   };
 #pragma unroll
   for (int j = 0; j < PRE; ++j)
@@ -951,37 +964,46 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
             score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kv[j]);
         }
     }
-  __syncthreads ();
-
-  // softmax over the L scores; probabilities rounded to fp16
-  float mx = -INFINITY;
-  for (int l = tid; l < L; l += kDecThreads)
-    mx = fmaxf (mx, sc[l]);
+  // the maximum travels with the scores: one barrier covers both
   mx = wave_max (mx);
   if ((tid & 63) == 0)
     red[kDecWaves + (tid >> 6)] = mx;
   __syncthreads ();
+  VKL_TRA (2);
+
+  // softmax over the L scores; probabilities rounded to fp16
   mx = red[kDecWaves];
 #pragma unroll
   for (int w = 1; w < kDecWaves; ++w)
     mx = fmaxf (mx, red[kDecWaves + w]);
-  float sum = 0.f;
-  for (int l = tid; l < L; l += kDecThreads)
+  const float e0 = tid < L ? expf (sc[tid < L ? tid : 0] - mx) : 0.f;
+  float sum = e0;
+  for (int l = tid + kDecThreads; l < L; l += kDecThreads)
     sum += expf (sc[l] - mx);
-  sum = block_sum (sum, red);
-  for (int l = tid; l < L; l += kDecThreads)
+  sum = wave_sum (sum);
+  if ((tid & 63) == 0)
+    red[tid >> 6] = sum;
+  __syncthreads ();
+  sum = 0.f;
+#pragma unroll
+  for (int w = 0; w < kDecWaves; ++w)
+    sum += red[w];
+  if (tid < L)
+    sc[tid] = h2f (f2h (e0 / sum));
+  for (int l = tid + kDecThreads; l < L; l += kDecThreads)
     sc[l] = h2f (f2h (expf (sc[l] - mx) / sum));
   __syncthreads ();
+  VKL_TRA (3);
 
   // out[j] = fp16(sum_l P[l] V[l][j]); thread = (row group, 8 columns)
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j)
     acc[j] = 0.f;
+  // no branch: a row past the context counts with probability 0 (its values
+  // are those of a real row, see the clamped loads)
   auto pv_row = [&] (int l, const uint4 vv) {
-    if (l >= L)
-      return;
-    const float pl = sc[l];
+    const float pl = l < L ? sc[min (l, L - 1)] : 0.f;
     const uint32_t w[4] = { vv.x, vv.y, vv.z, vv.w };
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -994,7 +1016,8 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   for (int j = 0; j < PRE; ++j)
     {
       const int l = grp + j * RPB;
-      pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vpre[j]);
+      if (j * RPB < L) // wave-uniform
+        pv_row (l, l >= (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vpre[j]);
     }
   for (int l0 = PRE * RPB; l0 < L; l0 += PRE * RPB)
     {
@@ -1006,25 +1029,37 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
       for (int j = 0; j < PRE; ++j)
         {
           const int l = l0 + j * RPB + grp;
-          pv_row (l, l == (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vv[j]);
+          if (l0 + j * RPB < L) // uniform over the workgroup
+            pv_row (l, l >= (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vv[j]);
         }
     }
+  ((float4 *)(part + grp * HD + sub * 8))[0] = make_float4 (acc[0], acc[1], acc[2], acc[3]);
+  ((float4 *)(part + grp * HD + sub * 8))[1] = make_float4 (acc[4], acc[5], acc[6], acc[7]);
+  __syncthreads ();
+  VKL_TRA (6);
+  // the RPB partial rows of a column are added by four lanes, a quarter of
+  // the rows each, and those four by DPP; the lane of an even column then
+  // takes the odd neighbour's result and stores the pair
+  {
+    const int c = tid >> 2, k = tid & 3;
+    float o = 0.f;
+    if (c < HD)
+      {
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
-    part[grp * HD + sub * 8 + j] = acc[j];
+        for (int g = 0; g < RPB / 4; ++g)
+          o += part[(k * (RPB / 4) + g) * HD + c];
+      }
+    o = row_sum<4> (o);
+    const float onext = dpp_get<0x104> (o); // row_shl:4: the lane four up
+    if (c < HD && (tid & 7) == 0)
+      st_u32<COH> ((uint32_t *)(p.s.att + head * HD) + (c >> 1),
+                   (uint32_t)f2h (o) | ((uint32_t)f2h (onext) << 16));
+  }
   __syncthreads ();
-  if (tid < HD / 2)
-    {
-      float o0 = 0.f, o1 = 0.f;
-      for (int g = 0; g < RPB; ++g)
-        {
-          o0 += part[g * HD + 2 * tid];
-          o1 += part[g * HD + 2 * tid + 1];
-        }
-      st_u32<COH> ((uint32_t *)(p.s.att + head * HD) + tid,
-                   (uint32_t)f2h (o0) | ((uint32_t)f2h (o1) << 16));
-    }
-  __syncthreads ();
+  if (is_k)
+    stg ((uint32_t *)(kc + (size_t)pos * HD) + pi, rot);
+  if (is_v)
+    stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
 }
 
 __host__ __device__ inline size_t
@@ -1034,7 +1069,7 @@ lds_bytes_needed (int dim, int ffn, int maxlen, int hd)
   // staged activation row + reduction words + parked norm weights
   const size_t stage = ((kmax + 31) / 32 * 32) * 2 + 256 + (size_t)dim * 4;
   const size_t rpb = kDecThreads / (hd / 8);
-  const size_t attn = 1024 + (size_t)maxlen * 4 + rpb * hd * 4 + 256;
+  const size_t attn = 1024 + (size_t)((maxlen + 3) & ~3) * 4 + rpb * hd * 4 + 256;
   return stage > attn ? stage : attn;
 }
 
@@ -1244,9 +1279,9 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         for (int h = wg; h < m.n_heads; h += G)
           {
             if (m.head_dim == 128)
-              attention_head<128, COH> (p, lw, h, lds);
+              attention_head<128, COH> (p, lw, h, lds, VKL_TRP);
             else
-              attention_head<64, COH> (p, lw, h, lds);
+              attention_head<64, COH> (p, lw, h, lds, VKL_TRP);
           }
         break;
       }
