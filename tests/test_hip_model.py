@@ -60,6 +60,24 @@ def test_prefill_then_decode_logits_and_caches(small, fused):
     m.close()
 
 
+def test_decode_from_position_zero_to_the_last_position():
+    """One-token steps from an empty cache (context length 1) up to the last
+    position the cache holds, with a cache length that is not a multiple of 4."""
+    cfg = dict(SMALL, maxlen=26)
+    w = M.synth_weights(cfg, seed=3)
+    m = M.Llama2(cfg, w)
+    m.set_option("fused_decode", 1)
+    om = O.OracleModel(cfg, w)
+    tok = 5
+    for pos in range(cfg["maxlen"]):
+        got = m.forward([tok], pos)
+        want = om.forward([tok], pos)
+        assert logit_err(got, want) < 1e-2, pos
+        assert int(np.argmax(got)) == int(np.argmax(want)), pos
+        tok = int(np.argmax(want))
+    m.close()
+
+
 def test_fused_decode_equals_operator_chain(small):
     cfg, w = small
     prompt = np.array([9, 8, 7, 6], np.uint32)
