@@ -550,10 +550,14 @@ struct PipeState
 // addressed as 2*K bytes, so the 16-byte loads of an item are laid out exactly
 // as for the int8 plane; only the scale load and the dot product differ.
 // NT: the weights are read with the non-temporal hint (a stream read once)
-template <bool COH, int WT = 8, bool NT = false> struct Gemv
+// RU: rows per unit, 2, or 1 (mode 0 only): a product with long rows and few
+// of them then has a unit for every wave and both of its items in flight
+// from the start.  An item is always 8 loads of 16 bytes per lane: RU rows x
+// 8 / RU k-steps of 1024.
+template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
 {
-  static constexpr int R = 2; // rows per unit
-  static constexpr int S = 4; // k-steps of 1024 per item
+  static constexpr int R = RU;     // rows per unit
+  static constexpr int S = 8 / RU; // k-steps of 1024 per item
   static constexpr int CHUNK = S * VKL_WAVE * 16;
 
   static __device__ __forceinline__ void
@@ -561,12 +565,14 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
            const uint16_t *(&d)[R])
   {
     const int Kp = ps.Kp, nb = ps.nb;
-    if (ps.mode == 0)
+    if (R == 1)
+      q[0] = ps.m0.q + (size_t)u * Kp, d[0] = ps.m0.d + (size_t)u * nb;
+    else if (ps.mode == 0)
       {
         const int r0 = 2 * u;
         const int r1 = min (r0 + 1, ps.N - 1);
         q[0] = ps.m0.q + (size_t)r0 * Kp, d[0] = ps.m0.d + (size_t)r0 * nb;
-        q[1] = ps.m0.q + (size_t)r1 * Kp, d[1] = ps.m0.d + (size_t)r1 * nb;
+        q[R - 1] = ps.m0.q + (size_t)r1 * Kp, d[R - 1] = ps.m0.d + (size_t)r1 * nb;
       }
     else if (ps.mode == 1)
       {
@@ -576,13 +582,13 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
         const long long od = (mat == 1 ? ps.dd1 : 0) + (mat == 2 ? ps.dd2 : 0);
         q[0] = ps.m0.q + oq + (size_t)r0 * Kp;
         d[0] = (const uint16_t *)((const uint8_t *)ps.m0.d + od) + (size_t)r0 * nb;
-        q[1] = q[0] + Kp, d[1] = d[0] + nb;
+        q[R - 1] = q[0] + Kp, d[R - 1] = d[0] + nb;
       }
     else
       {
         q[0] = ps.m0.q + (size_t)u * Kp, d[0] = ps.m0.d + (size_t)u * nb;
-        q[1] = ps.m0.q + ps.dq1 + (size_t)u * Kp;
-        d[1] = (const uint16_t *)((const uint8_t *)ps.m0.d + ps.dd1) + (size_t)u * nb;
+        q[R - 1] = ps.m0.q + ps.dq1 + (size_t)u * Kp;
+        d[R - 1] = (const uint16_t *)((const uint8_t *)ps.m0.d + ps.dd1) + (size_t)u * nb;
       }
   }
 
@@ -606,7 +612,7 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
       ps.Kp = K * 2, ps.nb = 0; // row bytes
     ps.nch = (ps.Kp + CHUNK - 1) / CHUNK;
     ps.lane = threadIdx.x & 63, ps.wave = threadIdx.x >> 6, ps.wg = wg;
-    const int U = mode == 0 ? (N + 1) >> 1 : (mode == 1 ? 3 * (N >> 1) : N);
+    const int U = mode == 0 ? (N + R - 1) / R : (mode == 1 ? 3 * (N >> 1) : N);
     const int lo = (int)((unsigned)U * (unsigned)wg / (unsigned)G);
     const int hi = (int)((unsigned)U * (unsigned)(wg + 1) / (unsigned)G);
     ps.u_lo = lo + ps.wave;
@@ -670,7 +676,10 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
     // The residual pair of the unit travels with the item, so the epilogue
     // does not start a dependent trip to memory at the end of the row.
     const uint16_t *rp = ps.residual ? ps.residual : (const uint16_t *)ps.m0.q;
-    b.res = ld_u32<COH> ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
+    if (R == 1)
+      b.res = ldg (rp + u);
+    else
+      b.res = ld_u32<COH> ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
     // an item past the wave's last (requested all the same when begin ()
     // issues unconditionally) reads one and the same KiB for every load, so
     // that it adds nothing to the traffic
@@ -750,6 +759,19 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
     if (ps.lane != 0)
       return;
     const int N = ps.N;
+    if (R == 1)
+      {
+        // one row per unit (mode 0, launch-per-phase kernels only)
+        uint16_t h = f2h (v[0]);
+        if (e.residual)
+          h = f2h (h2f (h) + h2f (ps.residual ? (uint16_t)(res & 0xffff) : ldg (e.residual + u)));
+        stg (e.y[0] + u, h);
+        if (e.y32)
+          stg (e.y32 + u, h2f (h));
+        if (e.amax_val && better (h2f (h), (uint32_t)u, ps.best_v, ps.best_i))
+          ps.best_v = h2f (h), ps.best_i = (uint32_t)u;
+        return;
+      }
     if (ps.mode == 1)
       {
         const int half = N >> 1;
@@ -757,7 +779,7 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
         // the three outputs are N elements apart
         uint16_t *y = e.y[0] + (size_t)mat * N;
         st_u32<COH> ((uint32_t *)(y + r0),
-                     (uint32_t)f2h (v[0]) | ((uint32_t)f2h (v[1]) << 16));
+                     (uint32_t)f2h (v[0]) | ((uint32_t)f2h (v[R - 1]) << 16));
         return;
       }
     if (ps.mode == 2)
@@ -765,14 +787,14 @@ template <bool COH, int WT = 8, bool NT = false> struct Gemv
         // fp16 when kernel boundaries order the phases; one 32-bit word per
         // element where it has to be a write-through atomic
         if (COH)
-          st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[1]) * v[0]));
+          st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[R - 1]) * v[0]));
         else
-          stg (e.y[0] + u, f2h (silu (v[1]) * v[0]));
+          stg (e.y[0] + u, f2h (silu (v[R - 1]) * v[0]));
         return;
       }
     const int r0 = 2 * u;
     const bool two = r0 + 1 < N;
-    uint16_t h0 = f2h (v[0]), h1 = f2h (v[1]);
+    uint16_t h0 = f2h (v[0]), h1 = f2h (v[R - 1]);
     if (e.residual)
       {
         // prefetched with the item unless the phase was begun without it
@@ -1424,7 +1446,11 @@ run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
   // long phases (the short Wo phase measured slower with it and keeps plain
   // loads).  Weights that fit the caches must not carry the hint: it would
   // keep them from staying there for the next token.
-  typedef Gemv<false, WT, NT && PHASE != PH_WO> GV;
+  // Wo, down and the stand-alone product have few rows (two-row units would
+  // leave half of the waves without work): one row per unit there
+  typedef Gemv<false, WT, NT && PHASE != PH_WO,
+               PHASE == PH_DOWN || PHASE == PH_GEMV || PHASE == PH_WO ? 1 : 2>
+      GV;
   constexpr int phase = PHASE;
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
