@@ -952,10 +952,12 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   const float scale = 1.0f / sqrtf ((float)HD);
   const uint4 qv = ((const uint4 *)qk)[sub];
   float mx = -INFINITY; // of the scores this lane has written
-  auto score_row = [&] (int l, const uint4 kv) {
-    float s = l < L ? dot8_f16 (qv, kv, 0.f) : 0.f;
+  // lim: rows below it are scored (the cached rows; the token's own row, which
+  // is in LDS, follows after the sweeps)
+  auto score_row = [&] (int l, int lim, const uint4 kv) {
+    float s = l < lim ? dot8_f16 (qv, kv, 0.f) : 0.f;
     s = row_sum<LPR> (s);
-    if (l < L && sub == 0)
+    if (l < lim && sub == 0)
       {
         const float r = h2f (f2h (s * scale + 0.f));
         sc[l] = r;
@@ -966,26 +968,29 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   for (int j = 0; j < PRE; ++j)
     {
       const int l = grp + j * RPB;
-      if (j * RPB < L) // wave-uniform
-        score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kpre[j]);
+      if (j * RPB < (int)pos) // wave-uniform
+        score_row (l, (int)pos, kpre[j]);
     }
   // the rest of the context, PRE sweeps at a time: unconditional loads from
   // clamped rows, all of a round in flight together (one load per iteration
   // would cost a trip to memory per sweep)
-  for (int l0 = PRE * RPB; l0 < L; l0 += PRE * RPB)
+  for (int l0 = PRE * RPB; l0 < (int)pos; l0 += PRE * RPB)
     {
       uint4 kv[PRE];
 #pragma unroll
       for (int j = 0; j < PRE; ++j)
-        kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPB + grp, L - 1) * HD + sub * 8);
+        kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPB + grp, lastrow) * HD + sub * 8);
 #pragma unroll
       for (int j = 0; j < PRE; ++j)
         {
           const int l = l0 + j * RPB + grp;
-          if (l0 + j * RPB < L) // uniform over the workgroup
-            score_row (l, l == (int)pos ? ((const uint4 *)(qk + HD))[sub] : kv[j]);
+          if (l0 + j * RPB < (int)pos) // uniform over the workgroup
+            score_row (l, (int)pos, kv[j]);
         }
     }
+  // the token's own row: every group forms it (no lane sits out of the
+  // cross-lane sum), group 0 records it
+  score_row (grp == 0 ? (int)pos : L, L, ((const uint4 *)(qk + HD))[sub]);
   // the maximum travels with the scores: one barrier covers both
   mx = wave_max (mx);
   if ((tid & 63) == 0)
@@ -1024,37 +1029,43 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
     acc[j] = 0.f;
   // no branch: a row past the context counts with probability 0 (its values
   // are those of a real row, see the clamped loads)
-  auto pv_row = [&] (int l, const uint4 vv) {
-    const float pl = l < L ? sc[min (l, L - 1)] : 0.f;
+  // (p and v are fp16 values: their product is exact in fp32, so the fused
+  // multiply-add rounds as a multiplication and an addition would)
+  auto pv_add = [&] (float pl, const uint4 vv) {
     const uint32_t w[4] = { vv.x, vv.y, vv.z, vv.w };
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       {
-        acc[2 * j] += pl * h2f ((uint16_t)(w[j] & 0xffff));
-        acc[2 * j + 1] += pl * h2f ((uint16_t)(w[j] >> 16));
+        acc[2 * j] = __builtin_fmaf (pl, h2f ((uint16_t)(w[j] & 0xffff)), acc[2 * j]);
+        acc[2 * j + 1] = __builtin_fmaf (pl, h2f ((uint16_t)(w[j] >> 16)), acc[2 * j + 1]);
       }
+  };
+  auto pv_row = [&] (int l, const uint4 vv) {
+    pv_add (l < (int)pos ? sc[min (l, lastrow)] : 0.f, vv);
   };
 #pragma unroll
   for (int j = 0; j < PRE; ++j)
     {
       const int l = grp + j * RPB;
-      if (j * RPB < L) // wave-uniform
-        pv_row (l, l >= (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vpre[j]);
+      if (j * RPB < (int)pos) // wave-uniform
+        pv_row (l, vpre[j]);
     }
-  for (int l0 = PRE * RPB; l0 < L; l0 += PRE * RPB)
+  for (int l0 = PRE * RPB; l0 < (int)pos; l0 += PRE * RPB)
     {
       uint4 vv[PRE];
 #pragma unroll
       for (int j = 0; j < PRE; ++j)
-        vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPB + grp, L - 1) * HD + sub * 8);
+        vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPB + grp, lastrow) * HD + sub * 8);
 #pragma unroll
       for (int j = 0; j < PRE; ++j)
         {
           const int l = l0 + j * RPB + grp;
-          if (l0 + j * RPB < L) // uniform over the workgroup
-            pv_row (l, l >= (int)pos ? ((const uint4 *)(qk + 2 * HD))[sub] : vv[j]);
+          if (l0 + j * RPB < (int)pos) // uniform over the workgroup
+            pv_row (l, vv[j]);
         }
     }
+  // the token's own row (from LDS) is the last of its group's rows
+  pv_add (grp == (int)pos % RPB ? sc[pos] : 0.f, ((const uint4 *)(qk + 2 * HD))[sub]);
   ((float4 *)(part + grp * HD + sub * 8))[0] = make_float4 (acc[0], acc[1], acc[2], acc[3]);
   ((float4 *)(part + grp * HD + sub * 8))[1] = make_float4 (acc[4], acc[5], acc[6], acc[7]);
   __syncthreads ();
