@@ -51,6 +51,7 @@ constexpr int kAttnChunks = 32;      // upper bound on chunks per head
 constexpr int kAttnSplitMinLen = 544; // shorter contexts use one workgroup per head (measured
                                       // break-even of the two forms at 7B: 540 positions)
 constexpr int kAttnSweeps = 8;        // sweeps of cache rows a chunk kernel keeps in flight
+constexpr int kAttnChunkRows = 1024;  // most rows of a chunk (longer contexts use one workgroup per head)
 
 __host__ __device__ inline size_t
 align256 (size_t v)
@@ -1712,33 +1713,45 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
         stg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid, 0.f);
       return;
     }
-  // One lane per chunk fetches that chunk's maximum and sum; the V rows and
-  // scores of the first sweeps are requested right behind them (unconditional,
-  // clamped rows), and travel while M and S are formed.
+  // One lane per chunk fetches that chunk's maximum and sum; the chunk's
+  // scores (one row per thread and round) and the V rows of the first sweeps
+  // are requested right behind them (unconditional, clamped rows), and travel
+  // while M and S are formed.
+  constexpr int RL = kAttnChunkRows / kAttnThreads; // score rounds per thread
+  __shared__ float pls[kAttnChunkRows];             // probabilities of the chunk
   const int ci = tid & 31; // kAttnChunks <= 32
   const float mi = ldg (p.s.part_max + head * kAttnChunks + min (ci, C - 1));
   const float si = ldg (p.s.part_sum + head * kAttnChunks + min (ci, C - 1));
+  uint16_t sh[RL];
+#pragma unroll
+  for (int k = 0; k < RL; ++k)
+    sh[k] = ldg (sc16 + min (l0 + tid + k * kAttnThreads, l1 - 1));
   uint4 vv[UN];
-  uint16_t sh[UN];
 #pragma unroll
   for (int j = 0; j < UN; ++j)
-    {
-      const int lc = min (l0 + j * RPS + grp, l1 - 1);
-      vv[j] = ldg4 (vc + (size_t)lc * HD + sub * 8);
-      sh[j] = ldg (sc16 + lc);
-    }
-  float M = ci < C ? mi : -INFINITY;
-#pragma unroll
-  for (int o = 16; o > 0; o >>= 1)
-    M = fmaxf (M, __shfl_xor (M, o, 64));
+    vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPS + grp, l1 - 1) * HD + sub * 8);
+  // lanes 0..31 (and their copies 32..63) hold the chunks: the maximum over a
+  // row of 16 by DPP, the two rows through scalar registers
+  float M = row_max<16> (ci < C ? mi : -INFINITY);
+  M = fmaxf (lane_value (M, 0), lane_value (M, 16));
   // chunks in index order, as a sequential loop would add them
   float S = 0.f;
-  for (int i = 0; i < C; ++i)
+#pragma unroll
+  for (int i = 0; i < kAttnChunks; ++i)
     {
-      const float m_i = __shfl (mi, i, 64), s_i = __shfl (si, i, 64);
-      if (m_i > -INFINITY)
+      const float m_i = lane_value (mi, i), s_i = lane_value (si, i);
+      if (i < C && m_i > -INFINITY)
         S += s_i * expf (m_i - M);
     }
+  // every probability is formed once (not by each of the LPR lanes of its row)
+#pragma unroll
+  for (int k = 0; k < RL; ++k)
+    {
+      const int r = tid + k * kAttnThreads;
+      if (l0 + r < l1)
+        pls[r] = h2f (f2h (expf (h2f (sh[k]) - M) / S));
+    }
+  __syncthreads ();
 
   float acc[8];
 #pragma unroll
@@ -1750,25 +1763,24 @@ attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
         {
 #pragma unroll
           for (int j = 0; j < UN; ++j)
-            {
-              const int lc = min (lb + j * RPS + grp, l1 - 1);
-              vv[j] = ldg4 (vc + (size_t)lc * HD + sub * 8);
-              sh[j] = ldg (sc16 + lc);
-            }
+            vv[j] = ldg4 (vc + (size_t)min (lb + j * RPS + grp, l1 - 1) * HD + sub * 8);
         }
 #pragma unroll
       for (int j = 0; j < UN; ++j)
         {
           const int l = lb + j * RPS + grp;
-          if (l >= l1)
+          if (lb + j * RPS >= l1) // uniform over the workgroup
             continue;
-          const float pl = h2f (f2h (expf (h2f (sh[j]) - M) / S));
+          // a row past the chunk counts with probability 0 (its values are
+          // those of the chunk's last row); p and v are fp16 values, so the
+          // fused multiply-add rounds as multiplication and addition would
+          const float pl = l < l1 ? pls[min (l, l1 - 1) - l0] : 0.f;
           const uint32_t w[4] = { vv[j].x, vv[j].y, vv[j].z, vv[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             {
-              acc[2 * i] += pl * h2f ((uint16_t)(w[i] & 0xffff));
-              acc[2 * i + 1] += pl * h2f ((uint16_t)(w[i] >> 16));
+              acc[2 * i] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] & 0xffff)), acc[2 * i]);
+              acc[2 * i + 1] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] >> 16)), acc[2 * i + 1]);
             }
         }
     }
@@ -2281,6 +2293,8 @@ launch_attention (const Params &p, const vkl_decode_model *m,
   C = std::max (C, (L + rows_in_flight - 1) / rows_in_flight);
   C = C < 1 ? 1 : (C > kAttnChunks ? kAttnChunks : C);
   const int R = (L + C - 1) / C;
+  if (R > kAttnChunkRows) // (contexts beyond 32768 positions)
+    return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
   const size_t lds_a = 1024 + 64 + (size_t)R * 4;
   VKL_CHECK_ARG (lds_a <= 64 * 1024);
   if (int e = timer_mark (PH_ATTN, false, s))
