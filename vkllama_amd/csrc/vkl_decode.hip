@@ -1610,66 +1610,66 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
         }
       return;
     }
-  // The first sweeps of K are requested before anything else, so that they
-  // travel while q is rotated: unconditional loads from clamped rows (a load
-  // under a branch would make every later wait a wait for all loads); rows
-  // past the chunk are ignored below, the row of the new position, which this
-  // kernel is writing at the same time, is replaced by the rotated k.
+  // The token's q and k pairs and their rotation factors are requested first,
+  // the first sweeps of K right behind them: loads return in order, so the
+  // few bytes that the rotation needs do not queue behind the cache rows, and
+  // the rotation runs while those travel.  All loads are unconditional, from
+  // clamped addresses (a load under a branch would make every later wait a
+  // wait for all loads): threads without a pair repeat pair 0, rows past the
+  // chunk repeat its last cached row and are ignored below.  The row of the
+  // new position is not read from the cache (this kernel writes it): it is
+  // scored from LDS after the sweeps.
+  const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
+  const bool is_v = tid >= HD && tid < HD + HD / 2;
+  const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
+  const uint16_t *src = p.s.kqv + (is_k ? 0 : (is_v ? 2 * dim : dim)) + head * HD;
+  const uint32_t inw = ldg ((const uint32_t *)src + pi);
+  const float cs = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
+  const float sn = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
+  __builtin_amdgcn_sched_barrier (0);
+  // cached rows of the chunk: [l0, lc1)
+  const int lc1 = has_new ? pos : l1;
+  const int lastrow = max (lc1 - 1, 0);
   uint4 kv[UN];
 #pragma unroll
   for (int j = 0; j < UN; ++j)
-    kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPS + grp, l1 - 1) * HD + sub * 8);
+    kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPS + grp, lastrow) * HD + sub * 8);
+  __builtin_amdgcn_sched_barrier (0);
 
-  if (tid < HD && (tid < HD / 2 || has_new))
-    {
-      const bool is_k = tid >= HD / 2;
-      const int i = is_k ? tid - HD / 2 : tid;
-      const uint16_t *src = p.s.kqv + (is_k ? 0 : dim) + head * HD;
-      const uint32_t v = ldg ((const uint32_t *)src + i);
-      const float cs = ldg (p.m.freqc + (size_t)pos * (HD / 2) + i);
-      const float sn = ldg (p.m.freqs + (size_t)pos * (HD / 2) + i);
-      const float a = h2f ((uint16_t)(v & 0xffff)), b = h2f ((uint16_t)(v >> 16));
-      const uint32_t r = (uint32_t)f2h (a * cs - b * sn)
-                         | ((uint32_t)f2h (a * sn + b * cs) << 16);
-      ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + i] = r;
-      if (is_k)
-        stg ((uint32_t *)(kc + (size_t)pos * HD) + i, r);
-    }
-  else if (has_new && tid >= HD && tid < HD + HD / 2)
-    {
-      const int i = tid - HD;
-      stg ((uint32_t *)(vc + (size_t)pos * HD) + i,
-           ldg ((const uint32_t *)(p.s.kqv + 2 * dim + head * HD) + i));
-    }
+  const float ra = h2f ((uint16_t)(inw & 0xffff)), rb = h2f ((uint16_t)(inw >> 16));
+  const uint32_t rot = (uint32_t)f2h (ra * cs - rb * sn)
+                       | ((uint32_t)f2h (ra * sn + rb * cs) << 16);
+  if (is_q || is_k)
+    ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + pi] = rot;
   __syncthreads ();
 
   const float scale = 1.0f / sqrtf ((float)HD);
   const uint4 qv = ((const uint4 *)qk)[sub];
   float mx = -INFINITY;
-  const uint4 knew = ((const uint4 *)(qk + HD))[sub];
-  for (int lb = l0; lb < l1; lb += UN * RPS)
+  auto score_row = [&] (int l, int lim, const uint4 kr) {
+    const float sv = row_sum<LPR> (dot8_f16 (qv, kr, 0.f));
+    if (l < lim && sub == 0)
+      {
+        const float r = h2f (f2h (sv * scale + 0.f));
+        sc[l - l0] = r;
+        mx = fmaxf (mx, r);
+      }
+  };
+  for (int lb = l0; lb < lc1; lb += UN * RPS)
     {
       if (lb > l0)
         {
 #pragma unroll
           for (int j = 0; j < UN; ++j)
-            kv[j] = ldg4 (kc + (size_t)min (lb + j * RPS + grp, l1 - 1) * HD + sub * 8);
+            kv[j] = ldg4 (kc + (size_t)min (lb + j * RPS + grp, lastrow) * HD + sub * 8);
         }
 #pragma unroll
       for (int j = 0; j < UN; ++j)
-        {
-          const int l = lb + j * RPS + grp;
-          const uint4 kr = l == pos ? knew : kv[j];
-          float sv = row_sum<LPR> (dot8_f16 (qv, kr, 0.f));
-          if (l < l1 && sub == 0)
-            {
-              const uint16_t h = f2h (sv * scale + 0.f);
-              stg (p.s.sc16 + (size_t)head * maxlen + l, h);
-              sc[l - l0] = h2f (h);
-              mx = fmaxf (mx, h2f (h));
-            }
-        }
+        if (lb + j * RPS < lc1) // uniform over the workgroup
+          score_row (lb + j * RPS + grp, lc1, kv[j]);
     }
+  if (has_new) // uniform over the workgroup: every row group forms it, group 0 records it
+    score_row (grp == 0 ? pos : l1, l1, ((const uint4 *)(qk + HD))[sub]);
   mx = wave_max (mx);
   if ((tid & 63) == 0)
     red[tid >> 6] = mx;
@@ -1689,6 +1689,14 @@ attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
       stg (p.s.part_sum + head * kAttnChunks + c,
            red[4] + red[5] + red[6] + red[7]);
     }
+  // the chunk's fp16 scores for the values kernel (sc holds fp16 values), and
+  // the new K and V rows of the cache
+  for (int l = l0 + tid; l < l1; l += kAttnThreads)
+    stg (p.s.sc16 + (size_t)head * maxlen + l, f2h (sc[l - l0]));
+  if (has_new && is_k)
+    stg ((uint32_t *)(kc + (size_t)pos * HD) + pi, rot);
+  if (has_new && is_v)
+    stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
 }
 
 template <int HD>
