@@ -203,13 +203,13 @@ def test_other_decode_modes_match_oracle(cfg, seed, mode):
 
 @pytest.mark.parametrize("heads", [4, 2])
 def test_long_context_decode_uses_split_attention(heads):
-    """Past 544 positions the decode step splits each head's context over
+    """From 1024 positions on the decode step splits each head's context over
     several workgroups (scores / values / combine launches); logits, greedy ids
     and the cache rows written on the way must still match the oracle."""
-    cfg = dict(dim=256, n_layers=2, n_heads=heads, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
+    cfg = dict(dim=256, n_layers=2, n_heads=heads, ffn=352, vocab=640, maxlen=1280, eps=1e-5, wtype=8)
     w = M.synth_weights(cfg, seed=21)
     rng = np.random.default_rng(21)
-    prompt = rng.integers(3, cfg["vocab"], 800).astype(np.uint32)
+    prompt = rng.integers(3, cfg["vocab"], 1100).astype(np.uint32)
     m = M.Llama2(cfg, w)
     om = O.OracleModel(cfg, w)
     assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
@@ -221,20 +221,20 @@ def test_long_context_decode_uses_split_attention(heads):
         pos += 1
     for layer in range(cfg["n_layers"]):
         for value in (0, 1):
-            g = m.read_kv_cache(layer, value)[:, 800:pos].astype(np.float32)
-            o = (om.vcache(layer) if value else om.kcache(layer))[:, 800:pos].astype(np.float32)
+            g = m.read_kv_cache(layer, value)[:, 1100:pos].astype(np.float32)
+            o = (om.vcache(layer) if value else om.kcache(layer))[:, 1100:pos].astype(np.float32)
             assert np.abs(g - o).max() <= 1e-2 * max(np.abs(o).max(), 1e-3), (layer, value)
     m.close()
 
 
-@pytest.mark.parametrize("n_prompt,n_gen", [(4, 40), (536, 24), (760, 24)])
+@pytest.mark.parametrize("n_prompt,n_gen", [(4, 40), (1016, 24), (1100, 24)])
 def test_graph_replayed_loop_equals_stepwise_and_oracle(n_prompt, n_gen):
     """generate_greedy replays one captured step per token (token index and
     position advance in device memory); the ids must equal those of the
     step-by-step launches and the oracle's, also across the switch of the
-    attention phase to its split form at 544 positions, and on a second use
+    attention phase to its split form at 1024 positions, and on a second use
     of the cached graphs."""
-    cfg = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=1024, eps=1e-5, wtype=8)
+    cfg = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=1280, eps=1e-5, wtype=8)
     w = M.synth_weights(cfg, seed=33)
     rng = np.random.default_rng(33)
     prompt = rng.integers(3, cfg["vocab"], n_prompt).astype(np.uint32)

@@ -48,8 +48,8 @@ struct Scratch
 };
 
 constexpr int kAttnChunks = 32;      // upper bound on chunks per head
-constexpr int kAttnSplitMinLen = 544; // shorter contexts use one workgroup per head (measured
-                                      // break-even of the two forms at 7B: 540 positions)
+constexpr int kAttnSplitMinLen = 1024; // shorter contexts use one workgroup per head (measured at 7B:
+                                       // 10.5 against 12.4 us at 768 positions, 12.6 / 12.5 at 1024)
 constexpr int kAttnSweeps = 8;        // sweeps of cache rows a chunk kernel keeps in flight
 constexpr int kAttnChunkRows = 1024;  // most rows of a chunk (longer contexts use one workgroup per head)
 
