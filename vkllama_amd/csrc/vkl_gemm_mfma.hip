@@ -31,19 +31,24 @@ typedef _Float16 half8 __attribute__ ((ext_vector_type (8)));
 typedef float float16v __attribute__ ((ext_vector_type (16)));
 
 constexpr int BN = 128;
-// k extent of a step.  Q8_0: one block, so that the block scale applies to a
-// whole step.  fp16 weights: 64, so that the eight 16-byte chunks of a tile
-// row are one full 128-byte cache line (with 32, every request is half a
-// line and the L2 delivers half the bytes per cycle).
+// k extent of a step: 64.  For fp16 operands the eight 16-byte chunks of a
+// tile row are then one full 128-byte cache line (with 32, every request is
+// half a line and the L2 delivers half the bytes per cycle); for Q8_0 a step
+// holds two blocks, each with its own scale (one block per step measured
+// slower: half the products per barrier).
 template <int WT> struct Geo
 {
-  static constexpr int BK = WT == 8 ? 32 : 64;
+  static constexpr int BK = 64;
   static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
-  static constexpr int LDK = BK + 8;  // LDS row stride in halves: 80 or 144
-                                      // bytes, conflict-free 16-byte accesses
-  static constexpr int NB = WT == 8 ? 1 : BN * CPR / 256; // weight chunks per thread
+  static constexpr int LDK = BK + 8;  // LDS row stride in halves: 144 bytes,
+                                      // conflict-free 16-byte accesses
+  static constexpr int NB = WT == 8 ? 2 : BN * CPR / 256; // weight chunks per thread
 };
 constexpr int kGemmThreads = 256;
+// fewer full-height tiles than this: half-height tiles; workgroups a launch
+// should have at least (two per compute unit): else the k range is split too
+constexpr int kGemmFewTiles = 384;
+constexpr int kGemmSplitTarget = 512;
 // k-tiles in flight in registers: more for the small-M configuration, where
 // few workgroups run and each has to hide the memory latency alone
 template <int BM> struct GemmDepth
@@ -73,8 +78,8 @@ struct TileLoads
   static constexpr int ACH = BM * Geo<WT>::CPR / kGemmThreads; // 16-byte chunks of x per thread
   static constexpr int NB = Geo<WT>::NB;
   uint4 a[ACH];
-  uint4 b[NB]; // fp16: weight chunks; Q8_0: b[0] = 16 quants
-  uint16_t bd; // Q8_0 block scale
+  uint4 b[NB]; // fp16: weight chunks; Q8_0: the 32 quants of one block
+  uint16_t bd; // Q8_0: its scale
 };
 
 // Per-thread source addresses of the tile loads.  They depend on k only
@@ -90,8 +95,9 @@ struct TileAddr
   static constexpr int NB = Geo<WT>::NB;
   const uint16_t *a[ACH]; // x chunk at k = 0, or null beyond M
   int ak[ACH];            // its column offset within a k-step
-  const uint8_t *bq;      // Q8_0: quants of this thread's row at k = 0
-  const uint16_t *bd;     // Q8_0: its scales
+  const uint8_t *bq;      // Q8_0: quants of this thread's row and block (0 or 1 of a step) at k = 0
+  const uint16_t *bd;     // Q8_0: that block's scale
+  int bko;                // Q8_0: 0 or 32, the block's offset within a step
   const uint16_t *b[NB];  // fp16: chunk pointers at k = 0
   int bk[NB];             // fp16 [N, K]: column offset; [K, N]: row offset
 };
@@ -117,21 +123,22 @@ tile_addresses (const GemmArgs &a, size_t xoff, size_t woff, int zmat, int m0,
       ta.ak[i] = (c % CPR) * 8;
       ta.a[i] = m < a.M ? a.x + xoff + (size_t)m * a.xs + ta.ak[i] : nullptr;
     }
-  ta.bq = nullptr, ta.bd = nullptr;
+  ta.bq = nullptr, ta.bd = nullptr, ta.bko = 0;
 #pragma unroll
   for (int i = 0; i < NB; ++i)
     ta.b[i] = nullptr, ta.bk[i] = 0;
   if (WT == 8)
     {
-      const int v = tid >> 1, seg = tid & 1;
+      const int v = tid >> 1, blk = tid & 1;
       const int mat = a.upgate ? (v >> 6) : zmat;
       const int n = a.upgate ? n0 + (v & 63) : n0 + v;
+      ta.bko = blk * 32;
       if (n < a.N)
         {
           ta.bq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat)
-                  + (size_t)n * a.Kp + seg * 16;
+                  + (size_t)n * a.Kp + blk * 32;
           ta.bd = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat)
-                  + (size_t)n * (a.Kp >> 5);
+                  + (size_t)n * (a.Kp >> 5) + blk;
         }
     }
   else if (WT == 2)
@@ -185,9 +192,10 @@ issue_tile (const GemmArgs &a, const TileAddr<BM, WT> &ta, int k0,
     }
   if (WT == 8)
     {
-      // rows beyond N: zero quants and a zero scale
-      const bool v = ta.bq != nullptr;
+      // rows beyond N, blocks beyond K: zero quants and a zero scale
+      const bool v = ta.bq != nullptr && k0 + ta.bko < a.Kp;
       t.b[0] = ldg16 (v ? (const void *)(ta.bq + k0) : zeros);
+      t.b[1] = ldg16 (v ? (const void *)(ta.bq + k0 + 16) : zeros);
       t.bd = ldg (v ? ta.bd + (k0 >> 5) : (const uint16_t *)zeros);
     }
   else
@@ -218,22 +226,23 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
     }
   if (WT == 8)
     {
-      const int v = tid >> 1, seg = tid & 1;
-      if (seg == 0)
-        Ds[v] = t.bd;
-      const uint32_t w[4] = { t.b[0].x, t.b[0].y, t.b[0].z, t.b[0].w };
-      uint32_t o[8];
+      const int v = tid >> 1, blk = tid & 1;
+      Ds[v * 2 + blk] = t.bd;
+      const uint32_t w[8] = { t.b[0].x, t.b[0].y, t.b[0].z, t.b[0].w,
+                              t.b[1].x, t.b[1].y, t.b[1].z, t.b[1].w };
+      uint32_t o[16];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 8; ++j)
         {
           h16x2 lo, hi;
           i8x4_to_h2x2 (w[j], lo, hi);
           o[2 * j] = __builtin_bit_cast (uint32_t, lo);
           o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
         }
-      uint4 *dst = (uint4 *)(Bs + v * LDK + seg * 16);
-      dst[0] = make_uint4 (o[0], o[1], o[2], o[3]);
-      dst[1] = make_uint4 (o[4], o[5], o[6], o[7]);
+      uint4 *dst = (uint4 *)(Bs + v * LDK + blk * 32);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        dst[j] = make_uint4 (o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
     }
   else if (WT == 2)
     {
@@ -266,7 +275,7 @@ store_tile (const TileLoads<BM, WT> &t, uint16_t *As, uint16_t *Bs,
 
 template <int BM, int WT>
 __device__ __forceinline__ void
-gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
+gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kbase, int kt, int nk,
            const uint16_t *Ac, const uint16_t *Bc, const uint16_t *Dc,
            uint16_t *An, uint16_t *Bn, uint16_t *Dn, TileLoads<BM, WT> &tn,
            float16v (&acc)[BM / 64][2], int wm, int vb0, int vb1)
@@ -288,22 +297,29 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
     }
   if (WT == 8)
     {
-      const float sc[2] = { h2f (Dc[vb0 + (lane & 31)]), h2f (Dc[vb1 + (lane & 31)]) };
+      // the two blocks of the step in turn: block sum from a zero
+      // accumulator, times the block's scale
+      const uint32_t d0 = *(const uint32_t *)(Dc + (vb0 + (lane & 31)) * 2);
+      const uint32_t d1 = *(const uint32_t *)(Dc + (vb1 + (lane & 31)) * 2);
+      const float sc[2][2] = { { h2f ((uint16_t)(d0 & 0xffff)), h2f ((uint16_t)(d1 & 0xffff)) },
+                               { h2f ((uint16_t)(d0 >> 16)), h2f ((uint16_t)(d1 >> 16)) } };
 #pragma unroll
-      for (int mi = 0; mi < TM; ++mi)
+      for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-          {
-            float16v part;
+        for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              part[r] = 0.f;
-            part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[0][mi], bf[0][ni], part, 0, 0, 0);
-            part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[1][mi], bf[1][ni], part, 0, 0, 0);
+          for (int ni = 0; ni < 2; ++ni)
+            {
+              float16v part;
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              acc[mi][ni][r] += part[r] * sc[ni];
-          }
+              for (int r = 0; r < 16; ++r)
+                part[r] = 0.f;
+              part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[2 * blk][mi], bf[2 * blk][ni], part, 0, 0, 0);
+              part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[2 * blk + 1][mi], bf[2 * blk + 1][ni], part, 0, 0, 0);
+#pragma unroll
+              for (int r = 0; r < 16; ++r)
+                acc[mi][ni][r] += part[r] * sc[blk][ni];
+            }
     }
   else
     {
@@ -317,14 +333,15 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kt, int nk,
                 af[ks][mi], bf[ks][ni], acc[mi][ni], 0, 0, 0);
     }
   store_tile<BM, WT> (tn, An, Bn, Dn);
-  const int knext = min (kt + 1 + D, nk - 1);
+  const int knext = kbase + min (kt + 1 + D, nk - 1);
   issue_tile<BM, WT> (a, ta, knext * BK, tn);
   __syncthreads ();
 }
 
 template <int BM, int WT>
 __global__ __launch_bounds__ (kGemmThreads, 2) void
-gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
+gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd,
+                  int ksplit, float *ws)
 {
   // element offsets of this problem of the batch (the argument block itself
   // stays untouched in constant memory: it is indexed by a run-time matrix
@@ -335,14 +352,18 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
   constexpr int BK = Geo<WT>::BK, LDK = Geo<WT>::LDK;
   __shared__ __align__ (16) uint16_t As[2][BM * LDK];
   __shared__ __align__ (16) uint16_t Bs[2][BN * LDK];
-  __shared__ uint16_t Ds[2][BN]; // Q8_0 block scales of the tile rows
+  __shared__ __align__ (4) uint16_t Ds[2][BN * 2]; // Q8_0: the two block scales of every tile row
 
   // XCD-aware tile numbering
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int tile = xcd * per_xcd + j;
-  if (j >= per_xcd || tile >= tiles_m * tiles_n)
+  if (j >= per_xcd || tile >= tiles_m * tiles_n * ksplit)
     return;
-  const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
+  // ksplit > 1: the k range is divided among ksplit workgroups per output
+  // tile; each writes its fp32 partial tile to the workspace and a second
+  // kernel adds the parts in order and applies the epilogue
+  const int ks = tile / (tiles_m * tiles_n), t2 = tile - ks * (tiles_m * tiles_n);
+  const int tn = t2 / tiles_m, tm = t2 - tn * tiles_m;
   const int bn_rows = a.upgate ? 64 : BN; // weight rows per matrix and tile
   const int m0 = tm * BM, n0 = tn * bn_rows;
   const int zmat = blockIdx.z;
@@ -362,7 +383,9 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
       for (int r = 0; r < 16; ++r)
         acc[mi][ni][r] = 0.f;
 
-  const int nk = (a.wtype == 8 ? a.Kp : ((a.K + BK - 1) / BK) * BK) / BK;
+  const int nk_all = ((a.wtype == 8 ? a.Kp : a.K) + BK - 1) / BK;
+  const int kbase = (int)((long)nk_all * ks / ksplit);
+  const int nk = (int)((long)nk_all * (ks + 1) / ksplit) - kbase; // k steps of this workgroup
   // D tiles are in flight in registers (tile k + 1 .. k + D while tile k is
   // being multiplied out of LDS): a k-step costs far less time than a trip to
   // memory, so one tile of look-ahead would leave every step waiting
@@ -370,14 +393,14 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
   TileAddr<BM, WT> ta;
   tile_addresses<BM, WT> (a, xoff, woff, zmat, m0, n0, ta);
   TileLoads<BM, WT> t[D];
-  issue_tile<BM, WT> (a, ta, 0, t[0]);
+  issue_tile<BM, WT> (a, ta, kbase * BK, t[0]);
   store_tile<BM, WT> (t[0], As[0], Bs[0], Ds[0]);
-  issue_tile<BM, WT> (a, ta, min (1, nk - 1) * BK, t[1 % D]);
-  issue_tile<BM, WT> (a, ta, min (2, nk - 1) * BK, t[2 % D]);
+  issue_tile<BM, WT> (a, ta, (kbase + min (1, nk - 1)) * BK, t[1 % D]);
+  issue_tile<BM, WT> (a, ta, (kbase + min (2, nk - 1)) * BK, t[2 % D]);
   if (D > 2)
     {
-      issue_tile<BM, WT> (a, ta, min (3, nk - 1) * BK, t[3]);
-      issue_tile<BM, WT> (a, ta, min (4, nk - 1) * BK, t[0]);
+      issue_tile<BM, WT> (a, ta, (kbase + min (3, nk - 1)) * BK, t[3]);
+      issue_tile<BM, WT> (a, ta, (kbase + min (4, nk - 1)) * BK, t[0]);
     }
   __syncthreads ();
 
@@ -387,7 +410,7 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
   // unconditional (past the end they repeat the last tile, which nothing
   // reads), so the waits in the unrolled body count loads exactly.
 #define VKL_GEMM_STEP(d)                                                      \
-  gemm_step<BM, WT> (a, ta, kt0 + (d), nk, As[(d) & 1], Bs[(d) & 1],        \
+  gemm_step<BM, WT> (a, ta, kbase, kt0 + (d), nk, As[(d) & 1], Bs[(d) & 1], \
                      Ds[(d) & 1], As[((d) & 1) ^ 1], Bs[((d) & 1) ^ 1],      \
                      Ds[((d) & 1) ^ 1], t[((d) + 1) % D], acc, wm, vb0, vb1)
   int kt0 = 0;
@@ -411,6 +434,30 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd)
 
   // epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) +
   // r%4, column l%32 of its 32x32 block
+  if (ksplit > 1)
+    {
+      // partial tile: matrix t of the launch (up = 0 and gate = 1 for the
+      // fused pair), k part ks, dense [M, N] fp32
+#pragma unroll
+      for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          {
+            const int m = m0 + wm * (BM / 2) + mi * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (m >= a.M)
+              continue;
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+              {
+                const int n = a.upgate ? n0 + wn * 32 + (lane & 31)
+                                       : n0 + wn * 64 + ni * 32 + (lane & 31);
+                const int t = a.upgate ? ni : zmat;
+                if (n < a.N)
+                  ws[((size_t)(t * ksplit + ks) * a.M + m) * a.N + n] = acc[mi][ni][r];
+              }
+          }
+      return;
+    }
   uint16_t *y = a.y[a.upgate ? 0 : zmat] + yoff;
   const uint16_t *res = a.residual ? a.residual + yoff : nullptr;
   float *y32 = a.y32 ? a.y32 + bi * (size_t)a.M * a.N : nullptr;
@@ -805,7 +852,7 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
 
 // sum over the slices in order, then the epilogue of the product
 __global__ __launch_bounds__ (256) void
-skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S)
+skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S, int mrows)
 {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= (size_t)a.M * a.N)
@@ -815,7 +862,7 @@ skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S)
   float v[3] = { 0.f, 0.f, 0.f };
   for (int t = 0; t < nm; ++t)
     for (int sl = 0; sl < S; ++sl)
-      v[t] += ldg (ws + ((size_t)(t * S + sl) * 32 + m) * a.N + n);
+      v[t] += ldg (ws + ((size_t)(t * S + sl) * mrows + m) * a.N + n);
   const size_t o = (size_t)m * a.ys + n;
   if (a.upgate)
     {
@@ -887,7 +934,7 @@ launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
   gemm_skinny2_kernel<WT><<<dim3 ((unsigned)((a.N + 31) / 32), (unsigned)S, (unsigned)nm),
                            dim3 (kSk2Waves * 64), lds, s>>> (a, ws, S);
   const size_t total = (size_t)a.M * a.N;
-  skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S);
+  skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S, 32);
   err = (int)hipGetLastError ();
   return true;
 }
@@ -924,12 +971,37 @@ launch_cfg (const GemmArgs &a, hipStream_t s)
 {
   const int tiles_m = (a.M + BM - 1) / BM;
   const int tiles_n = (a.N + (a.upgate ? 64 : BN) - 1) / (a.upgate ? 64 : BN);
-  const int tiles = tiles_m * tiles_n;
+  // Too few output tiles to occupy the compute units (a few hundred token
+  // rows against a 4096-row matrix): the k range is split as well, into parts
+  // of at least eight steps, as far as the fp32 workspace holds the partial
+  // tiles.  Not for batched products (there are tiles enough).
+  const int nz = a.upgate ? 1 : a.nmat, nm = a.upgate ? 2 : a.nmat;
+  const int nk = ((a.wtype == 8 ? a.Kp : a.K) + Geo<WT>::BK - 1) / Geo<WT>::BK;
+  int ksplit = 1;
+  float *ws = nullptr;
+  if (a.batch <= 1 && WT != 2)
+    {
+      // (measured on the 7B shapes: a split in two pays for Q8_0 weights, whose
+      // steps are slower, and not for fp16 weights)
+      const int want = kGemmSplitTarget / (tiles_m * tiles_n * nz);
+      ksplit = want < (WT == 8 ? 2 : 3) ? 1 : std::max (1, std::min (std::min (want, 8), nk / 8));
+      while (ksplit > 1 && (size_t)nm * ksplit * a.M * a.N * sizeof (float) > kSk2Workspace)
+        --ksplit;
+      if (ksplit > 1 && !(ws = skinny2_workspace (s)))
+        ksplit = 1;
+    }
+  const int tiles = tiles_m * tiles_n * ksplit;
   const int per_xcd = (tiles + 7) / 8;
   gemm_mfma_kernel<BM, WT>
       <<<dim3 ((unsigned)(per_xcd * 8), (unsigned)(a.batch > 1 ? a.batch : 1),
-               (unsigned)(a.upgate ? 1 : a.nmat)),
-         dim3 (kGemmThreads), 0, s>>> (a, tiles_m, tiles_n, per_xcd);
+               (unsigned)nz),
+         dim3 (kGemmThreads), 0, s>>> (a, tiles_m, tiles_n, per_xcd, ksplit, ws);
+  if (ksplit > 1)
+    {
+      const size_t total = (size_t)a.M * a.N;
+      skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (
+          a, ws, ksplit, a.M);
+    }
   return (int)hipGetLastError ();
 }
 } // namespace
@@ -967,10 +1039,18 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
 {
   if (!gemm_mfma_supported (a))
     return (int)hipErrorInvalidValue;
-  const bool small = a.M <= 64;
+  bool small = a.M <= 64;
   // few rows, one problem, no batch: the weight-streaming form
   if (small && a.batch <= 1 && a.wtype != 2 && (a.wtype == 8 || (a.K % 16) == 0))
     return a.wtype == 8 ? launch_skinny<8> (a, s) : launch_skinny<1> (a, s);
+  // the half-height tile also where full tiles would be too few to occupy the
+  // compute units (a few hundred token rows)
+  {
+    const long tiles = (long)((a.M + 127) / 128) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
+                       * (a.batch > 1 ? a.batch : 1) * (a.upgate ? 1 : a.nmat);
+    if (tiles < kGemmFewTiles)
+      small = true;
+  }
   if (a.wtype == 8)
     return small ? launch_cfg<64, 8> (a, s) : launch_cfg<128, 8> (a, s);
   if (a.wtype == 2)
