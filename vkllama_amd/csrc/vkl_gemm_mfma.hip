@@ -504,218 +504,18 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd,
 }
 
 // ---------------------------------------------------------------------------
-// few token rows (M <= 64): one workgroup per 32 weight rows, K split over
-// its four waves
+// few token rows (M <= 32): weight-streaming form, K split over workgroups
 // ---------------------------------------------------------------------------
-// With so few rows the product is bound by streaming the weights, and a
-// 128-row tile would leave most compute units idle.  Here a workgroup owns 32
-// weight rows (N/32 workgroups), each of its 8 or 16 waves a slice of K;
-// fragments go from
-// global memory straight into the MFMA operand registers (a lane's 16
-// consecutive k values feed two MFMAs; the x operand uses the same k
-// assignment, and a sum over k does not care which lane holds which k), four
-// blocks in flight per wave.  The four partial tiles are added through LDS.
-// Q8_0 keeps the exact arithmetic of the big kernel: block sum from a zero
-// accumulator, times the block scale in fp32.
-template <int WT, int TM, bool UPGATE, int NW>
-__global__ __launch_bounds__ (NW * 64) void
-gemm_skinny_kernel (const GemmArgs a)
-{
-  constexpr int NB = UPGATE ? 2 : 1; // weight matrices per workgroup
-  constexpr int UN = 4;              // 32-wide k blocks in flight
-  __shared__ float red[NW][NB][TM * 32][33];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * 32, zmat = UPGATE ? 0 : (int)blockIdx.z;
-  const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
-  const int g = lane >> 5;
-  const int nblk = (WT == 8 ? a.Kp : ((a.K + 31) / 32) * 32) / 32;
-  const int per = (nblk + NW - 1) / NW;
-  const int b0 = wave * per, b1 = min (nblk, b0 + per);
-
-  const uint8_t *wq[NB];
-  const uint16_t *wd[NB];
-  const uint16_t *wh[NB];
-#pragma unroll
-  for (int t = 0; t < NB; ++t)
-    {
-      const int mat = UPGATE ? t : zmat;
-      wq[t] = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat) + (size_t)nrow * a.Kp;
-      wd[t] = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat) + (size_t)nrow * (a.Kp >> 5);
-      wh[t] = (const uint16_t *)pick3 (a.wh[0], a.wh[1], a.wh[2], mat) + (size_t)nrow * a.ws;
-    }
-  const uint16_t *xr[TM];
-#pragma unroll
-  for (int mi = 0; mi < TM; ++mi)
-    xr[mi] = a.x + (size_t)min (mi * 32 + (lane & 31), a.M - 1) * a.xs;
-
-  float16v acc[NB][TM];
-#pragma unroll
-  for (int t = 0; t < NB; ++t)
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[t][mi][r] = 0.f;
-
-  for (int bb = b0; bb < b1; bb += UN)
-    {
-      uint4 wv[UN][NB][2]; // Q8_0 uses [0] (16 quants); fp16 both (2 x 8 halves)
-      uint16_t dv[UN][NB];
-      uint4 xv[UN][TM][2];
-#pragma unroll
-      for (int u = 0; u < UN; ++u)
-        {
-          const int b = min (bb + u, b1 - 1); // repeats the last block; masked below
-          const int k = b * 32 + g * 16;
-#pragma unroll
-          for (int t = 0; t < NB; ++t)
-            {
-              if (WT == 8)
-                {
-                  wv[u][t][0] = ldg16 (wq[t] + k);
-                  dv[u][t] = ldg (wd[t] + b);
-                }
-              else
-                {
-                  // columns past K (a partial last block) read the row's
-                  // start instead and are zeroed on the x side
-                  const int kc = k + 16 <= a.K ? k : 0;
-                  wv[u][t][0] = ldg16 (wh[t] + kc);
-                  wv[u][t][1] = ldg16 (wh[t] + kc + 8);
-                }
-            }
-#pragma unroll
-          for (int mi = 0; mi < TM; ++mi)
-            {
-              const bool in = k + 16 <= a.K;
-              const int kc = in ? k : 0;
-              xv[u][mi][0] = keep_if (in || k < a.K, ldg16 (xr[mi] + (k + 8 <= a.K ? k : 0)));
-              xv[u][mi][1] = keep_if (in, ldg16 (xr[mi] + kc + 8));
-            }
-        }
-#pragma unroll
-      for (int u = 0; u < UN; ++u)
-        {
-          if (bb + u >= b1)
-            continue;
-          half8 af[TM][2];
-#pragma unroll
-          for (int mi = 0; mi < TM; ++mi)
-            {
-              af[mi][0] = __builtin_bit_cast (half8, xv[u][mi][0]);
-              af[mi][1] = __builtin_bit_cast (half8, xv[u][mi][1]);
-            }
-#pragma unroll
-          for (int t = 0; t < NB; ++t)
-            {
-              half8 bf[2];
-              if (WT == 8)
-                {
-                  const uint32_t w[4] = { wv[u][t][0].x, wv[u][t][0].y, wv[u][t][0].z, wv[u][t][0].w };
-                  uint32_t o[8];
-#pragma unroll
-                  for (int j = 0; j < 4; ++j)
-                    {
-                      h16x2 lo, hi;
-                      i8x4_to_h2x2 (w[j], lo, hi);
-                      o[2 * j] = __builtin_bit_cast (uint32_t, lo);
-                      o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
-                    }
-                  bf[0] = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
-                  bf[1] = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
-                }
-              else
-                {
-                  bf[0] = __builtin_bit_cast (half8, wv[u][t][0]);
-                  bf[1] = __builtin_bit_cast (half8, wv[u][t][1]);
-                }
-#pragma unroll
-              for (int mi = 0; mi < TM; ++mi)
-                {
-                  // operands: A = x (rows = tokens), B = weights (columns = rows n)
-                  if (WT == 8)
-                    {
-                      float16v part;
-#pragma unroll
-                      for (int r = 0; r < 16; ++r)
-                        part[r] = 0.f;
-                      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[mi][0], bf[0], part, 0, 0, 0);
-                      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[mi][1], bf[1], part, 0, 0, 0);
-                      const float sc = h2f (dv[u][t]);
-#pragma unroll
-                      for (int r = 0; r < 16; ++r)
-                        acc[t][mi][r] += part[r] * sc;
-                    }
-                  else
-                    {
-                      acc[t][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[mi][0], bf[0], acc[t][mi], 0, 0, 0);
-                      acc[t][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[mi][1], bf[1], acc[t][mi], 0, 0, 0);
-                    }
-                }
-            }
-        }
-    }
-
-  // add the NW parts of K
-#pragma unroll
-  for (int t = 0; t < NB; ++t)
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        red[wave][t][mi * 32 + (r >> 2) * 8 + g * 4 + (r & 3)][lane & 31] = acc[t][mi][r];
-  __syncthreads ();
-  uint16_t *y = a.y[UPGATE ? 0 : zmat];
-  for (int i = threadIdx.x; i < TM * 32 * 32; i += NW * 64)
-    {
-      const int m = i >> 5, nn = i & 31, n = n0 + nn;
-      if (m >= a.M || n >= a.N)
-        continue;
-      float v[NB];
-#pragma unroll
-      for (int t = 0; t < NB; ++t)
-        {
-          v[t] = 0.f;
-#pragma unroll
-          for (int w = 0; w < NW; ++w)
-            v[t] += red[w][t][m][nn];
-        }
-      const size_t o = (size_t)m * a.ys + n;
-      if (UPGATE)
-        {
-          y[o] = f2h (silu (v[NB - 1]) * v[0]);
-          continue;
-        }
-      float r = v[0];
-      if (a.nmat == 1)
-        {
-          r = r * a.scale + a.bias;
-          if (a.act == 1)
-            r = silu (r);
-        }
-      uint16_t h = f2h (r);
-      if (a.nmat == 1 && a.residual)
-        h = f2h (h2f (h) + h2f (ldg (a.residual + o)));
-      y[o] = h;
-      if (a.nmat == 1 && a.y32)
-        a.y32[(size_t)m * a.N + n] = h2f (h);
-    }
-}
-
-// ---------------------------------------------------------------------------
-// few token rows (M <= 32), second form: K split over workgroups as well
-// ---------------------------------------------------------------------------
-// The form above keeps a wave's x fragments in registers next to its weight
-// fragments; an x fragment is twice the bytes of the Q8_0 weights it meets, so
-// few weight bytes are in flight per compute unit, in two dependent rounds, and
-// a matrix of 4096 rows occupies half the compute units.  Here a workgroup
-// owns 32 weight rows and a 1024-wide slice of K: its 32 x 1024 piece of x
-// goes to LDS once (64 KiB, so two workgroups share a compute unit and one
-// streams while the other reduces), each of the 8 waves requests ALL of its
-// weights (4 Q8_0 blocks of 32 rows) at the start, in one round, and reads
-// the x operand from LDS.  The slices' partial sums (fp32) go to a workspace and a
-// second small kernel adds them in slice order and applies the epilogue, so
-// the result does not depend on timing.
+// A workgroup owns 32 weight rows and a 1024-wide slice of K: its 32 x 1024
+// piece of x goes to LDS once (64 KiB, so two workgroups share a compute unit
+// and one streams while the other reduces), each of the 8 waves requests ALL
+// of its weights (4 Q8_0 blocks of 32 rows) at the start, in one round, and
+// reads the x operand from LDS.  The slices' partial sums (fp32) go to a
+// workspace and a second small kernel adds them in slice order and applies
+// the epilogue, so the result does not depend on timing.  (An earlier form
+// with the x fragments in registers next to the weights, one workgroup per 32
+// weight rows over the whole of K, streamed at half the rate; from 33 rows on
+// the tile kernel with its own k-split is faster than either.)
 constexpr int kSk2Waves = 8;
 constexpr int kSk2Slice = 1024;                // k extent of a workgroup
 constexpr int kSk2Ldx = kSk2Slice + 8;         // LDS row stride of x in halves
@@ -939,32 +739,6 @@ launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
   return true;
 }
 
-template <int WT>
-int
-launch_skinny (const GemmArgs &a, hipStream_t s)
-{
-  int err = 0;
-  if (launch_skinny2<WT> (a, s, err))
-    return err;
-  const dim3 grid ((unsigned)((a.N + 31) / 32), 1, (unsigned)(a.upgate ? 1 : a.nmat));
-  // sixteen waves where their registers (128 each) and the reduction buffer allow
-  if (a.upgate)
-    {
-      if (a.M <= 32)
-        gemm_skinny_kernel<WT, 1, true, 8><<<grid, dim3 (512), 0, s>>> (a);
-      else
-        gemm_skinny_kernel<WT, 2, true, 8><<<grid, dim3 (512), 0, s>>> (a);
-    }
-  else
-    {
-      if (a.M <= 32)
-        gemm_skinny_kernel<WT, 1, false, 16><<<grid, dim3 (1024), 0, s>>> (a);
-      else
-        gemm_skinny_kernel<WT, 2, false, 8><<<grid, dim3 (512), 0, s>>> (a);
-    }
-  return (int)hipGetLastError ();
-}
-
 template <int BM, int WT>
 int
 launch_cfg (const GemmArgs &a, hipStream_t s)
@@ -1040,9 +814,14 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
   if (!gemm_mfma_supported (a))
     return (int)hipErrorInvalidValue;
   bool small = a.M <= 64;
-  // few rows, one problem, no batch: the weight-streaming form
-  if (small && a.batch <= 1 && a.wtype != 2 && (a.wtype == 8 || (a.K % 16) == 0))
-    return a.wtype == 8 ? launch_skinny<8> (a, s) : launch_skinny<1> (a, s);
+  // up to 32 rows, one problem, no batch: the weight-streaming form (if its
+  // workspace holds the partial sums)
+  if (a.M <= 32 && a.batch <= 1 && a.wtype != 2 && (a.wtype == 8 || (a.K % 16) == 0))
+    {
+      int err = 0;
+      if (a.wtype == 8 ? launch_skinny2<8> (a, s, err) : launch_skinny2<1> (a, s, err))
+        return err;
+    }
   // the half-height tile also where full tiles would be too few to occupy the
   // compute units (a few hundred token rows)
   {
