@@ -140,8 +140,9 @@ def test_matmul_q8_0_epilogue(dev, rng):
 @pytest.mark.parametrize("M,N,K", [(9, 128, 32), (16, 130, 512), (64, 256, 4096), (100, 200, 1376), (300, 1376, 512),
                                    (129, 64, 11008), (65, 32000, 512)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
-    """M >= 9 token rows run on the matrix cores (weights dequantised to
-    fp16(q*d) on the way into LDS, fp32 accumulation)."""
+    """Several token rows run on the matrix cores (quants as exact fp16
+    integers, block sums by MFMA, block scale in fp32); the shapes cover the
+    few-row kernel, half- and full-height tiles and the k-split."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
@@ -152,8 +153,11 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     assert rel_err(got, exact) < 2e-3
 
 
-def test_gemm_q8_0_epilogue_and_strides(dev, rng):
-    M, N, K = 40, 200, 512
+@pytest.mark.parametrize("M,N,K", [(40, 200, 512), (72, 200, 2048), (20, 200, 2048)])
+def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
+    """scale / bias / activation, residual, widened copy and row strides: on
+    the tile kernel without (K 512) and with the k-split, and on the few-row
+    kernel (20 rows); the latter two finish in the reduction kernel"""
     raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
     x = rng.standard_normal((M, K)).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
