@@ -83,10 +83,9 @@ Llama2Block::init ()
 absl::StatusOr<Tensor>
 Llama2Block::operator() (Tensor in, const size_t offset)
 {
-  auto normed = norm_op_->operator() (in);
-  VKLLAMA_STATUS_OK (normed);
-  auto transformed = attn_op_->operator() (*normed, offset);
-  VKLLAMA_STATUS_OK (transformed);
+  // The residual additions of the reference's block (element_wise after the
+  // attention and after the feed-forward part) run in the launches of the two
+  // projections that precede them: the same fp16 values, two launches less.
   Tensor residual = in;
   if (transformer_params_.clip_output)
     {
@@ -100,14 +99,15 @@ Llama2Block::operator() (Tensor in, const size_t offset)
       VKLLAMA_STATUS_OK (cliped);
       residual = *cliped;
     }
-  // written in place into the residual operand
-  auto added = add_op_->operator() (*transformed, residual);
+  auto normed = norm_op_->operator() (in);
+  VKLLAMA_STATUS_OK (normed);
+  attn_op_->set_residual (&residual);
+  auto added = attn_op_->operator() (*normed, offset);
   VKLLAMA_STATUS_OK (added);
   auto normed2 = norm_op2_->operator() (*added);
   VKLLAMA_STATUS_OK (normed2);
-  auto feed = feedforward_op_->operator() (*normed2);
-  VKLLAMA_STATUS_OK (feed);
-  return add_op2_->operator() (*feed, *added);
+  feedforward_op_->set_residual (&*added);
+  return feedforward_op_->operator() (*normed2);
 }
 
 void

@@ -89,6 +89,8 @@ FeedForward::operator() (Tensor X) noexcept
                               (int)X.width (), t0_.data (), dev_->stream ());
   timer_.stop (dev_);
   VKLLAMA_STATUS_OK (launch_status ("feed_forward up/gate", err));
+  down_op_->set_residual (residual_);
+  residual_ = nullptr;
   return (*down_op_) (t0_);
 }
 }

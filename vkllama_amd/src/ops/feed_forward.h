@@ -18,6 +18,8 @@ public:
                const bool transposed_weight = false,
                const Tensor::DType dtype = FP16);
   absl::StatusOr<Tensor> operator() (Tensor X) noexcept;
+  // the next call only: the residual is added in the down projection's launch
+  void set_residual (const Tensor *r) noexcept { residual_ = r; }
   absl::Status init () noexcept override;
   uint64_t time () noexcept override;
   Tensor &w1 () { return w1_; }
@@ -25,6 +27,7 @@ public:
   Tensor &w3 () { return w3_; }
 
 private:
+  const Tensor *residual_ = nullptr;
   Tensor t0_;
   Tensor w1_;
   Tensor w2_;

@@ -124,6 +124,14 @@ MatMul::run_ (Tensor &a, Tensor &b) noexcept
   if (out_.size () == 0)
     return out_;
 
+  const Tensor *res = residual_;
+  residual_ = nullptr;
+  if (res
+      && (res->channels () != out_c || res->height () != out_h || res->width () != out_w
+          || res->hs () != out_.hs () || res->dtype () != FP16
+          || (b_dtype_ != Q8_0 && !transpose_b_) || out_c != 1))
+    return absl::InvalidArgumentError ("matmul residual operand does not fit the product");
+
   void *s = dev_->stream ();
   int err = 0;
   timer_.start (dev_);
@@ -135,7 +143,8 @@ MatMul::run_ (Tensor &a, Tensor &b) noexcept
             "matmul with Q8_0 weights supports channels = 1, got %zu", out_c));
       err = vkl_matmul_q8_0 (a.data (), b.data (), (int)out_h, (int)out_w,
                              (int)K, a.hs () / 2, out_.hs () / 2, scale_,
-                             bias_, act_, nullptr, out_.data (), nullptr, s);
+                             bias_, act_, res ? res->data () : nullptr,
+                             out_.data (), nullptr, s);
     }
   else
     {
@@ -148,8 +157,8 @@ MatMul::run_ (Tensor &a, Tensor &b) noexcept
         err = vkl_matmul_f16_tb (a.data (), b.data (), (int)out_c, (int)out_h,
                                  (int)out_w, (int)K, acs, a.hs () / 2, bcs,
                                  b.hs () / 2, out_.cs () / 2, out_.hs () / 2,
-                                 scale_, bias_, act_, nullptr, out_.data (),
-                                 nullptr, s);
+                                 scale_, bias_, act_, res ? res->data () : nullptr,
+                                 out_.data (), nullptr, s);
       else
         err = vkl_matmul_f16_nn (a.data (), b.data (), (int)out_c, (int)out_h,
                                  (int)out_w, (int)K, acs, a.hs () / 2, bcs,

@@ -27,8 +27,14 @@ public:
   absl::Status init () noexcept override;
   uint64_t time () noexcept override;
 
+  // The next product only: out = fp16(fp16(product) + r), r of the output's
+  // shape (what an ElementWise add after the product would give, in the same
+  // launch).  Not part of the reference's interface.
+  void set_residual (const Tensor *r) noexcept { residual_ = r; }
+
 private:
   absl::StatusOr<Tensor> run_ (Tensor &a, Tensor &b) noexcept;
+  const Tensor *residual_ = nullptr;
   Tensor weight_;
   const int broadcast_type_;
   const int act_;

@@ -218,6 +218,8 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
       attn_timer_.stop (dev_);
       VKLLAMA_STATUS_OK (launch_status ("attention", err));
       attn_fused_last_ = true;
+      matmul_o_->set_residual (residual_);
+      residual_ = nullptr;
       return (*matmul_o_) (attn_out_);
     }
 
@@ -290,6 +292,8 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
       attn_timer_.stop (dev_);
       VKLLAMA_STATUS_OK (launch_status ("attention", err));
       attn_fused_last_ = true;
+      matmul_o_->set_residual (residual_);
+      residual_ = nullptr;
       return (*matmul_o_) (attn_out_);
     }
 
@@ -310,6 +314,8 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
   //[1, seqlen, heads*dim]
   VKLLAMA_STATUS_OK (concated->reshape (
       1, concated->channels (), concated->height () * concated->width ()));
+  matmul_o_->set_residual (residual_);
+  residual_ = nullptr;
   return (*matmul_o_) (*concated);
 }
 

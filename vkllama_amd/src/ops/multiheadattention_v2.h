@@ -37,6 +37,9 @@ public:
   // 251 with rope_fp16.comp:34).  true (default) reproduces that.
   void set_lastblock_rope_quirk (bool on) { rope_quirk_ = on; }
 
+  // the next call only: the residual is added in the output projection's launch
+  void set_residual (const Tensor *r) noexcept { residual_ = r; }
+
   Tensor &wk () { return wk_; }
   Tensor &wq () { return wq_; }
   Tensor &wv () { return wv_; }
@@ -46,6 +49,7 @@ public:
   Rope *rope () { return rope_q_.get (); }
 
 private:
+  const Tensor *residual_ = nullptr;
   Tensor wk_, wq_, wv_, wo_;
   Tensor kcache_, vcache_;
   const int maxlen_;
