@@ -318,7 +318,7 @@ gemm_step (const GemmArgs &a, const TileAddr<BM, WT> &ta, int kbase, int kt, int
               part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[2 * blk + 1][mi], bf[2 * blk + 1][ni], part, 0, 0, 0);
 #pragma unroll
               for (int r = 0; r < 16; ++r)
-                acc[mi][ni][r] += part[r] * sc[blk][ni];
+                acc[mi][ni][r] = __builtin_fmaf (part[r], sc[blk][ni], acc[mi][ni][r]);
             }
     }
   else
@@ -619,7 +619,7 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
           const float sc = h2f (dv[u]);
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            acc[r] += part[r] * sc;
+            acc[r] = __builtin_fmaf (part[r], sc, acc[r]);
         }
       else
         {
