@@ -46,7 +46,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of a kernel from hardware counters (FETCH_SIZE +
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
-TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96197644}
+TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96185914}
 
 
 def cpu_baseline(cfg, weights, n_tokens):
