@@ -659,11 +659,24 @@ skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S, int mrows)
     return;
   const int m = (int)(i / a.N), n = (int)(i % a.N);
   const int nm = a.upgate ? 2 : a.nmat;
+  const size_t o = (size_t)m * a.ys + n;
+  // the residual value and the parts are requested unconditionally, eight
+  // parts at a time from clamped slices (a loop with a run-time bound around
+  // single loads would make one trip to memory per part); a part past the
+  // last counts as zero, so the parts are still added in slice order
+  const uint16_t rs = ldg (a.residual ? a.residual + o : (const uint16_t *)ws);
   float v[3] = { 0.f, 0.f, 0.f };
   for (int t = 0; t < nm; ++t)
-    for (int sl = 0; sl < S; ++sl)
-      v[t] += ldg (ws + ((size_t)(t * S + sl) * mrows + m) * a.N + n);
-  const size_t o = (size_t)m * a.ys + n;
+    for (int s0 = 0; s0 < S; s0 += 8)
+      {
+        float pc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          pc[j] = ldg (ws + ((size_t)(t * S + min (s0 + j, S - 1)) * mrows + m) * a.N + n);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          v[t] += s0 + j < S ? pc[j] : 0.f;
+      }
   if (a.upgate)
     {
       a.y[0][o] = f2h (silu (v[1]) * v[0]);
@@ -680,7 +693,7 @@ skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S, int mrows)
     r = silu (r);
   uint16_t h = f2h (r);
   if (a.residual)
-    h = f2h (h2f (h) + h2f (ldg (a.residual + o)));
+    h = f2h (h2f (h) + h2f (rs));
   a.y[0][o] = h;
   if (a.y32)
     a.y32[(size_t)m * a.N + n] = h2f (h);
