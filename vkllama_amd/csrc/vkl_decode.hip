@@ -1,11 +1,13 @@
 // Fused one-token decode step for Llama-2-shaped models with Q8_0 weights.
 //
-// Work decomposition: a grid of G workgroups of 512 threads (8 waves), G = the
-// number of compute units.  In a projection phase the output rows are grouped
-// into units of 2 rows (4 for the fused up/gate product: two up rows and the
-// two gate rows that pair with them); workgroup g owns a contiguous range of
-// units, so it streams one contiguous span of each int8 plane, and wave w of
-// the group takes every 8th unit.  Lane l of a wave handles the 16 quants at
+// Work decomposition: a grid of G workgroups of 512 threads (8 waves), two
+// per compute unit (one per compute unit in the persistent mode).  In a
+// projection phase the output rows are grouped into units: 2 rows (K/Q/V,
+// the output layer), an up row and the gate row that pairs with it (the
+// fused up/gate product), or 1 row (Wo and down, whose rows are few and long:
+// every wave then has a unit).  Workgroup g owns a contiguous range of units,
+// so it streams one contiguous span of each int8 plane, and wave w of the
+// group takes every 8th unit.  Lane l of a wave handles the 16 quants at
 // k = step*1024 + 16*l of a row (one dwordx4 load = half a Q8_0 block).
 //
 // A wave's work is a sequence of items (one unit x one K chunk, 8 dwordx4
