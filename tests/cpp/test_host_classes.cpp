@@ -353,6 +353,56 @@ test_matmul_q8 (Ctx &c, int M, int N, int K, int act)
   CHECK (re <= 1e-2f);
 }
 
+// MatMul::set_residual: the product with the residual added in its launch
+// equals the product followed by an ElementWise add, value for value, for the
+// one call it was set for
+void
+test_matmul_residual (Ctx &c, int M, int N, int K)
+{
+  g_test = "MatMul residual M" + std::to_string (M) + " N" + std::to_string (N) + " K" + std::to_string (K);
+  vec x = randn ((size_t)M * K), w = randn ((size_t)N * K, 0.05f), r = randn ((size_t)M * N);
+  auto tx = half_tensor (c, x, 1, M, K);
+  auto tw = q8_tensor (c, w, N, K);
+  auto tr = half_tensor (c, r, 1, M, N);
+  CHECK_OK (tx.status ());
+  CHECK_OK (tw.status ());
+  CHECK_OK (tr.status ());
+  MatMul fused (&c.dev, &c.cmd, *tw, 1.0f, 0.f, 0, 0, true, FP16, Q8_0);
+  MatMul plain (&c.dev, &c.cmd, *tw, 1.0f, 0.f, 0, 0, true, FP16, Q8_0);
+  ElementWise add (&c.dev, &c.cmd, 0, FP16);
+  CHECK_OK (fused.init ());
+  CHECK_OK (plain.init ());
+  CHECK_OK (add.init ());
+  fused.set_residual (&*tr);
+  auto a = fused (*tx);
+  CHECK_OK (a.status ());
+  auto got = fetch_half (c, *a);
+  CHECK_OK (got.status ());
+  auto b = plain (*tx);
+  CHECK_OK (b.status ());
+  auto prod = fetch_half (c, *b); // before the add writes in place
+  CHECK_OK (prod.status ());
+  auto sum = add (*b, *tr);
+  CHECK_OK (sum.status ());
+  auto want = fetch_half (c, *sum);
+  CHECK_OK (want.status ());
+  CHECK (*got == *want);
+  // the residual held for one call only
+  auto again = fused (*tx);
+  CHECK_OK (again.status ());
+  auto got2 = fetch_half (c, *again);
+  CHECK_OK (got2.status ());
+  CHECK (*got2 == *prod);
+  // a residual of another shape is refused
+  auto bad = half_tensor (c, r, 1, N, M);
+  CHECK_OK (bad.status ());
+  if (M != N)
+    {
+      fused.set_residual (&*bad);
+      CHECK (fused (*tx).status ().code () == absl::StatusCode::kInvalidArgument);
+    }
+}
+
 void
 test_matmul_f16 (Ctx &c)
 {
@@ -856,6 +906,10 @@ run_gpu ()
   test_matmul_q8 (c, 1, 512, 1376, 0);
   test_matmul_q8 (c, 3, 130, 512, 1);
   test_matmul_q8 (c, 70, 96, 256, 0);
+  test_matmul_residual (c, 1, 512, 1376);  // one row: the decode step's streaming kernel
+  test_matmul_residual (c, 20, 130, 2048); // few-row kernel and its reduction
+  test_matmul_residual (c, 70, 96, 2048);  // tile kernel with the k-split
+  test_matmul_residual (c, 150, 300, 256); // tile kernel
   test_matmul_f16 (c);
   test_elementwise_cast_argmax (c);
   test_embedding (c);
