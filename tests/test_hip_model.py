@@ -108,6 +108,29 @@ def test_greedy_ids_identical_to_oracle_small(cfg, seed, fused):
     m.close()
 
 
+@pytest.mark.parametrize("wtype", [8, 1])
+def test_wide_rows_decode_and_prompt(wtype):
+    """Row widths of the 13B shape (dim 5120, ffn 13824: activation rows of two
+    and four 4096-value chunks, weight rows of more than one item, 40 heads) on
+    a one-layer model: prompt pass and one-token steps against the oracle."""
+    cfg = dict(dim=5120, n_layers=1, n_heads=40, ffn=13824, vocab=512, maxlen=48, eps=1e-5, wtype=wtype)
+    w = M.synth_weights(cfg, seed=7)
+    m = M.Llama2(cfg, w)
+    om = O.OracleModel(cfg, w)
+    prompt = np.array([5, 17, 99, 3, 64, 8, 300, 2, 11], np.uint32)
+    assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
+    pos, tok = len(prompt), 7
+    for _ in range(4):
+        got, want = m.forward([tok], pos), om.forward([tok], pos)
+        assert logit_err(got, want) < 1e-2, pos
+        assert int(np.argmax(got)) == int(np.argmax(want)), pos
+        tok, pos = int(np.argmax(want)), pos + 1
+    ids, _, _ = m.generate_greedy(prompt, 8)
+    want_ids, _ = om.generate_greedy(prompt, 8)
+    assert list(ids) == list(want_ids)
+    m.close()
+
+
 def test_tiny_llama_config2_greedy_128_tokens():
     """Tiny-llama benchmark configuration: prompt of 16 ids in [3, 32000), greedy 128 tokens;
     the first 32 must equal the oracle's (here: all of them are compared and
