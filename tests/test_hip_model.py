@@ -131,6 +131,33 @@ def test_wide_rows_decode_and_prompt(wtype):
     m.close()
 
 
+def test_full_width_properties():
+    """The 7B widths (dim 4096, ffn 11008, 32 heads, vocabulary 32000) on two
+    layers, through properties that need no oracle: the decode step and the
+    prompt pass agree on the same position, generation is repeatable bit for
+    bit, and the replayed graph gives the ids of the step-by-step launches."""
+    cfg = dict(dim=4096, n_layers=2, n_heads=32, ffn=11008, vocab=32000, maxlen=96, eps=1e-5, wtype=8)
+    w = M.synth_weights(cfg, seed=99)
+    m = M.Llama2(cfg, w)
+    # (the reference rotates the last block's query of a prompt pass at the
+    # pass's first position; with that reproduced the two would differ)
+    m.set_option("lastblock_rope_quirk", 0)
+    rng = np.random.default_rng(99)
+    prompt = rng.integers(3, cfg["vocab"], 40).astype(np.uint32)
+    whole = m.forward(prompt, 0)                 # prompt pass, last row
+    m.forward(prompt[:-1], 0)
+    step = m.forward(prompt[-1:], len(prompt) - 1)  # the same position as a decode step
+    assert logit_err(step, whole) < 1e-2
+    assert int(np.argmax(step)) == int(np.argmax(whole))
+    runs = []
+    for graph in (1, 1, 0):
+        m.set_option("decode_graph", graph)
+        ids, _, _ = m.generate_greedy(prompt, 32)
+        runs.append(list(ids))
+    assert runs[0] == runs[1] == runs[2]
+    m.close()
+
+
 def test_tiny_llama_config2_greedy_128_tokens():
     """Tiny-llama benchmark configuration: prompt of 16 ids in [3, 32000), greedy 128 tokens;
     the first 32 must equal the oracle's (here: all of them are compared and
