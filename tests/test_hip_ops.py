@@ -527,3 +527,50 @@ def test_reduce_last_axis(dev, rng, op, shape):
         scale = np.abs(x64).sum(-1) / (shape[2] if op == 3 else 1)
         assert np.all(np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 0.1 * scale) + 1e-3)
 
+
+
+# ------------------------------------ full sizes, through exact properties ---
+def test_q8_roundtrip_full_size(dev, rng):
+    """The 7B down-projection matrix (4096 x 11008): GGUF blocks -> planar
+    device layout -> GGUF blocks, bit for bit."""
+    rows, K = 4096, 11008
+    raw, _ = q8_weights(rng, rows, K)
+    staging = dev.upload(raw)
+    planar = dev.alloc(raw.nbytes)
+    back = dev.alloc(raw.nbytes)
+    capi.check(L().vkl_q8_0_pack(staging.ptr, planar.ptr, rows, K, dev.stream))
+    capi.check(L().vkl_q8_0_unpack(planar.ptr, back.ptr, rows, K, dev.stream))
+    assert np.array_equal(back.read(np.uint8, raw.shape), raw)
+
+
+@pytest.mark.parametrize("M", [1, 20, 48, 200, 1024])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (4096, 11008)])
+def test_matmul_q8_0_full_size_scaling_and_rows(dev, rng, M, N, K):
+    """7B shapes on every product kernel (one row: the decode step's streaming
+    kernel; few rows; tiles with and without the k-split).  Doubling x doubles
+    every product, sum and (normal) rounded result exactly, so y(2x) must equal
+    2 y(x) bit for bit; and a row's result does not depend on the other rows of the
+    call (the same row alone, on the same kernel family, gives the same bits)."""
+    raw, _ = q8_weights(rng, N, K, 0.002, 0.006)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dw = dev.upload_q8_0(raw, N, K)
+
+    def run(xx):
+        dx = dev.upload(xx)
+        dy = dev.alloc(xx.shape[0] * N * 2)
+        capi.check(L().vkl_matmul_q8_0(dx.ptr, dw.ptr, xx.shape[0], N, K, K, N, 1.0, 0.0, 0,
+                                       None, dy.ptr, None, dev.stream))
+        return f16(dy, (xx.shape[0], N)).copy()
+
+    y1 = run(x)
+    y2 = run((x * np.float16(2)).astype(np.float16))
+    assert np.isfinite(y1.astype(np.float32)).all()
+    # (a subnormal fp16 result has a fixed absolute precision: doubling the
+    # exact value may round the other way there, within one unit)
+    normal = np.abs(y1.astype(np.float32)) >= 2.0 ** -14
+    d = (y1 * np.float16(2)).view(np.uint16).astype(np.int32) - y2.view(np.uint16).astype(np.int32)
+    assert not d[normal].any()
+    assert np.abs(d[~normal]).max(initial=0) <= 1
+    # permuting the rows of x permutes the rows of y
+    perm = rng.permutation(M)
+    assert np.array_equal(run(x[perm]).view(np.uint16), y1[perm].view(np.uint16))
