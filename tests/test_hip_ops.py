@@ -574,3 +574,50 @@ def test_matmul_q8_0_full_size_scaling_and_rows(dev, rng, M, N, K):
     # permuting the rows of x permutes the rows of y
     perm = rng.permutation(M)
     assert np.array_equal(run(x[perm]).view(np.uint16), y1[perm].view(np.uint16))
+
+
+@pytest.mark.parametrize("M", [1, 32, 300])
+def test_kqv_q8_0_full_size_scaling(dev, rng, M):
+    """Fused K/Q/V projection at the 7B width: y(2x) = 2 y(x) bit for bit
+    (normal results) for all three outputs."""
+    N = K = 4096
+    dws = [dev.upload_q8_0(q8_weights(rng, N, K, 0.002, 0.006)[0], N, K) for _ in range(3)]
+    x = rng.standard_normal((M, K)).astype(np.float16)
+
+    def run(xx):
+        dx = dev.upload(xx)
+        outs = [dev.alloc(M * N * 2) for _ in range(3)]
+        capi.check(L().vkl_kqv_q8_0(dx.ptr, dws[0].ptr, dws[1].ptr, dws[2].ptr, M, N, K, outs[0].ptr,
+                                    outs[1].ptr, outs[2].ptr, dev.stream))
+        return [f16(o, (M, N)).copy() for o in outs]
+
+    for y1, y2 in zip(run(x), run((x * np.float16(2)).astype(np.float16))):
+        normal = np.abs(y1.astype(np.float32)) >= 2.0 ** -14
+        d = (y1 * np.float16(2)).view(np.uint16).astype(np.int32) - y2.view(np.uint16).astype(np.int32)
+        assert not d[normal].any()
+        assert np.abs(d[~normal]).max(initial=0) <= 1
+
+
+def test_attn_prefill_causal_full_size_is_causal(dev, rng):
+    """Prompt attention at 32 heads x 1024 positions x 128: the output of a
+    position depends on nothing behind it.  Changing q, k and v from position
+    700 on must leave the outputs of positions 0..699 bit for bit."""
+    H, S, hd, cut = 32, 1024, 128, 700
+    sc = 1.0 / np.sqrt(hd)
+
+    def run(q, k, v):
+        dq, dk, dv = dev.upload(q), dev.upload(k), dev.upload(v)
+        do = dev.alloc(H * S * hd * 2)
+        capi.check(L().vkl_attn_prefill_causal_f16(dq.ptr, dk.ptr, dv.ptr, H, S, S, hd, S * hd, hd, S * hd, hd,
+                                                   S * hd, hd, sc, do.ptr, hd, S * hd, dev.stream))
+        return f16(do, (H, S, hd)).copy()
+
+    q, k, v = (rng.standard_normal((H, S, hd)).astype(np.float16) for _ in range(3))
+    a = run(q, k, v)
+    q2, k2, v2 = q.copy(), k.copy(), v.copy()
+    for t in (q2, k2, v2):
+        t[:, cut:] = rng.standard_normal((H, S - cut, hd)).astype(np.float16)
+    b = run(q2, k2, v2)
+    assert np.isfinite(a.astype(np.float32)).all()
+    assert np.array_equal(a[:, :cut].view(np.uint16), b[:, :cut].view(np.uint16))
+    assert not np.array_equal(a[:, cut:].view(np.uint16), b[:, cut:].view(np.uint16))
