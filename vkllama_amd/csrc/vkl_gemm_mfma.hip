@@ -531,7 +531,7 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
   float *red = (float *)lds;      // after the products: [waves][32][33]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5;
-  const int n0 = blockIdx.x * 32, slice = blockIdx.y, mat = blockIdx.z;
+  const int n0 = blockIdx.y * 32, slice = blockIdx.x, mat = blockIdx.z;
   const int k0 = slice * kSk2Slice;
   const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
   const void *zeros = g_zero_chunk;
@@ -744,7 +744,7 @@ launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
   float *ws = skinny2_workspace (s);
   if (!ws)
     return false;
-  gemm_skinny2_kernel<WT><<<dim3 ((unsigned)((a.N + 31) / 32), (unsigned)S, (unsigned)nm),
+  gemm_skinny2_kernel<WT><<<dim3 ((unsigned)S, (unsigned)((a.N + 31) / 32), (unsigned)nm),
                            dim3 (kSk2Waves * 64), lds, s>>> (a, ws, S);
   const size_t total = (size_t)a.M * a.N;
   skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S, 32);
