@@ -50,10 +50,13 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
 
 /* One token at KV position `pos` (context length becomes pos + 1).
  *  tok      device-visible uint32: the input token id (ids >= vocab -> 0)
- *  mode     0 = one launch per phase; 1 = one persistent launch per step
- *           with grid barriers; 2 = one launch per phase on two alternating
- *           streams, consecutive phases overlapping and handing over
- *           through an arrival counter
+ *  mode     0 = one launch per phase; 1 = one persistent launch per step:
+ *           the workgroups stay resident, hand activations over through
+ *           memory with bounded waits for one another, and keep the next
+ *           phase's weights streaming meanwhile (Q8_0 weights and contexts
+ *           below 1024 positions; other steps run as mode 0).  The GPU must
+ *           not be shared while a persistent launch runs: see
+ *           vkl_decode_status
  *  logits32 optional device fp32 [vocab]: widened fp16 logits
  *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
  * Returns 0 or a hipError_t; hipErrorInvalidValue for shapes the kernels do
@@ -61,6 +64,14 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
 int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
                      uint32_t pos, int mode, float *logits32,
                      uint32_t *next_tok, void *stream);
+
+/* Persistent launches (mode 1) need every workgroup resident at once; where
+ * that does not hold (a GPU shared with other work) a bounded wait inside the
+ * kernel gives up, the launch still ends, and its results are invalid.  This
+ * call synchronises the stream and returns 0 if no wait gave up since the
+ * last call, hipErrorLaunchFailure otherwise (the mark is cleared).  No
+ * counterpart in the reference, which has no persistent kernels. */
+int vkl_decode_status (const vkl_decode_model *m, void *stream);
 
 /* n_steps greedy tokens without a host round trip per token: step i reads
  * ids[i] (device memory) at position pos0 + i and writes its arg-max id to

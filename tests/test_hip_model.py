@@ -232,23 +232,27 @@ def test_errors(small):
         M.Llama2(cfg, short)
 
 
-@pytest.mark.parametrize("mode", [1, 2])
 @pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5), (TINY, 1234)])
-def test_other_decode_modes_match_oracle(cfg, seed, mode):
-    """decode_mode 1: one persistent launch per token with grid barriers;
-    decode_mode 2: one launch per phase on two alternating streams, each phase
-    prefetching its weights while it waits for its predecessor's arrivals."""
+def test_persistent_decode_matches_oracle(cfg, seed):
+    """decode_mode 1: one persistent launch per token; the workgroups hand the
+    activations over through memory and wait for one another.  Ids identical to
+    the oracle's, and logits bit-identical to the launch-per-phase step (both
+    keep the same order of every sum)."""
     w = M.synth_weights(cfg, seed=seed)
     prompt = np.array([5, 17, 99, 3], np.uint32)
     m = M.Llama2(cfg, w)
-    m.set_option("decode_mode", mode)
+    m.set_option("decode_mode", 1)
+    m0 = M.Llama2(cfg, w)
     om = O.OracleModel(cfg, w)
     assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
-    assert logit_err(m.forward([7], 4), om.forward([7], 4)) < 1e-2
+    m0.forward(prompt, 0)
+    got = m.forward([7], 4)
+    assert logit_err(got, om.forward([7], 4)) < 1e-2
+    assert np.array_equal(got, m0.forward([7], 4))
     ids, _, t_dec = m.generate_greedy(prompt, 32)
     want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 32)
     assert list(ids) == list(want)
-    m.close()
+    m.close(), m0.close()
 
 
 @pytest.mark.parametrize("heads", [4, 2])

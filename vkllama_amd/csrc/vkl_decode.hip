@@ -22,152 +22,15 @@
 // Every phase is HBM-bound: 34 bytes per 32 weights are read exactly once, the
 // activations (a few KiB) come from L2.
 #include "../../include/vkl_decode.h"
-#include "vkl_decode_dev.h"
+#include "vkl_decode_shared.h"
 #include <algorithm>
 #include <vector>
 
 namespace vkl
 {
+using namespace dec;
 namespace
 {
-struct Scratch
-{
-  uint16_t *x;        // [dim] residual stream
-  uint16_t *kqv;      // [3*dim]: k | q | v
-  uint16_t *att;      // [dim]
-  uint16_t *t;        // [ffn] 32-bit words, fp16 in the low half
-  uint16_t *logits16; // [vocab]
-  float *logits32;    // [vocab]
-  float *amax_val;    // [1024]
-  uint32_t *amax_idx; // [1024]
-  uint32_t *sync;     // barrier counter + error flag
-  // long-context attention, split over kAttnChunks chunks of the context
-  uint16_t *sc16;     // [heads][maxlen] fp16 scores
-  float *part_max;    // [heads][kAttnChunks]
-  float *part_sum;    // [heads][kAttnChunks]
-  float *part_out;    // [heads][kAttnChunks][head_dim]
-  size_t bytes;
-};
-
-constexpr int kAttnChunks = 32;      // upper bound on chunks per head
-constexpr int kAttnSplitMinLen = 1024; // shorter contexts use one workgroup per head (measured at 7B:
-                                       // 10.5 against 12.4 us at 768 positions, 12.6 / 12.5 at 1024)
-constexpr int kAttnSweeps = 8;        // sweeps of cache rows a chunk kernel keeps in flight
-constexpr int kAttnChunkRows = 1024;  // most rows of a chunk (longer contexts use one workgroup per head)
-
-__host__ __device__ inline size_t
-align256 (size_t v)
-{
-  return (v + 255) & ~(size_t)255;
-}
-
-__host__ __device__ inline Scratch
-carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd)
-{
-  Scratch s;
-  uint8_t *p = (uint8_t *)base;
-  size_t o = 0;
-  s.x = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
-  s.kqv = (uint16_t *)(p + o), o += align256 ((size_t)dim * 6);
-  s.att = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
-  s.t = (uint16_t *)(p + o), o += align256 ((size_t)ffn * 4);
-  s.logits16 = (uint16_t *)(p + o), o += align256 ((size_t)vocab * 2);
-  s.logits32 = (float *)(p + o), o += align256 ((size_t)vocab * 4);
-  s.amax_val = (float *)(p + o), o += 4096;
-  s.amax_idx = (uint32_t *)(p + o), o += 4096;
-  s.sync = (uint32_t *)(p + o), o += 256;
-  s.sc16 = (uint16_t *)(p + o), o += align256 ((size_t)heads * maxlen * 2);
-  s.part_max = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
-  s.part_sum = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
-  s.part_out = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * hd * 4);
-  s.bytes = o;
-  return s;
-}
-
-struct Params
-{
-  vkl_decode_model m;
-  Scratch s;
-  const uint32_t *tok;
-  uint32_t pos;
-  float *logits32;    // destination of the widened logits
-  uint32_t *next_tok; // may be null
-  uint32_t wait_target; // overlapped launches: arrivals to wait for
-  // replayed loop (vkl_decode_loop): token index and position live in device
-  // memory so that every step is the same sequence of launches
-  const uint32_t *loop; // {index into ids, position}, or null
-  uint32_t *ids;        // loop: input token ids[index], result to ids[index + 1]
-  const uint16_t *gemv_res; // stand-alone product (PH_GEMV): residual operand or null
-  int stream_once; // the weights of a step exceed the caches: request them non-temporally
-#ifdef VKL_TRACE
-  unsigned long long *trace; // [phase slot][wg][8] wall-clock stamps
-#endif
-};
-
-#ifdef VKL_TRACE
-#define VKL_TR(slot)                                                          \
-  if (threadIdx.x == 0 && p.trace)                                            \
-    p.trace[((size_t)(layer * 8 + phase) * 1024 + wg) * 8 + (slot)]           \
-        = wall_clock64 ();
-#define VKL_TRP                                                               \
-  (p.trace ? p.trace + ((size_t)(layer * 8 + phase) * 1024 + wg) * 8 : nullptr)
-#else
-#define VKL_TR(slot)
-#define VKL_TRP nullptr
-#endif
-
-// position and token of the step: kernel arguments, or the device-resident
-// loop state when the step is replayed from a graph
-__device__ __forceinline__ uint32_t
-step_pos (const Params &p)
-{
-  return p.loop ? ldg (p.loop + 1) : p.pos;
-}
-
-__device__ __forceinline__ const uint32_t *
-step_tok (const Params &p)
-{
-  return p.loop ? p.ids + ldg (p.loop) : p.tok;
-}
-
-// ---------------------------------------------------------------------------
-// activation staging
-// ---------------------------------------------------------------------------
-template <bool COH>
-__device__ __forceinline__ uint32_t
-ld_u32 (const uint32_t *p)
-{
-  if (COH)
-    return ld_coherent_u32 (p);
-  return ldg (p);
-}
-
-template <bool COH>
-__device__ __forceinline__ void
-st_u32 (uint32_t *p, uint32_t v)
-{
-  if (COH)
-    st_coherent_u32 (p, v);
-  else
-    stg (p, v);
-}
-
-// sum over the workgroup; `red` is an LDS array of kDecWaves floats
-__device__ __forceinline__ float
-block_sum (float v, float *red)
-{
-  v = wave_sum (v);
-  __syncthreads ();
-  if ((threadIdx.x & 63) == 0)
-    red[threadIdx.x >> 6] = v;
-  __syncthreads ();
-  float t = 0.f;
-#pragma unroll
-  for (int w = 0; w < kDecWaves; ++w)
-    t += red[w];
-  return t;
-}
-
 // The activation row (K fp16 values, K a multiple of 32, K <= 16384) is
 // fetched into registers first: thread t holds the 8-element chunks t,
 // t+512, t+1024, t+1536.  Issued before any weight load, these are the oldest
@@ -496,12 +359,6 @@ struct Epilogue
   uint32_t *amax_idx;
 };
 
-__device__ __forceinline__ bool
-better (float v, uint32_t i, float bv, uint32_t bi)
-{
-  return v > bv || (v == bv && i < bi);
-}
-
 // The pipeline's registers: two item buffers shared by every projection phase
 // (each item is 8 dwordx4 weight loads and 8 scales per lane), and the small
 // state of the phase in progress.  Keeping ONE pair of buffers for all phases
@@ -516,13 +373,6 @@ wmat (const void *w, int N, int K)
     return qmat (w, N, K);
   return QMat{ (const uint8_t *)w, (const uint16_t *)w };
 }
-
-struct PipeBuf
-{
-  uint4 w[8];
-  uint16_t d[8];
-  uint32_t res; // mode 0: the two residual values of the item's unit
-};
 
 struct PipeState
 {
@@ -877,239 +727,6 @@ template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
 };
 
 // ---------------------------------------------------------------------------
-// attention for one head, context length L = pos + 1
-// ---------------------------------------------------------------------------
-// LDS use: qk[3*HD] fp16 (rotated q, rotated k, v), sc[maxlen] fp32,
-// part[RPB][HD] fp32, red[2*kDecWaves].
-template <int HD, bool COH>
-__device__ __forceinline__ void
-attention_head (const Params &p, const vkl_layer_weights &lw, int head,
-                uint8_t *lds, unsigned long long *tr = nullptr)
-{
-#ifdef VKL_TRACE
-#define VKL_TRA(slot)                                                         \
-  if (tr && threadIdx.x == 0)                                                 \
-    tr[slot] = wall_clock64 ();
-#else
-#define VKL_TRA(slot)
-#endif
-  constexpr int LPR = HD / 8;            // lanes per cache row (16 B each)
-  constexpr int RPB = kDecThreads / LPR; // cache rows per sweep
-  constexpr int PRE = 8;                 // sweeps prefetched up front
-  const int dim = p.m.dim, maxlen = p.m.maxlen;
-  const uint32_t pos = step_pos (p);
-  const int L = (int)pos + 1;
-  uint16_t *qk = (uint16_t *)lds;    // [3*HD]
-  float *sc = (float *)(lds + 1024);      // [maxlen]
-  float *part = sc + ((maxlen + 3) & ~3); // [RPB][HD], 16-byte aligned
-  float *red = part + RPB * HD;           // [2*kDecWaves]
-  uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
-  uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
-  const uint16_t *kin = p.s.kqv + head * HD;
-  const uint16_t *qin = p.s.kqv + dim + head * HD;
-  const uint16_t *vin = p.s.kqv + 2 * dim + head * HD;
-  const int tid = threadIdx.x;
-  const int sub = tid % LPR, grp = tid / LPR;
-
-  // This token's q, k, v and its rotation factors are requested first and
-  // the first sweeps of cached K and V rows right behind them: loads return
-  // in order, so the few bytes the prologue needs are not queued behind the
-  // cache rows.  Every load is unconditional, from a clamped address (a branch
-  // around a load would make the wait below a wait for all of them): threads
-  // without a q/k/v pair repeat pair 0, cache rows past the context repeat the
-  // last row and are ignored where they would be used.
-  const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
-  const bool is_v = tid >= HD && tid < HD + HD / 2;
-  const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
-  const uint32_t inw
-      = ld_u32<COH> ((const uint32_t *)(is_k ? kin : (is_v ? vin : qin)) + pi);
-  const float fc = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
-  const float fs = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
-  // (the scheduler must not move the cache rows ahead of these)
-  __builtin_amdgcn_sched_barrier (0);
-  uint4 kpre[PRE], vpre[PRE];
-  const int lastrow = max ((int)pos - 1, 0);
-#pragma unroll
-  for (int j = 0; j < PRE; ++j)
-    kpre[j] = ldg4 (kc + (size_t)min (grp + j * RPB, lastrow) * HD + sub * 8);
-#pragma unroll
-  for (int j = 0; j < PRE; ++j)
-    vpre[j] = ldg4 (vc + (size_t)min (grp + j * RPB, lastrow) * HD + sub * 8);
-  __builtin_amdgcn_sched_barrier (0);
-
-  // RoPE on adjacent pairs at position pos.  The new K and V rows are used
-  // from LDS here; they go to the cache at the end of the head (a store
-  // under a branch at this point would turn the counted waits for the cache
-  // rows into waits for everything in flight).
-  const float ra = h2f ((uint16_t)(inw & 0xffff)), rb = h2f ((uint16_t)(inw >> 16));
-  const uint32_t rot = (uint32_t)f2h (ra * fc - rb * fs)
-                       | ((uint32_t)f2h (ra * fs + rb * fc) << 16);
-  if (is_q || is_k)
-    ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + pi] = rot;
-  if (is_v)
-    ((uint32_t *)qk)[HD + pi] = inw;
-  __syncthreads ();
-  VKL_TRA (1);
-
-  // scores[l] = fp16(dot(q, K[l]) / sqrt(HD)); LPR lanes share one cache row
-  const float scale = 1.0f / sqrtf ((float)HD);
-  const uint4 qv = ((const uint4 *)qk)[sub];
-  float mx = -INFINITY; // of the scores this lane has written
-  // lim: rows below it are scored (the cached rows; the token's own row, which
-  // is in LDS, follows after the sweeps)
-  auto score_row = [&] (int l, int lim, const uint4 kv) {
-    float s = l < lim ? dot8_f16 (qv, kv, 0.f) : 0.f;
-    s = row_sum<LPR> (s);
-    if (l < lim && sub == 0)
-      {
-        const float r = h2f (f2h (s * scale + 0.f));
-        sc[l] = r;
-        mx = fmaxf (mx, r);
-      }
-  };
-#pragma unroll
-  for (int j = 0; j < PRE; ++j)
-    {
-      const int l = grp + j * RPB;
-      if (j * RPB < (int)pos) // wave-uniform
-        score_row (l, (int)pos, kpre[j]);
-    }
-  // the rest of the context, PRE sweeps at a time: unconditional loads from
-  // clamped rows, all of a round in flight together (one load per iteration
-  // would cost a trip to memory per sweep)
-  for (int l0 = PRE * RPB; l0 < (int)pos; l0 += PRE * RPB)
-    {
-      uint4 kv[PRE];
-#pragma unroll
-      for (int j = 0; j < PRE; ++j)
-        kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPB + grp, lastrow) * HD + sub * 8);
-#pragma unroll
-      for (int j = 0; j < PRE; ++j)
-        {
-          const int l = l0 + j * RPB + grp;
-          if (l0 + j * RPB < (int)pos) // uniform over the workgroup
-            score_row (l, (int)pos, kv[j]);
-        }
-    }
-  // the token's own row: every group forms it (no lane sits out of the
-  // cross-lane sum), group 0 records it
-  score_row (grp == 0 ? (int)pos : L, L, ((const uint4 *)(qk + HD))[sub]);
-  // the maximum travels with the scores: one barrier covers both
-  mx = wave_max (mx);
-  if ((tid & 63) == 0)
-    red[kDecWaves + (tid >> 6)] = mx;
-  __syncthreads ();
-  VKL_TRA (2);
-
-  // softmax over the L scores; probabilities rounded to fp16
-  mx = red[kDecWaves];
-#pragma unroll
-  for (int w = 1; w < kDecWaves; ++w)
-    mx = fmaxf (mx, red[kDecWaves + w]);
-  const float e0 = tid < L ? expf (sc[tid < L ? tid : 0] - mx) : 0.f;
-  float sum = e0;
-  for (int l = tid + kDecThreads; l < L; l += kDecThreads)
-    sum += expf (sc[l] - mx);
-  sum = wave_sum (sum);
-  if ((tid & 63) == 0)
-    red[tid >> 6] = sum;
-  __syncthreads ();
-  sum = 0.f;
-#pragma unroll
-  for (int w = 0; w < kDecWaves; ++w)
-    sum += red[w];
-  if (tid < L)
-    sc[tid] = h2f (f2h (e0 / sum));
-  for (int l = tid + kDecThreads; l < L; l += kDecThreads)
-    sc[l] = h2f (f2h (expf (sc[l] - mx) / sum));
-  __syncthreads ();
-  VKL_TRA (3);
-
-  // out[j] = fp16(sum_l P[l] V[l][j]); thread = (row group, 8 columns)
-  float acc[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    acc[j] = 0.f;
-  // no branch: a row past the context counts with probability 0 (its values
-  // are those of a real row, see the clamped loads)
-  // (p and v are fp16 values: their product is exact in fp32, so the fused
-  // multiply-add rounds as a multiplication and an addition would)
-  auto pv_add = [&] (float pl, const uint4 vv) {
-    const uint32_t w[4] = { vv.x, vv.y, vv.z, vv.w };
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      {
-        acc[2 * j] = __builtin_fmaf (pl, h2f ((uint16_t)(w[j] & 0xffff)), acc[2 * j]);
-        acc[2 * j + 1] = __builtin_fmaf (pl, h2f ((uint16_t)(w[j] >> 16)), acc[2 * j + 1]);
-      }
-  };
-  auto pv_row = [&] (int l, const uint4 vv) {
-    pv_add (l < (int)pos ? sc[min (l, lastrow)] : 0.f, vv);
-  };
-#pragma unroll
-  for (int j = 0; j < PRE; ++j)
-    {
-      const int l = grp + j * RPB;
-      if (j * RPB < (int)pos) // wave-uniform
-        pv_row (l, vpre[j]);
-    }
-  for (int l0 = PRE * RPB; l0 < (int)pos; l0 += PRE * RPB)
-    {
-      uint4 vv[PRE];
-#pragma unroll
-      for (int j = 0; j < PRE; ++j)
-        vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPB + grp, lastrow) * HD + sub * 8);
-#pragma unroll
-      for (int j = 0; j < PRE; ++j)
-        {
-          const int l = l0 + j * RPB + grp;
-          if (l0 + j * RPB < (int)pos) // uniform over the workgroup
-            pv_row (l, vv[j]);
-        }
-    }
-  // the token's own row (from LDS) is the last of its group's rows
-  pv_add (grp == (int)pos % RPB ? sc[pos] : 0.f, ((const uint4 *)(qk + 2 * HD))[sub]);
-  ((float4 *)(part + grp * HD + sub * 8))[0] = make_float4 (acc[0], acc[1], acc[2], acc[3]);
-  ((float4 *)(part + grp * HD + sub * 8))[1] = make_float4 (acc[4], acc[5], acc[6], acc[7]);
-  __syncthreads ();
-  VKL_TRA (6);
-  // the RPB partial rows of a column are added by four lanes, a quarter of
-  // the rows each, and those four by DPP; the lane of an even column then
-  // takes the odd neighbour's result and stores the pair
-  {
-    const int c = tid >> 2, k = tid & 3;
-    float o = 0.f;
-    if (c < HD)
-      {
-#pragma unroll
-        for (int g = 0; g < RPB / 4; ++g)
-          o += part[(k * (RPB / 4) + g) * HD + c];
-      }
-    o = row_sum<4> (o);
-    const float onext = dpp_get<0x104> (o); // row_shl:4: the lane four up
-    if (c < HD && (tid & 7) == 0)
-      st_u32<COH> ((uint32_t *)(p.s.att + head * HD) + (c >> 1),
-                   (uint32_t)f2h (o) | ((uint32_t)f2h (onext) << 16));
-  }
-  __syncthreads ();
-  if (is_k)
-    stg ((uint32_t *)(kc + (size_t)pos * HD) + pi, rot);
-  if (is_v)
-    stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
-}
-
-__host__ __device__ inline size_t
-lds_bytes_needed (int dim, int ffn, int maxlen, int hd)
-{
-  const size_t kmax = (size_t)(dim > ffn ? dim : ffn);
-  // staged activation row + reduction words + parked norm weights
-  const size_t stage = ((kmax + 31) / 32 * 32) * 2 + 256 + (size_t)dim * 4;
-  const size_t rpb = kDecThreads / (hd / 8);
-  const size_t attn = 1024 + (size_t)((maxlen + 3) & ~3) * 4 + rpb * hd * 4 + 256;
-  return stage > attn ? stage : attn;
-}
-
-// ---------------------------------------------------------------------------
 // phases
 // ---------------------------------------------------------------------------
 enum Phase
@@ -1123,56 +740,6 @@ enum Phase
   PH_ARGMAX,
   PH_GEMV // a stand-alone y = W x (+ residual) on the down projection's path
 };
-
-template <bool COH>
-__device__ __forceinline__ void
-final_argmax (const Params &p, int G, uint8_t *lds)
-{
-  // G per-workgroup partials -> first maximum
-  float v = -INFINITY;
-  uint32_t idx = 0xffffffffu;
-  for (int i = threadIdx.x; i < G; i += kDecThreads)
-    {
-      const float pv = __uint_as_float (
-          ld_u32<COH> ((const uint32_t *)(p.s.amax_val + i)));
-      const uint32_t pi = ld_u32<COH> (p.s.amax_idx + i);
-      if (better (pv, pi, v, idx))
-        v = pv, idx = pi;
-    }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    {
-      const float ov = __shfl_xor (v, o, 64);
-      const uint32_t oi = __shfl_xor (idx, o, 64);
-      if (better (ov, oi, v, idx))
-        v = ov, idx = oi;
-    }
-  float *bv = (float *)lds;
-  uint32_t *bi = (uint32_t *)(lds + 64);
-  if ((threadIdx.x & 63) == 0)
-    {
-      bv[threadIdx.x >> 6] = v;
-      bi[threadIdx.x >> 6] = idx;
-    }
-  __syncthreads ();
-  if (threadIdx.x == 0)
-    {
-      for (int w = 1; w < kDecWaves; ++w)
-        if (better (bv[w], bi[w], v, idx))
-          v = bv[w], idx = bi[w];
-      const uint32_t id = idx == 0xffffffffu ? 0u : idx;
-      if (p.loop)
-        {
-          // hand the token to the next replay of the step
-          const uint32_t i = ldg (p.loop), ps = ldg (p.loop + 1);
-          stg (p.ids + i + 1, id);
-          stg ((uint32_t *)p.loop, i + 1);
-          stg ((uint32_t *)p.loop + 1, ps + 1);
-        }
-      else
-        stg (p.next_tok, id);
-    }
-}
 
 // ---------------------------------------------------------------------------
 // overlapped launches
@@ -1834,284 +1401,6 @@ decode_phase_kernel (const Params p, const vkl_layer_weights lw, int layer,
   run_phase<false, WT> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
 }
 
-// overlapped launches: two of these are resident per compute unit
-template <int PHASE>
-__global__ __launch_bounds__ (kDecThreads, 4) void
-decode_phase_overlap_kernel (const Params p, const vkl_layer_weights lw,
-                             int layer, int G)
-{
-  extern __shared__ __align__ (16) uint8_t lds[];
-  run_phase<true> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
-}
-
-// ---------------------------------------------------------------------------
-// persistent mode: one launch per token, phases separated by grid barriers
-// ---------------------------------------------------------------------------
-// All G workgroups are resident (G = number of compute units, one workgroup
-// each).  A barrier is a monotonically increasing arrival counter in device
-// memory: workgroup-level s_barrier, one relaxed agent-scope atomic add by
-// thread 0, which then polls the counter (bounded) while the other waves wait
-// on a second s_barrier.  Activations cross the barrier through agent-scope
-// relaxed atomic stores / loads, which bypass the per-XCD L2, so no cache
-// write-back or invalidate is needed.
-//
-// Waves 1..7 issue the first two weight items of the NEXT phase before they
-// enter the barrier, so HBM keeps streaming while the barrier and the
-// activation reload take place; wave 0 (which must read the counter, and whose
-// loads return in order) primes its pipeline after the barrier instead.
-// The per-layer pointer table is read-only for the lifetime of a launch:
-// reading it through the constant address space lets the compiler use scalar
-// loads (SGPR results, tracked by the scalar counter) instead of per-lane
-// vector loads whose wait would also drain every weight load in flight.
-__device__ __forceinline__ vkl_layer_weights
-load_layer (const vkl_layer_weights *table, int layer)
-{
-  typedef const __attribute__ ((address_space (4))) unsigned long long *cptr;
-  cptr t = (cptr) (table + layer);
-  vkl_layer_weights lw;
-  lw.wk = (const void *)t[0], lw.wq = (const void *)t[1];
-  lw.wv = (const void *)t[2], lw.wo = (const void *)t[3];
-  lw.w_gate = (const void *)t[4], lw.w_up = (const void *)t[5];
-  lw.w_down = (const void *)t[6];
-  lw.attn_norm = (const float *)t[7], lw.ffn_norm = (const float *)t[8];
-  lw.kcache = (void *)t[9], lw.vcache = (void *)t[10];
-  return lw;
-}
-
-struct GridSync
-{
-  uint32_t *counter; // arrivals so far
-  uint32_t *error;   // set when a wait gives up
-  uint32_t target;   // arrivals that complete the next barrier
-  uint32_t G;
-};
-
-__device__ __forceinline__ void
-grid_barrier (GridSync &g)
-{
-  // results of this phase were stored with write-through atomics; they are
-  // complete once this wave's vector-memory counter drains (the caller has
-  // not issued the next phase's prefetch yet for wave 0, see above)
-  __builtin_amdgcn_s_barrier ();
-  if (threadIdx.x == 0)
-    {
-      __hip_atomic_fetch_add (g.counter, 1u, __ATOMIC_RELAXED,
-                              __HIP_MEMORY_SCOPE_AGENT);
-      bool ok = false;
-      for (int spin = 0; spin < (1 << 22); ++spin)
-        {
-          const uint32_t v = ld_coherent_u32 (g.counter);
-          if ((int32_t)(v - g.target) >= 0)
-            {
-              ok = true;
-              break;
-            }
-          __builtin_amdgcn_s_sleep (1);
-        }
-      if (!ok)
-        st_coherent_u32 (g.error, 1u);
-    }
-  __builtin_amdgcn_s_barrier ();
-  g.target += g.G;
-}
-
-// stores of this wave complete (and every earlier load consumed)
-__device__ __forceinline__ void
-drain_vmem ()
-{
-  __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0) only
-}
-
-// kinds of phase in the flat sequence [5 per layer] + output layer
-enum Kind
-{
-  K_KQV = 0,
-  K_ATTN,
-  K_WO,
-  K_UPGATE,
-  K_DOWN,
-  K_HEAD
-};
-
-template <int HD>
-__global__ __launch_bounds__ (kDecThreads) void
-decode_mega_kernel (const Params p, int G, uint32_t sync_base)
-{
-  extern __shared__ __align__ (16) uint8_t lds[];
-  const vkl_decode_model &m = p.m;
-  const int wg = (int)blockIdx.x;
-  const int dim = m.dim, ffn = m.ffn, L = m.n_layers;
-  uint16_t *xl = (uint16_t *)lds;
-  GridSync gs = { p.s.sync, p.s.sync + 1, sync_base + (uint32_t)G, (uint32_t)G };
-  const int depth = (threadIdx.x >> 6) == 0 ? 0 : 2; // see the comment above
-
-  PipeState ps;
-  PipeBuf A, B;
-  XRegs x;
-  NormRegs nw;
-
-  // K/Q/V of layer 0 has no barrier in front of it: every wave primes its
-  // pipeline (the activation, the token's embedding row, is fetched in the
-  // loop below like any other)
-  {
-    const vkl_layer_weights lw = load_layer (m.layers, 0);
-    Gemv<true>::begin (ps, A, B, 1, qmat (lw.wk, dim, dim),
-                       qmat (lw.wq, dim, dim), qmat (lw.wv, dim, dim), dim,
-                       dim, wg, G, 2);
-  }
-
-  // Each call below appears once in the loop body on purpose: the compiler
-  // inlines every call site, and the whole kernel has to stay inside the
-  // 64 KiB instruction cache.
-  const int nph = 5 * L + 1;
-  for (int ph = 0; ph < nph; ++ph)
-    {
-      const int layer = ph < 5 * L ? ph / 5 : L - 1;
-      const int kind = ph < 5 * L ? ph - 5 * layer : K_HEAD;
-      const vkl_layer_weights lw = load_layer (m.layers, layer);
-#ifdef VKL_TRACE
-#define VKL_TRM(slot)                                                         \
-  if (threadIdx.x == 0 && p.trace)                                            \
-    p.trace[((size_t)ph * 1024 + wg) * 8 + (slot)] = wall_clock64 ();
-#else
-#define VKL_TRM(slot)
-#endif
-      VKL_TRM (0);
-      if (kind == K_ATTN)
-        {
-          if (wg < m.n_heads)
-            {
-              // nothing is in flight in these workgroups (see below); saying
-              // so lets the attention code use the buffers' registers
-              A = PipeBuf{};
-              B = PipeBuf{};
-              for (int h = wg; h < m.n_heads; h += G)
-                attention_head<HD, true> (p, lw, h, lds);
-            }
-        }
-      else
-        {
-          // activation source, its length, the norm that may precede the
-          // projection, and where the results go
-          const int K = kind == K_DOWN ? ffn : dim;
-          const bool norm = kind == K_KQV || kind == K_UPGATE || kind == K_HEAD;
-          const float *nwp = kind == K_KQV ? lw.attn_norm
-                             : (kind == K_UPGATE ? lw.ffn_norm : m.output_norm);
-          const float eps = kind == K_HEAD ? m.final_eps : m.eps;
-          // x and nw are (re)defined on every path, so neither stays live
-          // around the loop
-          if (ph == 0)
-            {
-              uint32_t tok = ld_coherent_u32 (p.tok);
-              if (tok >= (uint32_t)m.vocab)
-                tok = 0;
-              issue_embed_q8 (qmat (m.tok_embd, m.vocab, dim), tok, dim, x);
-            }
-          else if (kind == K_DOWN)
-            issue_x32<true> ((const uint32_t *)p.s.t, K, x);
-          else
-            issue_x<true> (kind == K_WO ? p.s.att : p.s.x, K, x);
-          if (norm)
-            issue_norm (nwp, dim, nw);
-          else
-            nw = NormRegs{};
-          Gemv<true>::prime (ps, A, B, 2);
-          if (ph == 0)
-            {
-              dequant_embed (x);
-              if (wg == 0) // the residual stream starts as the embedding row
-                {
-#pragma unroll
-                  for (int j = 0; j < 4; ++j)
-                    {
-                      const int idx = threadIdx.x + j * kDecThreads;
-                      if (idx * 8 < dim)
-                        {
-                          uint32_t *dst = (uint32_t *)p.s.x + idx * 4;
-                          st_coherent_u32 (dst, x.v[j].x);
-                          st_coherent_u32 (dst + 1, x.v[j].y);
-                          st_coherent_u32 (dst + 2, x.v[j].z);
-                          st_coherent_u32 (dst + 3, x.v[j].w);
-                        }
-                    }
-                }
-            }
-          float *red = (float *)(lds + (size_t)K * 2);
-          VKL_TRM (1);
-          if (norm)
-            finish_x<true> (x, K, xl, nw, eps, red);
-          else
-            finish_x<false> (x, K, xl, nw, 0.f, red);
-          VKL_TRM (2);
-          Epilogue e = {};
-          if (kind == K_KQV)
-            e.y[0] = p.s.kqv;
-          else if (kind == K_UPGATE)
-            e.y[0] = p.s.t;
-          else if (kind == K_HEAD)
-            {
-              e.y[0] = p.s.logits16, e.y32 = p.logits32;
-              e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
-            }
-          else
-            e.y[0] = p.s.x, e.residual = p.s.x;
-          Gemv<true>::run (ps, A, B, xl, e, red);
-        }
-      VKL_TRM (3);
-      if (ph + 1 == nph)
-        break;
-      // this phase's stores are complete; start the next projection's weights
-      // (after K/Q/V that is Wo, which streams while attention runs)
-      drain_vmem ();
-      VKL_TRM (4);
-      // Workgroups that run an attention head start Wo after it (the
-      // attention code needs the registers the pipeline buffers would hold);
-      // all others start Wo right after K/Q/V.
-      const bool attn_wg = wg < m.n_heads;
-      if (kind == K_ATTN ? attn_wg : !(kind == K_KQV && attn_wg))
-        {
-          int mode = 0, N = dim, K = dim;
-          QMat a, b, c;
-          if (kind == K_KQV || kind == K_ATTN)
-            a = b = c = qmat (lw.wo, dim, dim);
-          else if (kind == K_WO)
-            {
-              mode = 2, N = ffn;
-              a = c = qmat (lw.w_up, ffn, dim);
-              b = qmat (lw.w_gate, ffn, dim);
-            }
-          else if (kind == K_UPGATE)
-            {
-              K = ffn;
-              a = b = c = qmat (lw.w_down, dim, ffn);
-            }
-          else if (layer + 1 < L)
-            {
-              const vkl_layer_weights nx = load_layer (m.layers, layer + 1);
-              mode = 1;
-              a = qmat (nx.wk, dim, dim), b = qmat (nx.wq, dim, dim);
-              c = qmat (nx.wv, dim, dim);
-            }
-          else
-            {
-              N = m.vocab;
-              a = b = c = qmat (m.output, m.vocab, dim);
-            }
-          Gemv<true>::begin (ps, A, B, mode, a, b, c, N, K, wg, G, depth);
-        }
-      VKL_TRM (5);
-      grid_barrier (gs);
-      VKL_TRM (6);
-    }
-  if (p.next_tok)
-    {
-      drain_vmem ();
-      grid_barrier (gs);
-      if (wg == 0)
-        final_argmax<true> (p, G, lds);
-    }
-}
-
 int
 check_model (const vkl_decode_model *m)
 {
@@ -2325,127 +1614,6 @@ launch_attention (const Params &p, const vkl_decode_model *m,
   return timer_mark (PH_ATTN, true, s);
 }
 
-// The arrival counter of a scratch buffer restarts from zero with every token:
-// a one-thread kernel in front of the step clears it (a fill kernel rather
-// than a memset node, so that a caller may capture the step in a graph).
-__global__ void
-reset_arrivals_kernel (uint32_t *sync)
-{
-  st_coherent_u32 (sync, 0u);
-}
-
-// Persistent launch.  The grid must be co-resident: one workgroup per compute
-// unit is checked against the occupancy the runtime reports.
-int
-launch_mega (const Params &p, int G, size_t lds, hipStream_t s)
-{
-  static size_t lds_set = 0;
-  static int resident = -1;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_mega_kernel<64>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_mega_kernel<128>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-      resident = -1;
-    }
-  if (resident < 0)
-    {
-      int per_cu = 0;
-      VKL_HIP (hipOccupancyMaxActiveBlocksPerMultiprocessor (
-          &per_cu, (const void *)decode_mega_kernel<128>, kDecThreads, lds));
-      resident = per_cu;
-    }
-  if (resident < 1)
-    return (int)hipErrorLaunchOutOfResources;
-  reset_arrivals_kernel<<<dim3 (1), dim3 (1), 0, s>>> (p.s.sync);
-  if (p.m.head_dim == 128)
-    decode_mega_kernel<128><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
-        p, G, 0u);
-  else
-    decode_mega_kernel<64><<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (
-        p, G, 0u);
-  return vkl_launch_status ();
-}
-// Overlapped launches: phases alternate between the caller's stream and a
-// second stream of the library, so two consecutive phases are resident at the
-// same time and hand over through the arrival counter (see phase_wait).
-struct OverlapState
-{
-  hipStream_t second = nullptr;
-  hipEvent_t ev_in = nullptr, ev_out = nullptr;
-};
-
-template <int PHASE>
-int
-launch_overlap (Params &p, const vkl_layer_weights &lw, int layer, int grid,
-                int G, size_t lds, hipStream_t s, uint32_t &arrivals)
-{
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_overlap_kernel<PHASE>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
-  p.wait_target = arrivals;
-  decode_phase_overlap_kernel<PHASE>
-      <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G);
-  arrivals += (uint32_t)grid;
-  return 0;
-}
-
-int
-launch_overlapped_step (Params &p, const vkl_decode_model *m, int G,
-                        size_t lds, hipStream_t s0)
-{
-  static OverlapState st;
-  if (!st.second)
-    {
-      VKL_HIP (hipStreamCreateWithFlags (&st.second, hipStreamNonBlocking));
-      VKL_HIP (hipEventCreateWithFlags (&st.ev_in, hipEventDisableTiming));
-      VKL_HIP (hipEventCreateWithFlags (&st.ev_out, hipEventDisableTiming));
-    }
-  // two workgroups of 512 threads with this much LDS must fit a compute unit
-  VKL_CHECK_ARG (2 * lds <= 160 * 1024);
-  uint32_t arrivals = 0;
-  reset_arrivals_kernel<<<dim3 (1), dim3 (1), 0, s0>>> (p.s.sync);
-  // the second stream starts after whatever the caller queued before
-  VKL_HIP (hipEventRecord (st.ev_in, s0));
-  VKL_HIP (hipStreamWaitEvent (st.second, st.ev_in, 0));
-  hipStream_t ss[2] = { s0, st.second };
-  int k = 0;
-  for (int l = 0; l < m->n_layers; ++l)
-    {
-      const vkl_layer_weights &lw = m->layers_h[l];
-      if (int e = launch_overlap<PH_KQV> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
-        return e;
-      if (int e = launch_overlap<PH_ATTN> (p, lw, l, m->n_heads, m->n_heads, lds,
-                                           ss[k++ & 1], arrivals))
-        return e;
-      if (int e = launch_overlap<PH_WO> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
-        return e;
-      if (int e = launch_overlap<PH_UPGATE> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
-        return e;
-      if (int e = launch_overlap<PH_DOWN> (p, lw, l, G, G, lds, ss[k++ & 1], arrivals))
-        return e;
-    }
-  const vkl_layer_weights none = {};
-  if (int e = launch_overlap<PH_HEAD> (p, none, 0, G, G, lds, ss[k++ & 1], arrivals))
-    return e;
-  if (p.next_tok)
-    if (int e = launch_overlap<PH_ARGMAX> (p, none, 0, 1, G, lds, ss[k++ & 1], arrivals))
-      return e;
-  // later work on the caller's stream follows both streams
-  VKL_HIP (hipEventRecord (st.ev_out, st.second));
-  VKL_HIP (hipStreamWaitEvent (s0, st.ev_out, 0));
-  return vkl_launch_status ();
-}
-
 } // namespace
 } // namespace vkl
 
@@ -2456,7 +1624,8 @@ vkl_decode_scratch_bytes (const vkl_decode_model *m)
 {
   if (!m)
     return 0;
-  return carve (nullptr, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim).bytes;
+  return carve (nullptr, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim,
+                m->n_layers).bytes;
 }
 
 extern "C" const void *
@@ -2464,7 +1633,8 @@ vkl_decode_logits_f16 (const vkl_decode_model *m)
 {
   if (!m || !m->scratch)
     return nullptr;
-  return carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim).logits16;
+  return carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim,
+                m->n_layers).logits16;
 }
 
 #ifdef VKL_TRACE
@@ -2560,9 +1730,11 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (int e = check_model (m))
     return e;
   VKL_CHECK_ARG (tok != nullptr && pos < (uint32_t)m->maxlen);
-  VKL_CHECK_ARG (mode >= 0 && mode <= 2);
-  // the persistent and overlapped modes exist for Q8_0 weights only
-  VKL_CHECK_ARG (mode == 0 || m->wtype == 8);
+  VKL_CHECK_ARG (mode >= 0 && mode <= 1);
+  // the persistent launch covers Q8_0 weights and contexts that run one
+  // workgroup per attention head; elsewhere the step runs launch by launch
+  if (mode == 1 && (m->wtype != 8 || (int)pos + 1 >= kAttnSplitMinLen))
+    mode = 0;
   static int n_cu = 0;
   if (n_cu == 0)
     {
@@ -2575,7 +1747,8 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
       = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
   Params p = {};
   p.m = *m;
-  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim,
+                m->n_layers);
   p.tok = tok;
   p.pos = pos;
   p.logits32 = logits32 ? logits32 : p.s.logits32;
@@ -2587,20 +1760,35 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.trace = g_trace;
 #endif
   hipStream_t s = (hipStream_t)stream;
+  p.wait_target = 0;
+  if (mode == 1)
+    return launch_persistent (p, n_cu, s);
   // launch-per-phase: two workgroups per compute unit (their registers and
   // LDS fit side by side), which doubles the weight bytes in flight while the
   // activation row is still being staged
-  const int G = mode == 0 ? n_cu * 2 : n_cu;
-  p.wait_target = 0;
-  if (mode == 1)
-    return launch_mega (p, G, lds, s);
-  if (mode == 2)
-    return launch_overlapped_step (p, m, G, lds, s);
+  const int G = n_cu * 2;
   if (int e = launch_step (p, m, n_cu, G, lds, s))
     return e;
   if (int e = timer_collect (s))
     return e;
   return vkl_launch_status ();
+}
+
+extern "C" int
+vkl_decode_status (const vkl_decode_model *m, void *stream)
+{
+  VKL_CHECK_ARG (m != nullptr && m->scratch != nullptr);
+  const Scratch sc = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen,
+                            m->head_dim, m->n_layers);
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t gave_up = 0;
+  VKL_HIP (hipMemcpyAsync (&gave_up, sc.sync + 1, sizeof (gave_up), hipMemcpyDeviceToHost, s));
+  VKL_HIP (hipStreamSynchronize (s));
+  if (!gave_up)
+    return 0;
+  VKL_HIP (hipMemsetAsync (sc.sync + 1, 0, sizeof (uint32_t), s));
+  VKL_HIP (hipStreamSynchronize (s));
+  return (int)hipErrorLaunchFailure;
 }
 
 namespace
@@ -2674,7 +1862,8 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
   hipStream_t s = (hipStream_t)stream;
   Params p = {};
   p.m = *m;
-  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim,
+                m->n_layers);
   p.tok = nullptr;
   p.logits32 = logits32 ? logits32 : p.s.logits32;
   p.next_tok = nullptr;
@@ -2787,7 +1976,8 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   const size_t lds = lds_bytes_needed (m->dim, m->ffn, m->maxlen, m->head_dim);
   Params p = {};
   p.m = *m;
-  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim);
+  p.s = carve (m->scratch, m->dim, m->ffn, m->vocab, m->n_heads, m->maxlen, m->head_dim,
+                m->n_layers);
   p.tok = (const uint32_t *)p.s.amax_idx; // any device word: ids >= vocab read row 0
   p.pos = pos;
   p.logits32 = p.s.logits32;

@@ -44,13 +44,33 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
   const size_t hd = attn0->kcache ().width ();
   const size_t heads = attn0->kcache ().channels ();
   const size_t ffn = blocks[0]->feed_forward ()->w1 ().height ();
-  // the fused step takes models whose matrices are all Q8_0 or all FP16
+  // The fused kernels index every layer with ONE set of dimensions and ONE
+  // matrix type: they take models whose matrices are all Q8_0 or all FP16 and
+  // whose blocks all have the shapes of block 0 (a block that is smaller or of
+  // another type would be read past its end).
   const DType wt = emb.dtype ();
-  const bool uniform = (wt == Q8_0 || wt == FP16)
-                       && out->weight ().dtype () == wt
-                       && attn0->wk ().dtype () == wt
-                       && attn0->wo ().dtype () == wt
-                       && blocks[0]->feed_forward ()->w1 ().dtype () == wt;
+  bool uniform = (wt == Q8_0 || wt == FP16) && out->weight ().dtype () == wt
+                 && out->weight ().width () == dim && out->weight ().height () == vocab_
+                 && emb.height () == vocab_;
+  auto is_mat = [wt] (Tensor &t, size_t rows, size_t cols) {
+    return t.dtype () == wt && t.channels () == 1 && t.height () == rows && t.width () == cols;
+  };
+  for (auto *b : blocks)
+    {
+      auto *a = b->attention ();
+      auto *f = b->feed_forward ();
+      uniform = uniform && is_mat (a->wk (), dim, dim) && is_mat (a->wq (), dim, dim)
+                && is_mat (a->wv (), dim, dim) && is_mat (a->wo (), dim, dim)
+                && is_mat (f->w1 (), ffn, dim) && is_mat (f->w3 (), ffn, dim)
+                && is_mat (f->w2 (), dim, ffn)
+                && a->kcache ().channels () == heads && a->kcache ().width () == hd
+                && a->kcache ().height () == attn0->kcache ().height ()
+                && a->vcache ().channels () == heads && a->vcache ().width () == hd
+                && a->vcache ().height () == attn0->kcache ().height ()
+                && b->attn_norm ()->weight ().size () == dim
+                && b->ffn_norm ()->weight ().size () == dim;
+    }
+  uniform = uniform && out->norm ()->weight ().size () == dim;
   // norm weights are read as fp32 by the fused kernels
   bool norms32 = out->norm ()->weight ().dtype () == FP32;
   for (auto *b : blocks)
@@ -156,6 +176,19 @@ DecodePlan::loop (uint32_t *ids, size_t pos0, size_t n_steps)
 }
 
 absl::Status
+DecodePlan::check ()
+{
+  if (!usable_ || mode_ != 1)
+    return absl::OkStatus ();
+  if (int e = vkl_decode_status (&desc_, gpu_->stream ()))
+    return absl::InternalError (absl::StrFormat (
+        "persistent decode step: a wait between workgroups gave up (%s); the GPU must not be "
+        "shared while such a launch runs",
+        vkl_error_string (e)));
+  return absl::OkStatus ();
+}
+
+absl::Status
 DecodePlan::adopt_logits (Tensor logits32)
 {
   if (logits32.dtype () != FP32 || logits32.size () < vocab_)
@@ -173,7 +206,8 @@ DecodePlan::read_logits (float *dst)
   VKLLAMA_STATUS_OK (hip_status (
       "downloading logits",
       vkl_memcpy_d2h (dst, p, vocab_ * sizeof (float), gpu_->stream ())));
-  return hip_status ("downloading logits", vkl_stream_sync (gpu_->stream ()));
+  VKLLAMA_STATUS_OK (hip_status ("downloading logits", vkl_stream_sync (gpu_->stream ())));
+  return check ();
 }
 
 absl::Status

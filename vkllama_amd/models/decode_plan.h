@@ -36,6 +36,9 @@ struct DecodePlan
   // ids is device memory, ids[0] the first input token
   absl::Status loop (uint32_t *ids, size_t pos0, size_t n_steps);
   int mode () const { return mode_; }
+  // after the stream has been synchronised: did a persistent launch (mode 1)
+  // give up a wait?  (vkl_decode_status)
+  absl::Status check ();
   // copies the fp32 logits of the last step (fused or adopted) to the host
   absl::Status read_logits (float *dst);
   // remember the fp32 logits tensor of an operator-chain pass

@@ -562,6 +562,7 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
   if (int e = vkl_stream_sync (s))
     return absl::InternalError (vkl_error_string (e));
   const auto t2 = clock::now ();
+  VKLLAMA_STATUS_OK (plan_->check ());
   // run deferred work the operator chain may have queued
   VKLLAMA_STATUS_OK (input_command_->wait ());
   for (auto *c : block_commands_)
