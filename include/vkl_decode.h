@@ -73,6 +73,15 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
  * counterpart in the reference, which has no persistent kernels. */
 int vkl_decode_status (const vkl_decode_model *m, void *stream);
 
+/* From which context length on the attention phase runs in its split form
+ * (each head's rows over several workgroups; scores / values / combine
+ * launches) instead of one workgroup per head.  0 restores the default (1024,
+ * the measured break-even); a value beyond the context length never splits.
+ * Process-wide; a testing and measuring aid without counterpart in the
+ * reference.  Graphs captured by vkl_decode_loop hold the form they were
+ * captured with. */
+int vkl_decode_set_attn_split (int min_len);
+
 /* n_steps greedy tokens without a host round trip per token: step i reads
  * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
  * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the

@@ -1,6 +1,7 @@
 """Writes the committed fixtures under tests/golden/ from the CPU oracle.
 
 Run from the repository root: python tests/golden/make_golden.py
+(and once more with --llama2-7b for the fixture of the 7B-shape workload).
 The reference ships no golden vectors for this path (its tests draw unseeded
 random inputs), so the fixtures hold the oracle's outputs on seeded synthetic
 inputs; tests/test_golden.py checks both the oracle (CPU) and the HIP kernels
@@ -42,6 +43,31 @@ def tiny_llama():
     print("tiny llama ids:", out["oracle_ids"][:16], "...")
 
 
+# benchmark configuration 3: the Llama-2-7B shape with Q8_0 weights
+LLAMA7B = dict(dim=4096, n_layers=32, n_heads=32, ffn=11008, vocab=32000, maxlen=4096, eps=1e-5, wtype=8)
+
+
+def llama2_7b():
+    """The first 32 greedy ids of the oracle on the 7B-shape workload of
+    bench.py (weights of seed 1234, the 32 prompt ids of the same seed).
+    About 7 GB of weights and a minute of CPU time."""
+    w = M.synth_weights(LLAMA7B, seed=1234)
+    rng = np.random.default_rng(1234)
+    prompt = rng.integers(3, 32000, 32).astype(np.uint32)
+    om = O.OracleModel(LLAMA7B, w)
+    ids, first = om.generate_greedy(prompt, 32)
+    top = np.argsort(-first, kind="stable")[:8]
+    out = {
+        "config": LLAMA7B, "weight_seed": 1234, "prompt": [int(t) for t in prompt],
+        "oracle_ids": [int(t) for t in ids],
+        "first_logits_top8_idx": [int(i) for i in top],
+        "first_logits_top8_val": [float(first[i]) for i in top],
+    }
+    with open(os.path.join(HERE, "llama2_7b_q8_0_c3_greedy.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    print("7B ids:", out["oracle_ids"])
+
+
 def ops():
     rng = np.random.default_rng(2024)
     d = {}
@@ -78,5 +104,8 @@ def ops():
 
 
 if __name__ == "__main__":
-    ops()
-    tiny_llama()
+    if "--llama2-7b" in sys.argv:
+        llama2_7b()
+    else:
+        ops()
+        tiny_llama()

@@ -31,6 +31,9 @@ namespace vkl
 using namespace dec;
 namespace
 {
+// contexts from this length on run the split form of the attention phase
+int g_attn_split_min = kAttnSplitMinLen;
+
 // The activation row (K fp16 values, K a multiple of 32, K <= 16384) is
 // fetched into registers first: thread t holds the 8-element chunks t,
 // t+512, t+1024, t+1536.  Issued before any weight load, these are the oldest
@@ -1583,15 +1586,19 @@ launch_attention (const Params &p, const vkl_decode_model *m,
   // p.pos is the position of a single step, or the last position of the
   // steps a replayed loop will cover in this form (the LDS need grows with it)
   const int L = (int)p.pos + 1;
-  if (L < kAttnSplitMinLen)
+  if (L < g_attn_split_min)
     return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
-  // enough chunks to occupy the GPU, and, up to the bound, so many that a
-  // chunk's rows are all in flight at once (kAttnSweeps sweeps of 256 lanes)
+  // Enough chunks to occupy the GPU, and, up to the bound, so many that the
+  // rows of a chunk are all in flight at once (kAttnSweeps sweeps of 256
+  // lanes) at the longest context.  The count depends on the model and the
+  // GPU only, not on the position: the parts of a head are then added in the
+  // same grouping whether a step is launched by itself or replayed from a
+  // graph that was captured for the longest context.
   int C = (2 * n_cu + m->n_heads - 1) / m->n_heads;
   const int rows_in_flight = kAttnSweeps * kAttnThreads / (m->head_dim / 8);
-  C = std::max (C, (L + rows_in_flight - 1) / rows_in_flight);
+  C = std::max (C, (m->maxlen + rows_in_flight - 1) / rows_in_flight);
   C = C < 1 ? 1 : (C > kAttnChunks ? kAttnChunks : C);
-  const int R = (L + C - 1) / C;
+  const int R = (m->maxlen + C - 1) / C; // most rows of a chunk
   if (R > kAttnChunkRows) // (contexts beyond 32768 positions)
     return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
   const size_t lds_a = 1024 + 64 + (size_t)R * 4;
@@ -1733,7 +1740,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   VKL_CHECK_ARG (mode >= 0 && mode <= 1);
   // the persistent launch covers Q8_0 weights and contexts that run one
   // workgroup per attention head; elsewhere the step runs launch by launch
-  if (mode == 1 && (m->wtype != 8 || (int)pos + 1 >= kAttnSplitMinLen))
+  if (mode == 1 && (m->wtype != 8 || (int)pos + 1 >= g_attn_split_min))
     mode = 0;
   static int n_cu = 0;
   if (n_cu == 0)
@@ -1772,6 +1779,14 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (int e = timer_collect (s))
     return e;
   return vkl_launch_status ();
+}
+
+extern "C" int
+vkl_decode_set_attn_split (int min_len)
+{
+  VKL_CHECK_ARG (min_len >= 0);
+  g_attn_split_min = min_len == 0 ? kAttnSplitMinLen : std::max (min_len, 2);
+  return 0;
 }
 
 extern "C" int
@@ -1886,10 +1901,10 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
     {
       // steps [done, upto) share one form of the attention phase
       const int L_first = (int)pos0 + done + 1;
-      const int long_ctx = L_first >= kAttnSplitMinLen ? 1 : 0;
+      const int long_ctx = L_first >= g_attn_split_min ? 1 : 0;
       int upto = n_steps;
       if (!long_ctx)
-        upto = std::min (n_steps, kAttnSplitMinLen - 1 - (int)pos0);
+        upto = (int)std::min<long long> (n_steps, (long long)g_attn_split_min - 1 - (long long)pos0);
       StepGraph *g = nullptr, *lru = &g_graphs[0];
       for (StepGraph &c : g_graphs)
         {
@@ -1906,7 +1921,8 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
           drop_graph (*g);
           // the position only sizes the attention launch: the largest one
           // this form will see
-          p.pos = long_ctx ? (uint32_t)m->maxlen - 1 : (uint32_t)kAttnSplitMinLen - 2;
+          p.pos = long_ctx ? (uint32_t)m->maxlen - 1
+                           : (uint32_t)std::min (g_attn_split_min - 2, m->maxlen - 1);
           hipError_t e = hipStreamBeginCapture (s, hipStreamCaptureModeThreadLocal);
           if (e != hipSuccess)
             {

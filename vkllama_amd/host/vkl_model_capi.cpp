@@ -227,6 +227,11 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_decode_graph (value != 0);
   else if (n == "phase_timing")
     vkl_decode_phase_timing (value);
+  else if (n == "attn_split_min")
+    {
+      if (vkl_decode_set_attn_split (value))
+        return fail (m, absl::InvalidArgumentError ("attn_split_min must not be negative"));
+    }
   else
     return fail (m, absl::InvalidArgumentError ("unknown option " + n));
   return 0;
