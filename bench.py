@@ -47,23 +47,47 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
 TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96185914}
+TRAFFIC_SOURCE = "profiles/decode_phase_kernels_llama2-7b-q8_0_hbm_traffic.txt"
 
 
-def cpu_baseline(cfg, weights, n_tokens):
+def cpu_baseline(cfg, weights, n_tokens, gpu_model=None, n_parity=16):
     """The CPU oracle (a plain-C restatement of the reference's arithmetic,
-    OpenMP over output rows) decoding n_tokens after a 4-token prompt."""
+    OpenMP over output rows) decoding n_tokens after a 4-token prompt.  With a
+    GPU model of the same weights the first n_parity steps are also run on the
+    GPU, on the oracle's own token sequence, and compared: largest deviation of
+    a logit relative to the largest logit, and how often the arg-max agrees."""
     from oracle import oracle as O
     om = O.OracleModel(cfg, weights)
-    om.forward(np.array([5, 17, 99, 3], np.uint32), 0)
+    head = np.array([5, 17, 99, 3], np.uint32)
+    om.forward(head, 0)
+    parity = None
+    if gpu_model is not None:
+        gpu_model.forward(head, 0)
+        parity = {"against": "the CPU oracle on the same weights, step by step on the oracle's own ids",
+                  "steps": 0, "argmax_equal": 0, "max_rel_logit_err": 0.0,
+                  "largest_oracle_margin_where_argmax_differs": 0.0}
     tok, pos = 7, 4
-    t0 = time.perf_counter()
-    for _ in range(n_tokens):
+    dt = 0.0
+    for i in range(n_tokens):
+        t0 = time.perf_counter()
         logits = om.forward([tok], pos)
+        dt += time.perf_counter() - t0
+        if parity is not None and i < n_parity:
+            got = gpu_model.forward([tok], pos)
+            parity["steps"] += 1
+            parity["max_rel_logit_err"] = max(parity["max_rel_logit_err"],
+                                              float(np.abs(got - logits).max() / np.abs(logits).max()))
+            g, o = int(np.argmax(got)), int(np.argmax(logits))
+            parity["argmax_equal"] += int(g == o)
+            if g != o:
+                parity["largest_oracle_margin_where_argmax_differs"] = max(
+                    parity["largest_oracle_margin_where_argmax_differs"], float(logits[o] - logits[g]))
         tok = int(np.argmax(logits))
         pos += 1
-    dt = time.perf_counter() - t0
     om.close()
-    return n_tokens / dt, dt
+    if parity is not None:
+        parity["max_rel_logit_err"] = round(parity["max_rel_logit_err"], 5)
+    return n_tokens / dt, dt, parity
 
 
 def bench_single_matmul(args):
@@ -283,6 +307,8 @@ def main():
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC.get((args.workload, dom)),
+                     "traffic_source": ("quoted from the counter runs summarised in " + TRAFFIC_SOURCE
+                                        + ", not measured by this run") if (args.workload, dom) in TRAFFIC else None,
                      "kernel": dom_kernel,
                      "avg_launch_us": round(dom_us, 3), "launches_timed": dom_n,
                      "avg_launch_us_with_event_pair": dom_pair_us,
@@ -293,19 +319,21 @@ def main():
         "load_seconds": {"synthesize": round(t_synth, 1), "upload": round(t_load, 1)},
         "first_ids": [int(t) for t in ids[:8]],
     }
-    m.close()
 
     cpu_tokens = args.cpu_tokens
     if cpu_tokens < 0:
         cpu_tokens = 128 if cfg["dim"] >= 4096 else 1024
     cpu_tokens = min(cpu_tokens, cfg["maxlen"] - 8)     # 4-token prompt, then one position per token
     if cpu_tokens > 0:
-        v, dt = cpu_baseline(cfg, weights, cpu_tokens)
+        m.set_option("decode_graph", args.decode_graph)
+        v, dt, parity = cpu_baseline(cfg, weights, cpu_tokens, m)
+        result["parity"] = parity
         result["cpu_baseline"] = {
             "value": round(v, 3), "unit": "tok/s", "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count())),
             "kind": "port",
             "sample": "%d greedy decode tokens at context 5..%d after a 4-token prompt, same weights (%.1f s)"
                       % (cpu_tokens, 4 + cpu_tokens, dt)}
+    m.close()
     print(json.dumps(result))
 
 

@@ -44,6 +44,43 @@ def test_reader_returns_what_the_writer_wrote(model_file):
             assert t["type"] == 8 and t["dims"] == [K, rows]
 
 
+def test_reader_on_a_file_this_repository_did_not_write():
+    """tests/golden/handmade_v3.gguf was assembled field by field from the
+    published layout of GGUF version 3 (tests/golden/make_gguf_fixture.py, which
+    does not use the writer above): the fields the model loader reads
+    (models/llama2.h:367-431 of the reference) must come back as spelled out."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "handmade_v3.gguf")
+    raw = open(path, "rb").read()
+    assert len(raw) < 1024 and raw[:4] == b"GGUF"
+    g = gguf.read_gguf(path)
+    assert g["version"] == 3
+    k = g["keys"]
+    assert list(k)[:6] == ["general.architecture", "general.alignment", "llama.context_length",
+                           "llama.block_count", "llama.attention.head_count",
+                           "llama.attention.layer_norm_rms_epsilon"]          # file order
+    assert k["general.architecture"] == (8, "llama")
+    assert k["llama.context_length"] == (4, 4096)
+    assert k["llama.block_count"] == (4, 32)
+    assert k["llama.attention.head_count"] == (4, 32)
+    assert k["llama.attention.layer_norm_rms_epsilon"][0] == 6
+    assert k["llama.attention.layer_norm_rms_epsilon"][1] == np.float32(1e-5)
+    # stepped over correctly: the types and the keys behind them
+    assert [k[n][0] for n in ("x.u8", "x.i16", "x.bool", "x.u64", "x.f64")] == [0, 3, 7, 10, 12]
+    assert k["tokenizer.ggml.tokens"][0] == 9 and k["x.i32s"][0] == 9
+    assert len(k) == 13
+    t = g["tensors"]
+    assert list(t) == ["output_norm.weight", "blk.0.attn_q.weight"]
+    n = t["output_norm.weight"]
+    assert n["type"] == 0 and n["dims"] == [4] and n["bsize"] == 16
+    assert list(n["data"].view(np.float32)) == [1.0, -2.0, 0.5, 3.25]
+    q = t["blk.0.attn_q.weight"]
+    assert q["type"] == 8 and q["dims"] == [32, 2] and q["bsize"] == 68       # 34 bytes per block of 32
+    for row in range(2):
+        blk = q["data"][34 * row:34 * row + 34]
+        assert blk[:2].view(np.float16)[0] == np.float16(0.25 * (row + 1))
+        assert list(blk[2:].view(np.int8)) == [((i * (row + 1) - 16 + 128) % 256) - 128 for i in range(32)]
+
+
 def test_malformed_files_are_refused(model_file, tmp_path):
     path, _ = model_file
     raw = open(path, "rb").read()

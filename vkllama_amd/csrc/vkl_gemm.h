@@ -31,6 +31,10 @@ struct GemmArgs
   int act;                  // 1: SiLU
   const uint16_t *residual; // y = fp16(fp16(v) + residual), stride ys
   float *y32;               // dense [M, N] widened copy
+  // fp32 scratch for partial sums (k-split forms); null: the launcher's own
+  // per-stream buffer, allocated on first use
+  float *workspace;
+  size_t workspace_bytes; // size of `workspace` (checked before every use)
 };
 
 // smallest M for which the matrix-core kernels beat one weight-streaming pass
@@ -43,6 +47,11 @@ constexpr int kGemmMinRowsBatched = 9;
 // true if the shapes/alignments are ones the kernel covers
 bool gemm_mfma_supported (const GemmArgs &a);
 int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
+// bytes of fp32 scratch gemm_mfma_launch will use for this problem (0: none)
+size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
+// frees the scratch buffer that launches on this stream allocated (the
+// stream must be idle); called when a stream is destroyed
+void gemm_release_workspace (hipStream_t s);
 
 // One token row: y[N] = W[N, K] x[K] (+ residual) on the weight-streaming
 // kernel of the decode step (vkl_decode.hip); W planar Q8_0 (wtype 8) or

@@ -699,25 +699,55 @@ skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S, int mrows)
     a.y32[(size_t)m * a.N + n] = h2f (h);
 }
 
-// fp32 workspace of the split form, one per stream, kept for the life of the
-// process
+// fp32 workspace of the split forms: one per (device, stream), allocated on
+// first use and freed when the stream is destroyed
+std::mutex g_ws_mu;
+std::map<std::pair<int, hipStream_t>, float *> g_ws_table;
+
 float *
 skinny2_workspace (hipStream_t s)
 {
-  static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, float *> table;
-  std::lock_guard<std::mutex> lock (mu);
+  std::lock_guard<std::mutex> lock (g_ws_mu);
   int dev = 0;
   if (hipGetDevice (&dev) != hipSuccess)
     return nullptr;
-  auto it = table.find ({ dev, s });
-  if (it != table.end ())
+  auto it = g_ws_table.find ({ dev, s });
+  if (it != g_ws_table.end ())
     return it->second;
   void *p = nullptr;
   if (hipMalloc (&p, kSk2Workspace) != hipSuccess)
     return nullptr;
-  table[{ dev, s }] = (float *)p;
+  g_ws_table[{ dev, s }] = (float *)p;
   return (float *)p;
+}
+
+// K slices of the few-row form
+template <int WT>
+int
+skinny2_slices (const GemmArgs &a)
+{
+  const int keff = WT == 8 ? a.Kp : a.K;
+  return (keff + kSk2Slice - 1) / kSk2Slice;
+}
+
+// raises the kernel's LDS limit once per device
+template <int WT>
+bool
+skinny2_prepare (size_t lds)
+{
+  static bool lds_set[16] = {};
+  int dev = 0;
+  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
+    return false;
+  if (!lds_set[dev])
+    {
+      if (hipFuncSetAttribute ((const void *)gemm_skinny2_kernel<WT>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+          != hipSuccess)
+        return false;
+      lds_set[dev] = true;
+    }
+  return true;
 }
 
 template <int WT>
@@ -726,22 +756,15 @@ launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
 {
   if (a.M > 32 || a.batch > 1)
     return false;
-  const int keff = WT == 8 ? a.Kp : a.K;
-  const int S = (keff + kSk2Slice - 1) / kSk2Slice;
+  const int S = skinny2_slices<WT> (a);
   const int nm = a.upgate ? 2 : a.nmat;
-  if ((size_t)nm * S * 32 * a.N * sizeof (float) > kSk2Workspace)
+  const size_t need = (size_t)nm * S * 32 * a.N * sizeof (float);
+  if (need > kSk2Workspace || (a.workspace && need > a.workspace_bytes))
     return false;
-  static bool lds_set = false;
   const size_t lds = (size_t)32 * kSk2Ldx * 2;
-  if (!lds_set)
-    {
-      if (hipFuncSetAttribute ((const void *)gemm_skinny2_kernel<WT>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-          != hipSuccess)
-        return false;
-      lds_set = true;
-    }
-  float *ws = skinny2_workspace (s);
+  if (!skinny2_prepare<WT> (lds))
+    return false;
+  float *ws = a.workspace ? a.workspace : skinny2_workspace (s);
   if (!ws)
     return false;
   gemm_skinny2_kernel<WT><<<dim3 ((unsigned)S, (unsigned)((a.N + 31) / 32), (unsigned)nm),
@@ -750,6 +773,26 @@ launch_skinny2 (const GemmArgs &a, hipStream_t s, int &err)
   skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S, 32);
   err = (int)hipGetLastError ();
   return true;
+}
+
+// parts the k range of a tile is split into (1: no split, no workspace)
+template <int BM, int WT>
+int
+tile_ksplit (const GemmArgs &a)
+{
+  const int tiles_m = (a.M + BM - 1) / BM;
+  const int tiles_n = (a.N + (a.upgate ? 64 : BN) - 1) / (a.upgate ? 64 : BN);
+  const int nz = a.upgate ? 1 : a.nmat, nm = a.upgate ? 2 : a.nmat;
+  const int nk = ((a.wtype == 8 ? a.Kp : a.K) + Geo<WT>::BK - 1) / Geo<WT>::BK;
+  if (a.batch > 1 || WT == 2)
+    return 1;
+  // (measured on the 7B shapes: a split in two pays for Q8_0 weights, whose
+  // steps are slower, and not for fp16 weights)
+  const int want = kGemmSplitTarget / (tiles_m * tiles_n * nz);
+  int ksplit = want < (WT == 8 ? 2 : 3) ? 1 : std::max (1, std::min (std::min (want, 8), nk / 8));
+  while (ksplit > 1 && (size_t)nm * ksplit * a.M * a.N * sizeof (float) > kSk2Workspace)
+    --ksplit;
+  return ksplit;
 }
 
 template <int BM, int WT>
@@ -762,21 +805,15 @@ launch_cfg (const GemmArgs &a, hipStream_t s)
   // rows against a 4096-row matrix): the k range is split as well, into parts
   // of at least eight steps, as far as the fp32 workspace holds the partial
   // tiles.  Not for batched products (there are tiles enough).
-  const int nz = a.upgate ? 1 : a.nmat, nm = a.upgate ? 2 : a.nmat;
-  const int nk = ((a.wtype == 8 ? a.Kp : a.K) + Geo<WT>::BK - 1) / Geo<WT>::BK;
-  int ksplit = 1;
+  const int nz = a.upgate ? 1 : a.nmat;
+  int ksplit = tile_ksplit<BM, WT> (a);
+  // (a caller's workspace may be smaller than the launcher's own)
+  while (a.workspace && ksplit > 1
+         && (size_t)(a.upgate ? 2 : a.nmat) * ksplit * a.M * a.N * sizeof (float) > a.workspace_bytes)
+    --ksplit;
   float *ws = nullptr;
-  if (a.batch <= 1 && WT != 2)
-    {
-      // (measured on the 7B shapes: a split in two pays for Q8_0 weights, whose
-      // steps are slower, and not for fp16 weights)
-      const int want = kGemmSplitTarget / (tiles_m * tiles_n * nz);
-      ksplit = want < (WT == 8 ? 2 : 3) ? 1 : std::max (1, std::min (std::min (want, 8), nk / 8));
-      while (ksplit > 1 && (size_t)nm * ksplit * a.M * a.N * sizeof (float) > kSk2Workspace)
-        --ksplit;
-      if (ksplit > 1 && !(ws = skinny2_workspace (s)))
-        ksplit = 1;
-    }
+  if (ksplit > 1 && !(ws = a.workspace ? a.workspace : skinny2_workspace (s)))
+    ksplit = 1;
   const int tiles = tiles_m * tiles_n * ksplit;
   const int per_xcd = (tiles + 7) / 8;
   gemm_mfma_kernel<BM, WT>
@@ -821,32 +858,84 @@ gemm_mfma_supported (const GemmArgs &a)
   return false;
 }
 
+namespace
+{
+// the few-row, weight-streaming form: up to 32 rows, one problem, no batch
+bool
+few_rows_form (const GemmArgs &a)
+{
+  return a.M <= 32 && a.batch <= 1 && a.wtype != 2 && (a.wtype == 8 || (a.K % 16) == 0);
+}
+
+// the half-height tile for few rows, and where full tiles would be too few to
+// occupy the compute units (a few hundred token rows)
+bool
+half_height_tiles (const GemmArgs &a)
+{
+  if (a.M <= 64)
+    return true;
+  const long tiles = (long)((a.M + 127) / 128) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
+                     * (a.batch > 1 ? a.batch : 1) * (a.upgate ? 1 : a.nmat);
+  return tiles < kGemmFewTiles;
+}
+} // namespace
+
 int
 gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
 {
   if (!gemm_mfma_supported (a))
     return (int)hipErrorInvalidValue;
-  bool small = a.M <= 64;
-  // up to 32 rows, one problem, no batch: the weight-streaming form (if its
-  // workspace holds the partial sums)
-  if (a.M <= 32 && a.batch <= 1 && a.wtype != 2 && (a.wtype == 8 || (a.K % 16) == 0))
+  if (few_rows_form (a))
     {
+      // (if its workspace holds the partial sums)
       int err = 0;
       if (a.wtype == 8 ? launch_skinny2<8> (a, s, err) : launch_skinny2<1> (a, s, err))
         return err;
     }
-  // the half-height tile also where full tiles would be too few to occupy the
-  // compute units (a few hundred token rows)
-  {
-    const long tiles = (long)((a.M + 127) / 128) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
-                       * (a.batch > 1 ? a.batch : 1) * (a.upgate ? 1 : a.nmat);
-    if (tiles < kGemmFewTiles)
-      small = true;
-  }
+  const bool small = half_height_tiles (a);
   if (a.wtype == 8)
     return small ? launch_cfg<64, 8> (a, s) : launch_cfg<128, 8> (a, s);
   if (a.wtype == 2)
     return small ? launch_cfg<64, 2> (a, s) : launch_cfg<128, 2> (a, s);
   return small ? launch_cfg<64, 1> (a, s) : launch_cfg<128, 1> (a, s);
 }
+
+size_t
+gemm_mfma_workspace_bytes (const GemmArgs &a)
+{
+  if (!gemm_mfma_supported (a))
+    return 0;
+  const size_t nm = a.upgate ? 2 : a.nmat;
+  if (few_rows_form (a))
+    {
+      const int S = a.wtype == 8 ? skinny2_slices<8> (a) : skinny2_slices<1> (a);
+      const size_t need = nm * S * 32 * a.N * sizeof (float);
+      if (need <= kSk2Workspace)
+        return need;
+    }
+  const bool small = half_height_tiles (a);
+  int ksplit;
+  if (a.wtype == 8)
+    ksplit = small ? tile_ksplit<64, 8> (a) : tile_ksplit<128, 8> (a);
+  else if (a.wtype == 2)
+    ksplit = 1;
+  else
+    ksplit = small ? tile_ksplit<64, 1> (a) : tile_ksplit<128, 1> (a);
+  return ksplit > 1 ? nm * ksplit * a.M * a.N * sizeof (float) : 0;
+}
+
+void
+gemm_release_workspace (hipStream_t s)
+{
+  std::lock_guard<std::mutex> lock (g_ws_mu);
+  for (auto it = g_ws_table.begin (); it != g_ws_table.end ();)
+    if (it->first.second == s)
+      {
+        (void)hipFree (it->second);
+        it = g_ws_table.erase (it);
+      }
+    else
+      ++it;
+}
+
 } // namespace vkl

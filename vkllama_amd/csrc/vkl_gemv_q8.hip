@@ -210,11 +210,10 @@ fill_common (GemvQ8Args &a, const void *x, int M, int N, int K, size_t xs,
 }
 
 // the same problem on the matrix cores when there are enough token rows
-bool
-try_gemm (const GemvQ8Args &a, int nmat, int upgate, hipStream_t s, int &err)
+// the problem as the matrix-core launcher takes it
+vkl::GemmArgs
+gemm_args (const GemvQ8Args &a, int nmat, int upgate)
 {
-  if (a.M < vkl::kGemmMinRows)
-    return false;
   vkl::GemmArgs g = {};
   g.x = a.x, g.xs = a.xs;
   g.M = a.M, g.N = a.N, g.K = a.K, g.Kp = a.Kp;
@@ -224,6 +223,17 @@ try_gemm (const GemvQ8Args &a, int nmat, int upgate, hipStream_t s, int &err)
   g.ys = a.ys;
   g.scale = a.scale, g.bias = a.bias, g.act = a.act;
   g.residual = a.residual, g.y32 = a.y32;
+  return g;
+}
+
+bool
+try_gemm (const GemvQ8Args &a, int nmat, int upgate, hipStream_t s, int &err,
+          float *workspace = nullptr, size_t workspace_bytes = 0)
+{
+  if (a.M < vkl::kGemmMinRows)
+    return false;
+  vkl::GemmArgs g = gemm_args (a, nmat, upgate);
+  g.workspace = workspace, g.workspace_bytes = workspace_bytes;
   if (!vkl::gemm_mfma_supported (g))
     return false;
   err = vkl::gemm_mfma_launch (g, s);
@@ -240,10 +250,14 @@ set_mat (GemvQ8Args &a, int t, const void *w, void *y)
 }
 } // namespace
 
-extern "C" int
-vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
-                 size_t xs, size_t ys, float scale, float bias, int act,
-                 const void *residual, void *y, float *y32, void *stream)
+namespace
+{
+// no_alloc: scratch comes from the library's static device array or the call
+// is refused; nothing is allocated
+int
+matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K, size_t xs,
+             size_t ys, float scale, float bias, int act, const void *residual,
+             void *y, float *y32, void *stream, bool no_alloc)
 {
   GemvQ8Args a = {};
   if (int e = fill_common (a, x, M, N, K, xs, ys))
@@ -262,10 +276,23 @@ vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
   if (M == 1 && scale == 1.0f && bias == 0.0f && act == 0 && !y32
       && ((uintptr_t)x % 16) == 0 && vkl::decode_gemv_supported (N, K, 8))
     return vkl::decode_gemv_launch (x, w_planar, 8, N, K, residual, y, (hipStream_t)stream);
+  float *workspace = nullptr;
+  size_t have = 0;
+  (void)no_alloc;
   int err = 0;
-  if (try_gemm (a, 1, 0, (hipStream_t)stream, err))
+  if (try_gemm (a, 1, 0, (hipStream_t)stream, err, workspace, have))
     return err;
   return launch<0, 1> (a, (hipStream_t)stream);
+}
+} // namespace
+
+extern "C" int
+vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
+                 size_t xs, size_t ys, float scale, float bias, int act,
+                 const void *residual, void *y, float *y32, void *stream)
+{
+  return matmul_q8_0 (x, w_planar, M, N, K, xs, ys, scale, bias, act, residual, y, y32, stream,
+                      false);
 }
 
 extern "C" int

@@ -1,6 +1,7 @@
 // Device, stream, memory and event entry points of the C ABI (include/vkl_hip.h).
 #include "../../include/vkl_hip.h"
 #include "vkl_common.h"
+#include "vkl_gemm.h"
 #include <string.h>
 
 extern "C" {
@@ -55,6 +56,9 @@ vkl_stream_create (void **stream)
 int
 vkl_stream_destroy (void *stream)
 {
+  // scratch that launches on this stream allocated goes with it
+  VKL_HIP (hipStreamSynchronize ((hipStream_t)stream));
+  vkl::gemm_release_workspace ((hipStream_t)stream);
   VKL_HIP (hipStreamDestroy ((hipStream_t)stream));
   return 0;
 }

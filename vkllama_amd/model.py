@@ -264,24 +264,3 @@ class Llama2:
 
     def phase_bytes(self, kind, L):
         return int(lib().vkl_model_phase_bytes(self._h, self.PHASES.index(kind), L))
-
-
-TINY_SMOKE_CFG = dict(dim=256, n_layers=2, n_heads=4, ffn=704, vocab=1024, maxlen=64, eps=1e-5, wtype=8)
-
-
-def smoke(dev=None):
-    """Tiny llama: prompt pass + a few greedy tokens, checked against the CPU
-    oracle (token ids identical, logits within fp16 noise)."""
-    from oracle import oracle as O
-    cfg = TINY_SMOKE_CFG
-    w = synth_weights(cfg, seed=7)
-    prompt = np.array([5, 17, 99, 3, 64, 8], np.uint32)
-    m = Llama2(cfg, w)
-    logits = m.forward(prompt, 0)
-    ids, _, _ = m.generate_greedy(prompt, 8)
-    om = O.OracleModel(cfg, w)
-    want_ids, want_logits = om.generate_greedy(prompt, 8)
-    err = float(np.abs(logits - want_logits).max() / max(np.abs(want_logits).max(), 1e-6))
-    assert err < 2e-2, err
-    assert list(ids) == list(want_ids), (list(ids), list(want_ids))
-    print("smoke: tiny llama prefill logits rel err %.3g, 8 greedy ids identical to the oracle" % err)
