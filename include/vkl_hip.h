@@ -103,6 +103,21 @@ int vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N,
                      int K, size_t xs, size_t ys, float scale, float bias,
                      int act, const void *residual, void *y, float *y32,
                      void *stream);
+/* vkl_matmul_q8_0 for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid it); it has no
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results, but it calls no hipMalloc / hipFree: the fp32 partial sums that the
+ * few-row and k-split kernels exchange (M from 2 up to a few hundred rows) go
+ * through a static device array of 8 MiB that every GPU the library runs on
+ * holds until the process ends (its address on a device is looked up once, at
+ * vkl_device_open or at the first call there).  A problem whose partial sums
+ * do not fit (e.g. 2..32 rows: 128 * N * ceil(K / 1024) bytes) is refused with
+ * hipErrorInvalidValue.  All calls on one GPU share the array: calls that
+ * overlap in time on one GPU (different streams) race. */
+int vkl_matmul_q8_0_noalloc (const void *x, const void *w_planar, int M,
+                             int N, int K, size_t xs, size_t ys, float scale,
+                             float bias, int act, const void *residual,
+                             void *y, float *y32, void *stream);
 /* src/ops/multiheadattention_v2.cpp:190-202, src/shaders/kqv_fp16_x_q8_0.comp */
 int vkl_kqv_q8_0 (const void *x, const void *wk, const void *wq,
                   const void *wv, int M, int N, int K, void *k, void *q,

@@ -56,6 +56,7 @@ SIGNATURES = {
     "vkl_embed_f16": (i32, [vp, u32, u32, vp, u32, u32, vp, vp]),
     "vkl_rmsnorm_f16": (i32, [vp, vp, i32, i32, f32, vp, vp]),
     "vkl_matmul_q8_0": (i32, [vp, vp, i32, i32, i32, sz, sz, f32, f32, i32, vp, vp, vp, vp]),
+    "vkl_matmul_q8_0_noalloc": (i32, [vp, vp, i32, i32, i32, sz, sz, f32, f32, i32, vp, vp, vp, vp]),
     "vkl_kqv_q8_0": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp]),
     "vkl_ffn_upgate_q8_0": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "vkl_rope_kvwrite_f16": (i32, [vp, vp, vp, i32, i32, i32, sz, i32, i32, u32, u32, vp, vp, i32, vp, vp, i32, vp]),

@@ -52,6 +52,9 @@ size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
 // frees the scratch buffer that launches on this stream allocated (the
 // stream must be idle); called when a stream is destroyed
 void gemm_release_workspace (hipStream_t s);
+// this GPU's copy of the library's static scratch array and its size in bytes
+// (resolved once per device); null if the address cannot be resolved
+float *gemm_static_scratch (size_t *bytes);
 
 // One token row: y[N] = W[N, K] x[K] (+ residual) on the weight-streaming
 // kernel of the decode step (vkl_decode.hip); W planar Q8_0 (wtype 8) or

@@ -721,6 +721,14 @@ skinny2_workspace (hipStream_t s)
   return (float *)p;
 }
 
+// Scratch for callers that must not allocate (vkl_matmul_q8_0_noalloc): a
+// file-scope device array.  Every GPU the library runs on holds its own copy
+// at its own address until the process ends; in host code the array's name is
+// only a handle for hipGetSymbolAddress, never an address to pass to a kernel.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__ (256) unsigned char scratch[kStaticScratchBytes];
+float *g_static_scratch[16] = {};
+
 // K slices of the few-row form
 template <int WT>
 int
@@ -938,4 +946,22 @@ gemm_release_workspace (hipStream_t s)
       ++it;
 }
 
+float *
+gemm_static_scratch (size_t *bytes)
+{
+  if (bytes)
+    *bytes = kStaticScratchBytes;
+  int dev = 0;
+  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
+    return nullptr;
+  if (!g_static_scratch[dev])
+    {
+      // with this device current: the address of ITS copy of the array
+      void *p = nullptr;
+      if (hipGetSymbolAddress (&p, HIP_SYMBOL (scratch)) != hipSuccess)
+        return nullptr;
+      g_static_scratch[dev] = (float *)p;
+    }
+  return g_static_scratch[dev];
+}
 } // namespace vkl

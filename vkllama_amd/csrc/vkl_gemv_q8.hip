@@ -278,7 +278,16 @@ matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K, size_t xs
     return vkl::decode_gemv_launch (x, w_planar, 8, N, K, residual, y, (hipStream_t)stream);
   float *workspace = nullptr;
   size_t have = 0;
-  (void)no_alloc;
+  if (no_alloc && M >= vkl::kGemmMinRows)
+    {
+      // the scratch the launch would use must fit the static array
+      const vkl::GemmArgs g = gemm_args (a, 1, 0);
+      workspace = vkl::gemm_static_scratch (&have);
+      if (!workspace)
+        return (int)hipErrorInvalidSymbol;
+      if (vkl::gemm_mfma_workspace_bytes (g) > have)
+        return (int)hipErrorInvalidValue;
+    }
   int err = 0;
   if (try_gemm (a, 1, 0, (hipStream_t)stream, err, workspace, have))
     return err;
@@ -293,6 +302,15 @@ vkl_matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K,
 {
   return matmul_q8_0 (x, w_planar, M, N, K, xs, ys, scale, bias, act, residual, y, y32, stream,
                       false);
+}
+
+extern "C" int
+vkl_matmul_q8_0_noalloc (const void *x, const void *w_planar, int M, int N, int K,
+                         size_t xs, size_t ys, float scale, float bias, int act,
+                         const void *residual, void *y, float *y32, void *stream)
+{
+  return matmul_q8_0 (x, w_planar, M, N, K, xs, ys, scale, bias, act, residual, y, y32, stream,
+                      true);
 }
 
 extern "C" int

@@ -21,6 +21,9 @@ vkl_device_open (int dev, vkl_device_info *info)
   VKL_HIP (hipGetDeviceCount (&n));
   VKL_CHECK_ARG (dev >= 0 && dev < n);
   VKL_HIP (hipSetDevice (dev));
+  // this device's copy of the static scratch array (vkl_matmul_q8_0_noalloc)
+  // is looked up here, once, with the device current
+  (void)vkl::gemm_static_scratch (nullptr);
   if (info)
     {
       hipDeviceProp_t p;
