@@ -67,6 +67,13 @@ enum Kind
 // written in front of every launch and read with scalar loads.  A unit is two
 // rows: rows 2u and 2u + 1 of a matrix, or row u of the up matrix and row u of
 // the gate matrix.
+// fields of vkl_layer_weights as 64-bit words (the layer table is read with
+// scalar loads, one field at a time)
+constexpr int kLwAttnNorm = offsetof (vkl_layer_weights, attn_norm) / 8;
+constexpr int kLwFfnNorm = offsetof (vkl_layer_weights, ffn_norm) / 8;
+constexpr int kLwKcache = offsetof (vkl_layer_weights, kcache) / 8;
+constexpr int kLwVcache = offsetof (vkl_layer_weights, vcache) / 8;
+
 struct PhaseRec
 {
   // int8 plane and scale plane of the first matrix; K/Q/V has three matrices,
@@ -585,7 +592,7 @@ persistent_control (const Params &p, int G, uint8_t *lds)
           if (attn_wg)
             {
               vkl_layer_weights w = {};
-              w.kcache = (void *)lwp[9], w.vcache = (void *)lwp[10];
+              w.kcache = (void *)lwp[kLwKcache], w.vcache = (void *)lwp[kLwVcache];
               VKL_PTR (ph, 0)
               psync_wait (gs, epoch - 1u, false);
               VKL_PTR (ph, 1)
@@ -612,8 +619,8 @@ persistent_control (const Params &p, int G, uint8_t *lds)
       VKL_PTR (ph, 0)
       if (norm)
         {
-          const float *nwp = kind == K_KQV ? (const float *)lwp[7]
-                             : (kind == K_UPGATE ? (const float *)lwp[8] : m.output_norm);
+          const float *nwp = kind == K_KQV ? (const float *)lwp[kLwAttnNorm]
+                             : (kind == K_UPGATE ? (const float *)lwp[kLwFfnNorm] : m.output_norm);
           copy_to_lds<false> (nwp, (uint32_t)dim * 4, l.nl, lane);
         }
       if (ph == 0)
@@ -806,7 +813,7 @@ persistent_worker (const Params &p, int G, uint8_t *lds, int wv)
           typedef const __attribute__ ((address_space (4))) unsigned long long *cptr;
           cptr lwp = (cptr)(m.layers + iph / 5);
           vkl_layer_weights w = {};
-          w.kcache = (void *)lwp[9], w.vcache = (void *)lwp[10];
+          w.kcache = (void *)lwp[kLwKcache], w.vcache = (void *)lwp[kLwVcache];
           __syncthreads (); // wave 0 has seen the K/Q/V phase complete
           for (int h = wg; h < m.n_heads; h += G)
             attention_head<HD, true> (p, w, h, lds);

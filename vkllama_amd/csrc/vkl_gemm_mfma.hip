@@ -536,7 +536,21 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
   const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
   const void *zeros = g_zero_chunk;
 
-  // all weights of the wave, then the workgroup's piece of x
+  // The workgroup's piece of x first (it comes from the caches and returns
+  // well before the weights: loads return in order), then all weights of the
+  // wave; x goes to LDS while the weights are still on their way.
+  constexpr int CPR = kSk2Slice / 8;               // chunks per x row
+  constexpr int NCH = 32 * CPR / (kSk2Waves * 64); // per thread: 8
+  uint4 xv[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kSk2Waves * 64;
+      const int row = c / CPR, k = k0 + (c % CPR) * 8;
+      const bool v = row < a.M && k + 8 <= a.K;
+      xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
+    }
+  __builtin_amdgcn_sched_barrier (0);
   uint4 wv[UN][WT == 8 ? 1 : 2];
   uint16_t dv[UN];
   const int bw = k0 / 32 + wave * UN; // first block of the wave
@@ -562,25 +576,13 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
           dv[u] = 0;
         }
     }
-  {
-    constexpr int CPR = kSk2Slice / 8;                         // chunks per x row
-    constexpr int NCH = 32 * CPR / (kSk2Waves * 64);           // per thread: 8
-    uint4 xv[NCH];
+  __builtin_amdgcn_sched_barrier (0);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i)
-      {
-        const int c = tid + i * kSk2Waves * 64;
-        const int row = c / CPR, k = k0 + (c % CPR) * 8;
-        const bool v = row < a.M && k + 8 <= a.K;
-        xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
-      }
-#pragma unroll
-    for (int i = 0; i < NCH; ++i)
-      {
-        const int c = tid + i * kSk2Waves * 64;
-        *(uint4 *)(xs + (c / CPR) * kSk2Ldx + (c % CPR) * 8) = xv[i];
-      }
-  }
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kSk2Waves * 64;
+      *(uint4 *)(xs + (c / CPR) * kSk2Ldx + (c % CPR) * 8) = xv[i];
+    }
   __syncthreads ();
 
   float16v acc;
