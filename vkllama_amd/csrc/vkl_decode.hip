@@ -50,7 +50,6 @@ struct NormRegs
   uint4 w[4][2]; // 8 fp32 weights per chunk
 };
 
-template <bool COH>
 __device__ __forceinline__ void
 issue_x (const uint16_t *src, int K, XRegs &x)
 {
@@ -60,50 +59,7 @@ issue_x (const uint16_t *src, int K, XRegs &x)
       const int idx = threadIdx.x + j * kDecThreads;
       x.v[j] = make_uint4 (0, 0, 0, 0);
       if (idx * 8 < K)
-        {
-          if (COH)
-            {
-              const uint32_t *s32 = (const uint32_t *)src + idx * 4;
-              x.v[j] = make_uint4 (ld_coherent_u32 (s32), ld_coherent_u32 (s32 + 1),
-                                   ld_coherent_u32 (s32 + 2), ld_coherent_u32 (s32 + 3));
-            }
-          else
-            x.v[j] = ldg4 (src + idx * 8);
-        }
-    }
-}
-
-// the same from a row stored as one 32-bit word per element (fp16 in the low
-// half)
-template <bool COH>
-__device__ __forceinline__ void
-issue_x32 (const uint32_t *src, int K, XRegs &x)
-{
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    {
-      const int idx = threadIdx.x + j * kDecThreads;
-      x.v[j] = make_uint4 (0, 0, 0, 0);
-      if (idx * 8 < K)
-        {
-          uint32_t w[8];
-          if (COH)
-            {
-#pragma unroll
-              for (int i = 0; i < 8; ++i)
-                w[i] = ld_coherent_u32 (src + idx * 8 + i);
-            }
-          else
-            {
-              const uint4 a = ldg4 (src + idx * 8), b = ldg4 (src + idx * 8 + 4);
-              w[0] = a.x, w[1] = a.y, w[2] = a.z, w[3] = a.w;
-              w[4] = b.x, w[5] = b.y, w[6] = b.z, w[7] = b.w;
-            }
-          x.v[j] = make_uint4 ((w[0] & 0xffffu) | (w[1] << 16),
-                               (w[2] & 0xffffu) | (w[3] << 16),
-                               (w[4] & 0xffffu) | (w[5] << 16),
-                               (w[6] & 0xffffu) | (w[7] << 16));
-        }
+        x.v[j] = ldg4 (src + idx * 8);
     }
 }
 
@@ -165,30 +121,12 @@ issue_norm (const float *w, int K, NormRegs &n)
     }
 }
 
-// Parks the norm weights in LDS so that they do not occupy 32 registers while
-// a phase waits for its predecessor; finish_x reads them back from there.
-__device__ __forceinline__ void
-stash_norm (const NormRegs &n, int K, uint8_t *nl)
-{
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    {
-      const int idx = threadIdx.x + j * kDecThreads;
-      if (idx * 8 < K)
-        {
-          ((uint4 *)nl)[2 * idx] = n.w[j][0];
-          ((uint4 *)nl)[2 * idx + 1] = n.w[j][1];
-        }
-    }
-}
-
 // Writes the row to LDS as fp16; with `n` it is RMS-normalised on the way:
 // y = fp16(x * w * (1 / sqrt(mean(x^2) + eps))).  Ends with a barrier.
-template <bool NORM, bool NLDS = false>
+template <bool NORM>
 __device__ __forceinline__ void
 finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
-          float *red, const uint8_t *nl = nullptr,
-          unsigned long long *tr = nullptr)
+          float *red, unsigned long long *tr = nullptr)
 {
   float alpha = 0.f;
 #ifdef VKL_TRACE
@@ -233,9 +171,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
       if (NORM)
         {
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
-          // norm weights: from registers, or from where stash_norm parked them
-          const uint4 g0 = NLDS ? ((const uint4 *)nl)[2 * idx] : n.w[j][0];
-          const uint4 g1 = NLDS ? ((const uint4 *)nl)[2 * idx + 1] : n.w[j][1];
+          const uint4 g0 = n.w[j][0], g1 = n.w[j][1];
           const uint32_t g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
           uint32_t r[4];
 #pragma unroll
@@ -745,76 +681,31 @@ enum Phase
 };
 
 // ---------------------------------------------------------------------------
-// overlapped launches
+// one phase of the step in its general form
 // ---------------------------------------------------------------------------
-// In this mode consecutive phases are separate launches on two alternating
-// streams, so the next phase's workgroups become resident while the current
-// phase is still running: they fetch their kernel arguments, warm the
-// instruction cache and put their first two weight items in flight, and only
-// then wait (bounded) for the arrival counter to show that every workgroup of
-// the previous phases has finished.  Each workgroup adds one arrival when its
-// stores are complete.  Activations travel through write-through atomics, as
-// in the persistent kernel.  Wave 0 polls the counter, so it primes its own
-// pipeline after the wait (loads return in order).
-template <bool COH>
-__device__ __forceinline__ void
-phase_wait (const Params &p)
-{
-  if (!COH)
-    return;
-  if (threadIdx.x == 0)
-    {
-      bool ok = false;
-      for (int spin = 0; spin < (1 << 22); ++spin)
-        {
-          const uint32_t v = ld_coherent_u32 (p.s.sync);
-          if ((int32_t)(v - p.wait_target) >= 0)
-            {
-              ok = true;
-              break;
-            }
-          __builtin_amdgcn_s_sleep (1);
-        }
-      if (!ok)
-        st_coherent_u32 (p.s.sync + 1, 1u);
-    }
-  __builtin_amdgcn_s_barrier ();
-}
-
-template <bool COH>
-__device__ __forceinline__ void
-phase_signal (const Params &p)
-{
-  if (!COH)
-    return;
-  __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0): this wave's stores are done
-  __builtin_amdgcn_s_barrier ();
-  if (threadIdx.x == 0)
-    __hip_atomic_fetch_add (p.s.sync, 1u, __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Every projection phase runs in this order: activation loads, norm-weight
-// loads, first weight item (all issued back to back), then the activation is
-// normalised / written to LDS, then the weight pipeline runs.
-template <bool COH, int WT = 8>
+// Used for the phases that do not have (or need) the branch-free form below:
+// the K/Q/V projection of layer 0 (which embeds the token), attention with
+// one workgroup per head, the final arg-max, and every phase of a model
+// whose rows exceed what the direct kernels stage.  Every projection phase
+// runs in this order: activation loads, norm-weight loads, first weight item
+// (all issued back to back), then the activation is normalised / written to
+// LDS, then the weight pipeline runs.
+template <int WT = 8>
 __device__ __forceinline__ void
 run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
            int wg, int G, uint8_t *lds)
 {
+  typedef Gemv<false, WT> GV;
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
   uint16_t *xl = (uint16_t *)lds;
   const int kstage = phase == PH_DOWN || phase == PH_GEMV ? ffn : dim;
   float *red = (float *)(lds + (size_t)kstage * 2); // 2*kDecWaves words
-  uint8_t *nl = lds + (size_t)kstage * 2 + 256;     // parked norm weights
   Epilogue e = {};
   XRegs x;
   NormRegs nw;
   PipeState ps;
   PipeBuf A, B;
-  // overlapped mode: weights first, then the wait, then the activations
-  const int pre = (threadIdx.x >> 6) == 0 ? 0 : 2;
   VKL_TR (0);
   switch (phase)
     {
@@ -822,35 +713,20 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
       {
         const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
                    wv = wmat<WT> (lw.wv, dim, dim);
-        if (COH)
-          {
-            issue_norm (lw.attn_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, pre);
-            stash_norm (nw, dim, nl);
-            phase_wait<COH> (p);
-            VKL_TR (5);
-          }
         if (layer == 0)
           {
-            uint32_t tok = COH ? ld_coherent_u32 (p.tok) : ldg (step_tok (p));
+            uint32_t tok = ldg (step_tok (p));
             if (tok >= (uint32_t)m.vocab)
               tok = 0;
             if (WT == 8)
               issue_embed_q8 (wmat<WT> (m.tok_embd, m.vocab, dim), tok, dim, x);
             else
-              issue_x<false> ((const uint16_t *)m.tok_embd + (size_t)tok * dim, dim, x);
+              issue_x ((const uint16_t *)m.tok_embd + (size_t)tok * dim, dim, x);
           }
         else
-          issue_x<COH> (p.s.x, dim, x);
-        if (COH)
-          {
-            Gemv<COH, WT>::prime (ps, A, B, 2);
-          }
-        else
-          {
-            issue_norm (lw.attn_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1);
-          }
+          issue_x (p.s.x, dim, x);
+        issue_norm (lw.attn_norm, dim, nw);
+        GV::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1);
         if (layer == 0)
           {
             if (WT == 8)
@@ -864,101 +740,63 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
                     if (idx * 8 < dim)
                       {
                         uint32_t *dst = (uint32_t *)p.s.x + idx * 4;
-                        st_u32<COH> (dst, x.v[j].x);
-                        st_u32<COH> (dst + 1, x.v[j].y);
-                        st_u32<COH> (dst + 2, x.v[j].z);
-                        st_u32<COH> (dst + 3, x.v[j].w);
+                        stg (dst, x.v[j].x);
+                        stg (dst + 1, x.v[j].y);
+                        stg (dst + 2, x.v[j].z);
+                        stg (dst + 3, x.v[j].w);
                       }
                   }
               }
           }
-        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
+        finish_x<true> (x, dim, xl, nw, m.eps, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ATTN:
       {
-        phase_wait<COH> (p);
-            VKL_TR (5);
         for (int h = wg; h < m.n_heads; h += G)
           {
             if (m.head_dim == 128)
-              attention_head<128, COH> (p, lw, h, lds, VKL_TRP);
+              attention_head<128, false> (p, lw, h, lds, VKL_TRP);
             else
-              attention_head<64, COH> (p, lw, h, lds, VKL_TRP);
+              attention_head<64, false> (p, lw, h, lds, VKL_TRP);
           }
         break;
       }
     case PH_WO:
       {
         const QMat w = wmat<WT> (lw.wo, dim, dim);
-        if (COH)
-          {
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, pre, p.s.x);
-            phase_wait<COH> (p);
-            VKL_TR (5);
-          }
-        issue_x<COH> (p.s.att, dim, x);
-        if (COH)
-          Gemv<COH, WT>::prime (ps, A, B, 2);
-        else
-          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x);
-        finish_x<false> (x, dim, xl, nw, 0.f, red, nullptr, VKL_TRP);
+        issue_x (p.s.att, dim, x);
+        GV::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x);
+        finish_x<false> (x, dim, xl, nw, 0.f, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_UPGATE:
       {
         const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
-        if (COH)
-          {
-            issue_norm (lw.ffn_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, pre);
-            stash_norm (nw, dim, nl);
-            phase_wait<COH> (p);
-            VKL_TR (5);
-          }
-        issue_x<COH> (p.s.x, dim, x);
-        if (COH)
-          {
-            Gemv<COH, WT>::prime (ps, A, B, 2);
-          }
-        else
-          {
-            issue_norm (lw.ffn_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
-          }
-        finish_x<true, COH> (x, dim, xl, nw, m.eps, red, nl, VKL_TRP);
+        issue_x (p.s.x, dim, x);
+        issue_norm (lw.ffn_norm, dim, nw);
+        GV::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 1);
+        finish_x<true> (x, dim, xl, nw, m.eps, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.t;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_DOWN:
       {
         const QMat w = wmat<WT> (lw.w_down, dim, ffn);
-        if (COH)
-          {
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, pre, p.s.x);
-            phase_wait<COH> (p);
-            VKL_TR (5);
-          }
-        if (COH)
-          issue_x32<COH> ((const uint32_t *)p.s.t, ffn, x);
-        else
-          issue_x<COH> (p.s.t, ffn, x);
-        if (COH)
-          Gemv<COH, WT>::prime (ps, A, B, 2);
-        else
-          Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.s.x);
-        finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
+        issue_x (p.s.t, ffn, x);
+        GV::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.s.x);
+        finish_x<false> (x, ffn, xl, nw, 0.f, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.x, e.residual = p.s.x;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_GEMV:
@@ -966,51 +804,32 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         // y[dim] = W[dim, ffn] x[ffn] (+ residual) for a caller's operands:
         // x in s.t, y in s.x, W in w_down
         const QMat w = wmat<WT> (lw.w_down, dim, ffn);
-        issue_x<COH> (p.s.t, ffn, x);
-        Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.gemv_res);
-        finish_x<false> (x, ffn, xl, nw, 0.f, red, nullptr, VKL_TRP);
+        issue_x (p.s.t, ffn, x);
+        GV::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 1, p.gemv_res);
+        finish_x<false> (x, ffn, xl, nw, 0.f, red, VKL_TRP);
         e.y[0] = p.s.x, e.residual = p.gemv_res;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_HEAD:
       {
         const QMat w = wmat<WT> (m.output, m.vocab, dim);
-        if (COH)
-          {
-            issue_norm (m.output_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, pre);
-            stash_norm (nw, dim, nl);
-            phase_wait<COH> (p);
-            VKL_TR (5);
-          }
-        issue_x<COH> (p.s.x, dim, x);
-        if (COH)
-          {
-            Gemv<COH, WT>::prime (ps, A, B, 2);
-          }
-        else
-          {
-            issue_norm (m.output_norm, dim, nw);
-            Gemv<COH, WT>::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
-          }
-        finish_x<true, COH> (x, dim, xl, nw, m.final_eps, red, nl, VKL_TRP);
+        issue_x (p.s.x, dim, x);
+        issue_norm (m.output_norm, dim, nw);
+        GV::begin (ps, A, B, 0, w, w, w, m.vocab, dim, wg, G, 1);
+        finish_x<true> (x, dim, xl, nw, m.final_eps, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.logits16, e.y32 = p.logits32;
         e.amax_val = p.s.amax_val, e.amax_idx = p.s.amax_idx;
-        Gemv<COH, WT>::run (ps, A, B, xl, e, red);
+        GV::run (ps, A, B, xl, e, red);
         break;
       }
     case PH_ARGMAX:
-      phase_wait<COH> (p);
-            VKL_TR (5);
       if (wg == 0 && (p.next_tok || p.loop))
-        final_argmax<COH> (p, G, lds);
+        final_argmax<false> (p, G, lds);
       break;
     }
   VKL_TR (4);
-  phase_signal<COH> (p);
-  VKL_TR (6);
 }
 
 // ---------------------------------------------------------------------------
@@ -1393,7 +1212,7 @@ decode_phase_kernel (const Params p, const vkl_layer_weights lw, int layer,
                      int G)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
-  run_phase<false, WT> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
+  run_phase<WT> (p, lw, layer, PHASE, (int)blockIdx.x, G, lds);
 }
 
 int
@@ -1751,7 +1570,6 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   p.trace = g_trace;
 #endif
   hipStream_t s = (hipStream_t)stream;
-  p.wait_target = 0;
   if (mode == 1)
     return launch_persistent (p, n_cu, s);
   // launch-per-phase: two workgroups per compute unit (their registers and
@@ -1868,7 +1686,6 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
   p.next_tok = nullptr;
   p.loop = p.s.sync + 16;
   p.ids = ids;
-  p.wait_target = 0;
   p.gemv_res = nullptr;
   p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
 #ifdef VKL_TRACE
@@ -1985,7 +1802,6 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.loop = nullptr, p.ids = nullptr;
   p.gemv_res = nullptr;
   p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
-  p.wait_target = 0;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;
   const bool was_on = g_timer.on;

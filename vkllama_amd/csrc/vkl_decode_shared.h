@@ -75,7 +75,6 @@ struct Params
   uint32_t pos;
   float *logits32;    // destination of the widened logits
   uint32_t *next_tok; // may be null
-  uint32_t wait_target; // overlapped launches: arrivals to wait for
   // replayed loop (vkl_decode_loop): token index and position live in device
   // memory so that every step is the same sequence of launches
   const uint32_t *loop; // {index into ids, position}, or null
