@@ -38,7 +38,7 @@ def _both(dev, rng, M, N, K, residual=False):
 
 
 def test_noalloc_equals_the_allocating_entry_point_on_two_calls_in_a_row(dev, rng):
-    # few-row kernel: 20 rows against a 4096 x 4096 matrix (2.6 MB of partial sums) ...
+    # few-row kernel: 20 rows against a 4096 x 4096 matrix (4.2 MB of partial sums) ...
     a, b = _both(dev, rng, 20, 4096, 4096)
     assert np.isfinite(a.astype(np.float32)).all() and a.any()
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
@@ -54,7 +54,7 @@ def test_noalloc_equals_the_allocating_entry_point_on_two_calls_in_a_row(dev, rn
 
 
 def test_noalloc_refuses_what_does_not_fit(dev, rng):
-    # 32 rows x 32000 columns x 4 slices of K: 16 MB of partial sums > 8 MiB
+    # 32 rows x 32000 columns x 4 slices of K: 16 MB of partial sums > 8 MiB (32 MB with slices of 512)
     M, N, K = 32, 32000, 4096
     raw, _ = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)

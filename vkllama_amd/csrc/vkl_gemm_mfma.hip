@@ -519,7 +519,7 @@ gemm_mfma_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd,
 constexpr int kSk2Waves = 8;
 constexpr int kSk2Slice = 1024;                // k extent of a workgroup
 constexpr int kSk2Ldx = kSk2Slice + 8;         // LDS row stride of x in halves
-constexpr size_t kSk2Workspace = 32u << 20;    // bytes, per stream
+constexpr size_t kSk2Workspace = 64u << 20;    // bytes, per stream
 
 template <int WT>
 __global__ __launch_bounds__ (kSk2Waves * 64) void
@@ -652,6 +652,152 @@ gemm_skinny2_kernel (const GemmArgs a, float *ws, int S)
     }
 }
 
+// ---------------------------------------------------------------------------
+// few token rows (M <= 32), Q8_0 weights: whole cache lines per weight row
+// ---------------------------------------------------------------------------
+// The kernel above has a lane fetch 16 bytes of "its" weight row, so a load
+// instruction touches 32 rows with 32 contiguous bytes each; memory delivers
+// such pieces at well under the rate of whole lines.  Here a workgroup owns 64
+// weight rows and a 512-wide slice of K, wave (rb, kq) the 32 rows of row block
+// rb and the 128-wide quarter kq of the slice: a load instruction fetches 8
+// rows x 128 contiguous bytes (one line per row), four of them the wave's
+// whole 32 x 128 piece.  The piece goes through a private LDS region of the
+// wave (no workgroup barrier) to reach the matrix-core operand order (lane =
+// row, 16 consecutive k).  The slice of x is half as large as above for the
+// same weight bytes, and three workgroups fit a compute unit.  Partial sums
+// and their reduction are as above (slices of 512).
+constexpr int kR64Waves = 8;
+constexpr int kR64Slice = 512;
+constexpr int kR64Ldx = kR64Slice + 8;      // LDS row stride of x in halves
+constexpr int kR64Tstride = 128 + 16;       // LDS row stride of a wave's weight piece in bytes
+constexpr size_t kR64XBytes = (size_t)32 * kR64Ldx * 2;
+constexpr size_t kR64TBytes = (size_t)kR64Waves * 32 * kR64Tstride;
+constexpr size_t kR64RedBytes = (size_t)kR64Waves * 32 * 33 * 4;
+constexpr size_t kR64Lds = kR64XBytes + (kR64TBytes > kR64RedBytes ? kR64TBytes : kR64RedBytes);
+
+__global__ __launch_bounds__ (kR64Waves * 64) void
+gemm_rows64_q8_kernel (const GemmArgs a, float *ws, int S)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  uint16_t *xs = (uint16_t *)lds;                 // [32][kR64Ldx]
+  uint8_t *tr = lds + kR64XBytes;                 // [waves][32][kR64Tstride]
+  float *red = (float *)(lds + kR64XBytes);       // after the products: [waves][32][33]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rb = wave >> 2, kq = wave & 3, g = lane >> 5;
+  const int slice = blockIdx.x, mat = blockIdx.z;
+  const int n0 = blockIdx.y * 64 + rb * 32;
+  const int k0 = slice * kR64Slice, kw = k0 + kq * 128; // first k of the slice / of the wave
+  const void *zeros = g_zero_chunk;
+  const uint8_t *wq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat);
+  const uint16_t *wd = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat);
+
+  // the workgroup's piece of x first (from the caches, back before the
+  // weights: loads return in order), then the scales, then the weights
+  constexpr int CPR = kR64Slice / 8;                // 16-byte chunks per x row
+  constexpr int NCH = 32 * CPR / (kR64Waves * 64);  // per thread: 4
+  uint4 xv[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kR64Waves * 64;
+      const int row = c / CPR, k = k0 + (c % CPR) * 8;
+      const bool v = row < a.M && k + 8 <= a.K;
+      xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
+    }
+  // lane (n, g): the four block scales of row n0 + n in the wave's quarter
+  const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
+  uint16_t dv[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    {
+      const int blk = (kw >> 5) + u;
+      const bool v = blk * 32 < a.Kp;
+      dv[u] = ldg (v ? wd + (size_t)nrow * (a.Kp >> 5) + blk : (const uint16_t *)zeros);
+    }
+  __builtin_amdgcn_sched_barrier (0);
+  // load j: rows 8 j .. 8 j + 7 of the row block, 128 contiguous bytes each
+  uint4 wv[4];
+  const int lr = lane >> 3, lc = (lane & 7) * 16;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    {
+      const int row = min (n0 + j * 8 + lr, a.N - 1);
+      const bool v = kw + lc < a.Kp;
+      wv[j] = ldg16 (v ? (const void *)(wq + (size_t)row * a.Kp + kw + lc) : zeros);
+    }
+  __builtin_amdgcn_sched_barrier (0);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kR64Waves * 64;
+      *(uint4 *)(xs + (c / CPR) * kR64Ldx + (c % CPR) * 8) = xv[i];
+    }
+  // the wave's piece into its own LDS region, row-major
+  uint8_t *tw = tr + (size_t)wave * 32 * kR64Tstride;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    *(uint4 *)(tw + (j * 8 + lr) * kR64Tstride + lc) = wv[j];
+  __syncthreads ();
+
+  float16v acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+  const uint16_t *xa = xs + (lane & 31) * kR64Ldx + kq * 128 + g * 16;
+  const uint8_t *tb = tw + (lane & 31) * kR64Tstride + g * 16;
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    {
+      // operands: A = x (rows = tokens), B = weights (columns = rows n); a
+      // lane's 16 consecutive k values feed two MFMAs; Q8_0: block sum from a
+      // zero accumulator, times the block scale
+      const half8 a0 = *(const half8 *)(xa + u * 32), a1 = *(const half8 *)(xa + u * 32 + 8);
+      const uint4 wq4 = *(const uint4 *)(tb + u * 32);
+      const uint32_t w[4] = { wq4.x, wq4.y, wq4.z, wq4.w };
+      uint32_t o[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        {
+          h16x2 lo, hi;
+          i8x4_to_h2x2 (w[j], lo, hi);
+          o[2 * j] = __builtin_bit_cast (uint32_t, lo);
+          o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
+        }
+      const half8 b0 = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
+      const half8 b1 = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
+      float16v part;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        part[r] = 0.f;
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, part, 0, 0, 0);
+      const float sc = h2f (dv[u]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[r] = __builtin_fmaf (part[r], sc, acc[r]);
+    }
+
+  // add the four quarters of each row block (the weight pieces in LDS are no
+  // longer needed)
+  __syncthreads ();
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    red[(wave * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) * 33 + (lane & 31)] = acc[r];
+  __syncthreads ();
+  for (int i = tid; i < 2 * 32 * 32; i += kR64Waves * 64)
+    {
+      const int b = i >> 10, m = (i >> 5) & 31, nn = i & 31, n = blockIdx.y * 64 + b * 32 + nn;
+      if (m < a.M && n < a.N)
+        {
+          float v = 0.f;
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            v += red[((b * 4 + q) * 32 + m) * 33 + nn];
+          ws[((size_t)(mat * S + slice) * 32 + m) * a.N + n] = v;
+        }
+    }
+}
+
 // sum over the slices in order, then the epilogue of the product
 __global__ __launch_bounds__ (256) void
 skinny2_reduce_kernel (const GemmArgs a, const float *ws, int S, int mrows)
@@ -757,6 +903,40 @@ skinny2_prepare (size_t lds)
         return false;
       lds_set[dev] = true;
     }
+  return true;
+}
+
+// the whole-line form for Q8_0 weights
+bool
+launch_rows64_q8 (const GemmArgs &a, hipStream_t s, int &err)
+{
+  if (a.wtype != 8 || a.M > 32 || a.batch > 1)
+    return false;
+  const int S = (a.Kp + kR64Slice - 1) / kR64Slice;
+  const int nm = a.upgate ? 2 : a.nmat;
+  const size_t need = (size_t)nm * S * 32 * a.N * sizeof (float);
+  if (need > kSk2Workspace || (a.workspace && need > a.workspace_bytes))
+    return false;
+  static bool lds_set[16] = {};
+  int dev = 0;
+  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
+    return false;
+  if (!lds_set[dev])
+    {
+      if (hipFuncSetAttribute ((const void *)gemm_rows64_q8_kernel,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kR64Lds)
+          != hipSuccess)
+        return false;
+      lds_set[dev] = true;
+    }
+  float *ws = a.workspace ? a.workspace : skinny2_workspace (s);
+  if (!ws)
+    return false;
+  gemm_rows64_q8_kernel<<<dim3 ((unsigned)S, (unsigned)((a.N + 63) / 64), (unsigned)nm),
+                          dim3 (kR64Waves * 64), kR64Lds, s>>> (a, ws, S);
+  const size_t total = (size_t)a.M * a.N;
+  skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S, 32);
+  err = (int)hipGetLastError ();
   return true;
 }
 
@@ -897,8 +1077,10 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
     return (int)hipErrorInvalidValue;
   if (few_rows_form (a))
     {
-      // (if its workspace holds the partial sums)
       int err = 0;
+      if (launch_rows64_q8 (a, s, err))
+        return err;
+      // (if its workspace holds the partial sums)
       if (a.wtype == 8 ? launch_skinny2<8> (a, s, err) : launch_skinny2<1> (a, s, err))
         return err;
     }
@@ -918,6 +1100,14 @@ gemm_mfma_workspace_bytes (const GemmArgs &a)
   const size_t nm = a.upgate ? 2 : a.nmat;
   if (few_rows_form (a))
     {
+      // Q8_0: the whole-line form with slices of 512 if its sums fit, else
+      // the form with slices of 1024
+      if (a.wtype == 8)
+        {
+          const size_t need = nm * ((a.Kp + kR64Slice - 1) / kR64Slice) * 32 * a.N * sizeof (float);
+          if (need <= kSk2Workspace && (!a.workspace || need <= a.workspace_bytes))
+            return need;
+        }
       const int S = a.wtype == 8 ? skinny2_slices<8> (a) : skinny2_slices<1> (a);
       const size_t need = nm * S * 32 * a.N * sizeof (float);
       if (need <= kSk2Workspace)

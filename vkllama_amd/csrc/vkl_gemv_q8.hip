@@ -281,10 +281,11 @@ matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K, size_t xs
   if (no_alloc && M >= vkl::kGemmMinRows)
     {
       // the scratch the launch would use must fit the static array
-      const vkl::GemmArgs g = gemm_args (a, 1, 0);
+      vkl::GemmArgs g = gemm_args (a, 1, 0);
       workspace = vkl::gemm_static_scratch (&have);
       if (!workspace)
         return (int)hipErrorInvalidSymbol;
+      g.workspace = workspace, g.workspace_bytes = have;
       if (vkl::gemm_mfma_workspace_bytes (g) > have)
         return (int)hipErrorInvalidValue;
     }
