@@ -674,18 +674,37 @@ constexpr size_t kR64XBytes = (size_t)32 * kR64Ldx * 2;
 constexpr size_t kR64TBytes = (size_t)kR64Waves * 32 * kR64Tstride;
 constexpr size_t kR64RedBytes = (size_t)kR64Waves * 32 * 33 * 4;
 constexpr size_t kR64Lds = kR64XBytes + (kR64TBytes > kR64RedBytes ? kR64TBytes : kR64RedBytes);
+static_assert (2 * kR64RedBytes <= kR64Lds, "two passes' partial sums fit over x and the weight pieces");
+
+#ifdef VKL_TRACE
+__device__ unsigned long long *g_r64_trace = nullptr;
+#define VKL_R64T(slot)                                                        \
+  if (threadIdx.x == 0 && g_r64_trace)                                        \
+    g_r64_trace[((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + (slot)] \
+        = wall_clock64 ();
+#else
+#define VKL_R64T(slot)
+#endif
 
 __global__ __launch_bounds__ (kR64Waves * 64) void
 gemm_rows64_q8_kernel (const GemmArgs a, float *ws, int S)
 {
+  VKL_R64T (0)
+  // row blocks a wave works through one after the other (the workgroup owns
+  // 64 * PASSES weight rows, all loads requested at the start).  Two measured
+  // slower than one on the 7B shapes (8.4 k against 9.0 k tok/s on a 32-token
+  // prompt) although they double the bytes a workgroup has in flight.
+  constexpr int PASSES = 1;
   extern __shared__ __align__ (16) uint8_t lds[];
   uint16_t *xs = (uint16_t *)lds;                 // [32][kR64Ldx]
   uint8_t *tr = lds + kR64XBytes;                 // [waves][32][kR64Tstride]
-  float *red = (float *)(lds + kR64XBytes);       // after the products: [waves][32][33]
+  // after the products: [PASSES][waves][32][33] (over the weight pieces and,
+  // with two passes, the slice of x)
+  float *red = (float *)(PASSES == 1 ? lds + kR64XBytes : lds);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rb = wave >> 2, kq = wave & 3, g = lane >> 5;
   const int slice = blockIdx.x, mat = blockIdx.z;
-  const int n0 = blockIdx.y * 64 + rb * 32;
+  const int nwg = blockIdx.y * 64 * PASSES;       // first row of the workgroup
   const int k0 = slice * kR64Slice, kw = k0 + kq * 128; // first k of the slice / of the wave
   const void *zeros = g_zero_chunk;
   const uint8_t *wq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat);
@@ -704,27 +723,34 @@ gemm_rows64_q8_kernel (const GemmArgs a, float *ws, int S)
       const bool v = row < a.M && k + 8 <= a.K;
       xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
     }
-  // lane (n, g): the four block scales of row n0 + n in the wave's quarter
-  const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
-  uint16_t dv[4];
+  // pass p of wave (rb, kq): rows nwg + (2 p + rb) * 32 ... + 31.
+  // lane (n, g): the four block scales of row n of each pass in the wave's quarter
+  uint16_t dv[PASSES][4];
 #pragma unroll
-  for (int u = 0; u < 4; ++u)
+  for (int p = 0; p < PASSES; ++p)
     {
-      const int blk = (kw >> 5) + u;
-      const bool v = blk * 32 < a.Kp;
-      dv[u] = ldg (v ? wd + (size_t)nrow * (a.Kp >> 5) + blk : (const uint16_t *)zeros);
+      const int nrow = min (nwg + (2 * p + rb) * 32 + (lane & 31), a.N - 1); // clamped, masked at the end
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        {
+          const int blk = (kw >> 5) + u;
+          const bool v = blk * 32 < a.Kp;
+          dv[p][u] = ldg (v ? wd + (size_t)nrow * (a.Kp >> 5) + blk : (const uint16_t *)zeros);
+        }
     }
   __builtin_amdgcn_sched_barrier (0);
-  // load j: rows 8 j .. 8 j + 7 of the row block, 128 contiguous bytes each
-  uint4 wv[4];
+  // load j of a pass: rows 8 j .. 8 j + 7 of the row block, 128 contiguous bytes each
+  uint4 wv[PASSES][4];
   const int lr = lane >> 3, lc = (lane & 7) * 16;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    {
-      const int row = min (n0 + j * 8 + lr, a.N - 1);
-      const bool v = kw + lc < a.Kp;
-      wv[j] = ldg16 (v ? (const void *)(wq + (size_t)row * a.Kp + kw + lc) : zeros);
-    }
+  for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      {
+        const int row = min (nwg + (2 * p + rb) * 32 + j * 8 + lr, a.N - 1);
+        const bool v = kw + lc < a.Kp;
+        wv[p][j] = ldg16 (v ? (const void *)(wq + (size_t)row * a.Kp + kw + lc) : zeros);
+      }
   __builtin_amdgcn_sched_barrier (0);
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
@@ -732,70 +758,245 @@ gemm_rows64_q8_kernel (const GemmArgs a, float *ws, int S)
       const int c = tid + i * kR64Waves * 64;
       *(uint4 *)(xs + (c / CPR) * kR64Ldx + (c % CPR) * 8) = xv[i];
     }
-  // the wave's piece into its own LDS region, row-major
-  uint8_t *tw = tr + (size_t)wave * 32 * kR64Tstride;
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-    *(uint4 *)(tw + (j * 8 + lr) * kR64Tstride + lc) = wv[j];
+  VKL_R64T (1)
   __syncthreads ();
+  VKL_R64T (2)
 
-  float16v acc;
-#pragma unroll
-  for (int r = 0; r < 16; ++r)
-    acc[r] = 0.f;
+  uint8_t *tw = tr + (size_t)wave * 32 * kR64Tstride; // the wave's own LDS region
   const uint16_t *xa = xs + (lane & 31) * kR64Ldx + kq * 128 + g * 16;
   const uint8_t *tb = tw + (lane & 31) * kR64Tstride + g * 16;
+  float16v acc[PASSES];
 #pragma unroll
-  for (int u = 0; u < 4; ++u)
+  for (int p = 0; p < PASSES; ++p)
     {
-      // operands: A = x (rows = tokens), B = weights (columns = rows n); a
-      // lane's 16 consecutive k values feed two MFMAs; Q8_0: block sum from a
-      // zero accumulator, times the block scale
-      const half8 a0 = *(const half8 *)(xa + u * 32), a1 = *(const half8 *)(xa + u * 32 + 8);
-      const uint4 wq4 = *(const uint4 *)(tb + u * 32);
-      const uint32_t w[4] = { wq4.x, wq4.y, wq4.z, wq4.w };
-      uint32_t o[8];
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[p][r] = 0.f;
+      // the pass's piece into the wave's LDS region, row-major, and back in
+      // matrix-core order (a wave's LDS operations complete in order; no
+      // other wave touches the region)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
+        *(uint4 *)(tw + (j * 8 + lr) * kR64Tstride + lc) = wv[p][j];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
         {
-          h16x2 lo, hi;
-          i8x4_to_h2x2 (w[j], lo, hi);
-          o[2 * j] = __builtin_bit_cast (uint32_t, lo);
-          o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
+          // operands: A = x (rows = tokens), B = weights (columns = rows n); a
+          // lane's 16 consecutive k values feed two MFMAs; Q8_0: block sum from
+          // a zero accumulator, times the block scale
+          const half8 a0 = *(const half8 *)(xa + u * 32), a1 = *(const half8 *)(xa + u * 32 + 8);
+          const uint4 wq4 = *(const uint4 *)(tb + u * 32);
+          const uint32_t w[4] = { wq4.x, wq4.y, wq4.z, wq4.w };
+          uint32_t o[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              h16x2 lo, hi;
+              i8x4_to_h2x2 (w[j], lo, hi);
+              o[2 * j] = __builtin_bit_cast (uint32_t, lo);
+              o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
+            }
+          const half8 b0 = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
+          const half8 b1 = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
+          float16v part;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            part[r] = 0.f;
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, part, 0, 0, 0);
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, part, 0, 0, 0);
+          const float sc = h2f (dv[p][u]);
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[p][r] = __builtin_fmaf (part[r], sc, acc[p][r]);
         }
-      const half8 b0 = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
-      const half8 b1 = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
-      float16v part;
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        part[r] = 0.f;
-      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, part, 0, 0, 0);
-      const float sc = h2f (dv[u]);
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[r] = __builtin_fmaf (part[r], sc, acc[r]);
     }
 
-  // add the four quarters of each row block (the weight pieces in LDS are no
-  // longer needed)
+  // add the four quarters of each row block (x and the weight pieces in LDS
+  // are no longer needed)
+#ifdef VKL_TRACE
+  asm volatile("" ::"v"(acc[0][0]));
+#endif
+  VKL_R64T (3)
   __syncthreads ();
+  VKL_R64T (4)
 #pragma unroll
-  for (int r = 0; r < 16; ++r)
-    red[(wave * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) * 33 + (lane & 31)] = acc[r];
+  for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      red[((p * kR64Waves + wave) * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) * 33 + (lane & 31)] = acc[p][r];
   __syncthreads ();
-  for (int i = tid; i < 2 * 32 * 32; i += kR64Waves * 64)
+  for (int i = tid; i < PASSES * 2 * 32 * 32; i += kR64Waves * 64)
     {
-      const int b = i >> 10, m = (i >> 5) & 31, nn = i & 31, n = blockIdx.y * 64 + b * 32 + nn;
+      // row block b of the workgroup = pass b / 2, waves 4 (b % 2) ... + 3
+      const int b = i >> 10, m = (i >> 5) & 31, nn = i & 31, n = nwg + b * 32 + nn;
       if (m < a.M && n < a.N)
         {
           float v = 0.f;
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            v += red[((b * 4 + q) * 32 + m) * 33 + nn];
+            v += red[(((b >> 1) * kR64Waves + (b & 1) * 4 + q) * 32 + m) * 33 + nn];
           ws[((size_t)(mat * S + slice) * 32 + m) * a.N + n] = v;
         }
     }
+  VKL_R64T (5)
+}
+
+// The same with waves that do not wait for one another: a workgroup of four
+// waves owns 128 weight rows and a 512-wide slice of K, each wave 32 rows over
+// the whole slice (16 loads of 8 rows x 128 bytes, all requested at the
+// start).  The only barrier follows the staging of x; a wave then works
+// through its four 128-wide quarters as their loads arrive and stores its
+// 32 x 32 partial sums from registers: no sum over waves.  In the form above
+// the time from "weights arrived" to "workgroup done" (two barriers, the sum
+// over the waves through LDS) was twice the load latency.
+constexpr int kR128Waves = 4;
+constexpr size_t kR128Lds = kR64XBytes + (size_t)kR128Waves * 32 * kR64Tstride;
+
+__global__ __launch_bounds__ (kR128Waves * 64, 3) void
+gemm_rows128_q8_kernel (const GemmArgs a, float *ws, int S)
+{
+  VKL_R64T (0)
+  extern __shared__ __align__ (16) uint8_t lds[];
+  uint16_t *xs = (uint16_t *)lds;                 // [32][kR64Ldx]
+  uint8_t *tr = lds + kR64XBytes;                 // [waves][32][kR64Tstride]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 5;
+  const int slice = blockIdx.x, mat = blockIdx.z;
+  const int n0 = blockIdx.y * 128 + wave * 32;    // first row of the wave
+  const int k0 = slice * kR64Slice;
+  const void *zeros = g_zero_chunk;
+  const uint8_t *wq = (const uint8_t *)pick3 (a.wq[0], a.wq[1], a.wq[2], mat);
+  const uint16_t *wd = (const uint16_t *)pick3 (a.wd[0], a.wd[1], a.wd[2], mat);
+
+  // the workgroup's piece of x first (from the caches, back before the
+  // weights: loads return in order), then the scales, then the weights
+  constexpr int CPR = kR64Slice / 8;                 // 16-byte chunks per x row
+  constexpr int NCH = 32 * CPR / (kR128Waves * 64);  // per thread: 8
+  uint4 xv[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kR128Waves * 64;
+      const int row = c / CPR, k = k0 + (c % CPR) * 8;
+      const bool v = row < a.M && k + 8 <= a.K;
+      xv[i] = ldg16 (v ? (const void *)(a.x + (size_t)row * a.xs + k) : zeros);
+    }
+  // lane (n, g): the 16 block scales of row n0 + n in this slice, 32
+  // contiguous bytes (16-byte aligned: Kp is a multiple of 256 here; the
+  // second half of the row's last slice may lie past K)
+  const int nrow = min (n0 + (lane & 31), a.N - 1); // clamped, masked at the end
+  const uint16_t *dp = wd + (size_t)nrow * (a.Kp >> 5) + (k0 >> 5);
+  const uint4 d0 = ldg16 (k0 < a.Kp ? (const void *)dp : zeros);
+  const uint4 d1 = ldg16 (k0 + 256 < a.Kp ? (const void *)(dp + 8) : zeros);
+  __builtin_amdgcn_sched_barrier (0);
+  // load (q, j): rows 8 j .. 8 j + 7 of the wave's rows, the 128 contiguous
+  // bytes of quarter q each; two quarters are in flight
+  // (two arrays passed by reference: an array reached through a pointer
+  // would live in scratch memory instead of registers)
+  uint4 wva[4], wvb[4];
+  const int lr = lane >> 3, lc = (lane & 7) * 16;
+  auto issue = [&] (int q, uint4 (&dst)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      {
+        const int row = min (n0 + j * 8 + lr, a.N - 1);
+        const int k = k0 + q * 128 + lc;
+        dst[j] = ldg16 (k < a.Kp ? (const void *)(wq + (size_t)row * a.Kp + k) : zeros);
+      }
+  };
+  issue (0, wva);
+  issue (1, wvb);
+  __builtin_amdgcn_sched_barrier (0);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+    {
+      const int c = tid + i * kR128Waves * 64;
+      *(uint4 *)(xs + (c / CPR) * kR64Ldx + (c % CPR) * 8) = xv[i];
+    }
+  VKL_R64T (1)
+  __syncthreads ();
+  VKL_R64T (2)
+
+  uint8_t *tw = tr + (size_t)wave * 32 * kR64Tstride; // the wave's own LDS region
+  const uint16_t *xa = xs + (lane & 31) * kR64Ldx + g * 16;
+  const uint8_t *tb = tw + (lane & 31) * kR64Tstride + g * 16;
+  const uint32_t dw[8] = { d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w };
+  float16v acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    {
+      // the quarter's piece into the wave's LDS region, row-major, and back in
+      // matrix-core order (a wave's LDS operations complete in order; no
+      // other wave touches the region); its registers then take the quarter
+      // after next
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *(uint4 *)(tw + (j * 8 + lr) * kR64Tstride + lc) = (q & 1) ? wvb[j] : wva[j];
+      __builtin_amdgcn_sched_barrier (0);
+      if (q + 2 < 4)
+        {
+          if (q & 1)
+            issue (q + 2, wvb);
+          else
+            issue (q + 2, wva);
+        }
+      __builtin_amdgcn_sched_barrier (0);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        {
+          // operands: A = x (rows = tokens), B = weights (columns = rows n); a
+          // lane's 16 consecutive k values feed two MFMAs; Q8_0: block sum from
+          // a zero accumulator, times the block scale
+          const half8 a0 = *(const half8 *)(xa + q * 128 + u * 32);
+          const half8 a1 = *(const half8 *)(xa + q * 128 + u * 32 + 8);
+          const uint4 wq4 = *(const uint4 *)(tb + u * 32);
+          const uint32_t w[4] = { wq4.x, wq4.y, wq4.z, wq4.w };
+          uint32_t o[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              h16x2 lo, hi;
+              i8x4_to_h2x2 (w[j], lo, hi);
+              o[2 * j] = __builtin_bit_cast (uint32_t, lo);
+              o[2 * j + 1] = __builtin_bit_cast (uint32_t, hi);
+            }
+          const half8 b0 = __builtin_bit_cast (half8, make_uint4 (o[0], o[1], o[2], o[3]));
+          const half8 b1 = __builtin_bit_cast (half8, make_uint4 (o[4], o[5], o[6], o[7]));
+          float16v part;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            part[r] = 0.f;
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a0, b0, part, 0, 0, 0);
+          part = __builtin_amdgcn_mfma_f32_32x32x16_f16 (a1, b1, part, 0, 0, 0);
+          const int bi = q * 4 + u; // block of the slice
+          const float sc = h2f ((uint16_t)(dw[bi >> 1] >> (16 * (bi & 1))));
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[r] = __builtin_fmaf (part[r], sc, acc[r]);
+          // (the sums are formed here and now: left alone, the compiler moves
+          // these sixteen products down to the conditional stores at the end
+          // and keeps every block's partial sums alive until then)
+          asm volatile("" : "+v"(acc));
+        }
+    }
+#ifdef VKL_TRACE
+  asm volatile("" ::"v"(acc[0]));
+#endif
+  VKL_R64T (3)
+  // the wave's 32 x 32 partial sums: accumulator r of lane (n, g) belongs to
+  // token row (r / 4) * 8 + g * 4 + r % 4
+  const int n = n0 + (lane & 31);
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    {
+      const int m = (r >> 2) * 8 + g * 4 + (r & 3);
+      if (m < a.M && n < a.N)
+        ws[((size_t)(mat * S + slice) * 32 + m) * a.N + n] = acc[r];
+    }
+  VKL_R64T (5)
 }
 
 // sum over the slices in order, then the epilogue of the product
@@ -925,15 +1126,24 @@ launch_rows64_q8 (const GemmArgs &a, hipStream_t s, int &err)
     {
       if (hipFuncSetAttribute ((const void *)gemm_rows64_q8_kernel,
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kR64Lds)
-          != hipSuccess)
+              != hipSuccess
+          || hipFuncSetAttribute ((const void *)gemm_rows128_q8_kernel,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kR128Lds)
+                 != hipSuccess)
         return false;
       lds_set[dev] = true;
     }
   float *ws = a.workspace ? a.workspace : skinny2_workspace (s);
   if (!ws)
     return false;
-  gemm_rows64_q8_kernel<<<dim3 ((unsigned)S, (unsigned)((a.N + 63) / 64), (unsigned)nm),
-                          dim3 (kR64Waves * 64), kR64Lds, s>>> (a, ws, S);
+  // The form with independent waves reads a row's 16 scales of a slice as two
+  // aligned 16-byte words: rows of scales must be multiples of 16 bytes.
+  if ((a.Kp % 256) == 0)
+    gemm_rows128_q8_kernel<<<dim3 ((unsigned)S, (unsigned)((a.N + 127) / 128), (unsigned)nm),
+                             dim3 (kR128Waves * 64), kR128Lds, s>>> (a, ws, S);
+  else
+    gemm_rows64_q8_kernel<<<dim3 ((unsigned)S, (unsigned)((a.N + 63) / 64), (unsigned)nm),
+                            dim3 (kR64Waves * 64), kR64Lds, s>>> (a, ws, S);
   const size_t total = (size_t)a.M * a.N;
   skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, S, 32);
   err = (int)hipGetLastError ();
@@ -1157,3 +1367,11 @@ gemm_static_scratch (size_t *bytes)
   return g_static_scratch[dev];
 }
 } // namespace vkl
+
+#ifdef VKL_TRACE
+extern "C" void
+vkl_debug_set_r64_trace (void *buf)
+{
+  (void)hipMemcpyToSymbol (HIP_SYMBOL (vkl::g_r64_trace), &buf, sizeof (buf));
+}
+#endif
