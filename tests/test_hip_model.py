@@ -232,6 +232,34 @@ def test_errors(small):
         M.Llama2(cfg, short)
 
 
+def test_blocks_of_different_type_never_reach_the_fused_step():
+    """The fused decode kernels index every block with ONE dtype and ONE set of
+    shapes.  A model whose second block holds FP16 matrices while the first
+    holds Q8_0 (models/llama2.h:348-431 would load such a file) must be served
+    by the operator chain: the decode plan reports no phases (it is not
+    usable), and a decode step still equals the last row of a prompt pass."""
+    cfg = dict(SMALL, n_layers=2)
+    w = M.synth_weights(cfg, seed=17)
+    w16 = M.synth_weights(dict(cfg, wtype=1), seed=17)
+    mixed = dict(w)
+    for name in w:
+        if name.startswith("blk.1.") and not name.endswith("_norm.weight"):
+            mixed[name] = w16[name]
+    m = M.Llama2(cfg, mixed)
+    assert m.phase_bytes("upgate", 8) == 0
+    uniform = M.Llama2(cfg, w)
+    assert uniform.phase_bytes("upgate", 8) > 0
+    uniform.close()
+    prompt = np.array([5, 17, 99, 3, 64], np.uint32)
+    m.set_option("lastblock_rope_quirk", 0)
+    m.forward(prompt[:4], 0)
+    step = m.forward(prompt[4:], 4)
+    full = m.forward(prompt, 0)
+    assert np.isfinite(step).all()
+    assert logit_err(step, full) < 1e-2
+    m.close()
+
+
 @pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5), (TINY, 1234)])
 def test_persistent_decode_matches_oracle(cfg, seed):
     """decode_mode 1: one persistent launch per token; the workgroups hand the
