@@ -268,8 +268,7 @@ def main():
                 "true" if wbytes > (288 << 20) else "false", dom)
         dom_pair_us = per_phase[dom]["avg_us"]
     else:
-        # persistent / overlapped modes: one launch (or one overlapped train of
-        # launches) per token, priced as a whole
+        # persistent mode: one launch per token, priced as a whole
         dom, dom_us, dom_n, dom_bytes = None, ms_per_step * 1e3, steps, step_bytes
         dom_kernel, dom_pair_us = "decode step (all phases of one token)", None
     dom_gbs = dom_bytes / (dom_us * 1e-6) / 1e9
@@ -301,7 +300,7 @@ def main():
                 + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
                    "decode_mode": ("launch-per-phase" + (", replayed from a HIP graph" if args.decode_graph else ""),
-                                   "persistent", "overlapped-launches")[args.decode_mode],
+                                   "persistent")[args.decode_mode],
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "decode_tokens_per_second_host_interface": round(host_tok_s, 1),
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),

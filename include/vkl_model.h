@@ -72,7 +72,10 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
                                 uint32_t *out_ids_h, double *prefill_ms,
                                 double *decode_ms);
 /* options: fused one-token decode on/off, decode launch mode (0 = one launch
- * per phase, 1 = persistent, 2 = overlapped launches), the reference's last-block RoPE position quirk */
+ * per phase, 1 = one persistent launch per token), replay of the greedy loop
+ * from a HIP graph on/off, the context length from which attention is split
+ * over several workgroups per head, the reference's last-block RoPE position
+ * quirk */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);
 /* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */
 int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,

@@ -332,12 +332,9 @@ struct PipeState
 // mode 0: y = x W^T (+ residual); a unit is 2 consecutive rows of m0
 // mode 1: three matrices with three outputs; a unit is 2 rows of one of them
 // mode 2: y = silu(x Wgate^T) * (x Wup^T); a unit is row r of m0 (up) and
-//         row r of m1 (gate); the result goes out as one 32-bit word per
-//         element (fp16 in the low half) so that it can be stored with a
-//         32-bit write-through atomic
+//         row r of m1 (gate)
 // One copy of the code serves all three (the mode only steers the cheap row
-// addressing and the lane-0 epilogue), which keeps the persistent kernel
-// inside the instruction cache.
+// addressing and the lane-0 epilogue).
 // WT: 8 = planar Q8_0 weights, 1 = dense fp16 weights.  For fp16 a row is
 // addressed as 2*K bytes, so the 16-byte loads of an item are laid out exactly
 // as for the int8 plane; only the scale load and the dot product differ.
@@ -346,7 +343,7 @@ struct PipeState
 // of them then has a unit for every wave and both of its items in flight
 // from the start.  An item is always 8 loads of 16 bytes per lane: RU rows x
 // 8 / RU k-steps of 1024.
-template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
+template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
 {
   static constexpr int R = RU;     // rows per unit
   static constexpr int S = 8 / RU; // k-steps of 1024 per item
@@ -471,7 +468,7 @@ template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
     if (R == 1)
       b.res = ldg (rp + u);
     else
-      b.res = ld_u32<COH> ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
+      b.res = ldg ((const uint32_t *)(rp + (2 * u + 1 < ps.N ? 2 * u : 0)));
     // an item past the wave's last (requested all the same when begin ()
     // issues unconditionally) reads one and the same KiB for every load, so
     // that it adds nothing to the traffic
@@ -570,18 +567,12 @@ template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
         const int mat = u / half, r0 = 2 * (u - mat * half);
         // the three outputs are N elements apart
         uint16_t *y = e.y[0] + (size_t)mat * N;
-        st_u32<COH> ((uint32_t *)(y + r0),
-                     (uint32_t)f2h (v[0]) | ((uint32_t)f2h (v[R - 1]) << 16));
+        stg ((uint32_t *)(y + r0), (uint32_t)f2h (v[0]) | ((uint32_t)f2h (v[R - 1]) << 16));
         return;
       }
     if (ps.mode == 2)
       {
-        // fp16 when kernel boundaries order the phases; one 32-bit word per
-        // element where it has to be a write-through atomic
-        if (COH)
-          st_u32<COH> ((uint32_t *)e.y[0] + u, (uint32_t)f2h (silu (v[R - 1]) * v[0]));
-        else
-          stg (e.y[0] + u, f2h (silu (v[R - 1]) * v[0]));
+        stg (e.y[0] + u, f2h (silu (v[R - 1]) * v[0]));
         return;
       }
     const int r0 = 2 * u;
@@ -593,12 +584,12 @@ template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
         const uint32_t rr
             = !two ? (uint32_t)ldg (e.residual + r0)
                    : (ps.residual ? res
-                                  : ld_u32<COH> ((const uint32_t *)(e.residual + r0)));
+                                  : ldg ((const uint32_t *)(e.residual + r0)));
         h0 = f2h (h2f (h0) + h2f ((uint16_t)(rr & 0xffff)));
         h1 = f2h (h2f (h1) + h2f ((uint16_t)(rr >> 16)));
       }
     if (two)
-      st_u32<COH> ((uint32_t *)(e.y[0] + r0), (uint32_t)h0 | ((uint32_t)h1 << 16));
+      stg ((uint32_t *)(e.y[0] + r0), (uint32_t)h0 | ((uint32_t)h1 << 16));
     else
       stg (e.y[0] + r0, h0);
     if (e.y32)
@@ -658,8 +649,8 @@ template <bool COH, int WT = 8, bool NT = false, int RU = 2> struct Gemv
             for (int w = 1; w < kDecWaves; ++w)
               if (better (bv[w], bi[w], v, i))
                 v = bv[w], i = bi[w];
-            st_u32<COH> ((uint32_t *)(e.amax_val + ps.wg), __float_as_uint (v));
-            st_u32<COH> (e.amax_idx + ps.wg, i);
+            stg ((uint32_t *)(e.amax_val + ps.wg), __float_as_uint (v));
+            stg (e.amax_idx + ps.wg, i);
           }
       }
   }
@@ -695,7 +686,7 @@ __device__ __forceinline__ void
 run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
            int wg, int G, uint8_t *lds)
 {
-  typedef Gemv<false, WT> GV;
+  typedef Gemv<WT> GV;
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn;
   uint16_t *xl = (uint16_t *)lds;
@@ -851,7 +842,7 @@ run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
   // keep them from staying there for the next token.
   // Wo, down and the stand-alone product have few rows (two-row units would
   // leave half of the waves without work): one row per unit there
-  typedef Gemv<false, WT, NT && PHASE != PH_WO,
+  typedef Gemv<WT, NT && PHASE != PH_WO,
                PHASE == PH_DOWN || PHASE == PH_GEMV || PHASE == PH_WO ? 1 : 2>
       GV;
   constexpr int phase = PHASE;
