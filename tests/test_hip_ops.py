@@ -138,11 +138,14 @@ def test_matmul_q8_0_epilogue(dev, rng):
 
 # ------------------------------------------------- prompt-pass GEMM (MFMA) --
 @pytest.mark.parametrize("M,N,K", [(9, 128, 32), (16, 130, 512), (64, 256, 4096), (100, 200, 1376), (300, 1376, 512),
-                                   (129, 64, 11008), (65, 32000, 512)])
+                                   (129, 64, 11008), (65, 32000, 512),
+                                   (7, 200, 1376), (32, 129, 768), (5, 64, 256), (31, 300, 11008), (2, 1000, 5120)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
-    few-row kernel, half- and full-height tiles and the k-split."""
+    few-row kernels (K a multiple of 256 or not, a last slice that is half
+    empty, row counts that do not fill the last workgroup), half- and
+    full-height tiles and the k-split."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
