@@ -130,6 +130,37 @@ def test_infer_cli_on_a_gguf_file(model_file, capsys):
 
 
 @pytest.mark.gpu
+def test_infer_cli_with_a_sentencepiece_tokenizer(tmp_path, capsys):
+    """Text in, text out, the flow of app/llama2_infer.cpp:75-111,178-197: the
+    prompt is encoded with a sentencepiece model (BOS first), the generated ids
+    are decoded with it.  The tokenizer is trained here on a few sentences
+    (64 pieces) and the model's vocabulary has that size."""
+    spm = pytest.importorskip("sentencepiece")
+    from vkllama_amd import infer
+    cfg = dict(CFG, vocab=64)
+    w = M.synth_weights(cfg, seed=10)
+    path = str(tmp_path / "tiny64.gguf")
+    gguf.write_gguf(path, cfg, w, tokens=["<unk>", "<s>", "</s>"])
+    corpus = tmp_path / "corpus.txt"
+    corpus.write_text("\n".join(["the quick brown fox jumps over the lazy dog",
+                                 "hello world this is a test of the tokenizer",
+                                 "small models make small talk about the weather today"] * 50))
+    spm.SentencePieceTrainer.train(input=str(corpus), model_prefix=str(tmp_path / "tok"), vocab_size=64,
+                                   model_type="bpe", bos_id=1, eos_id=2, unk_id=0, minloglevel=2)
+    sp = spm.SentencePieceProcessor()
+    sp.Load(str(tmp_path / "tok.model"))
+    prompt = "hello world"
+    assert infer.main([path, "8", "--tokenizer", str(tmp_path / "tok.model"), "--prompt", prompt]) == 0
+    lines = capsys.readouterr().out.strip().split("\n")
+    ids = [int(t) for t in lines[0].split("ids:")[1].split()]
+    m = M.Llama2(cfg, w)
+    want, _, _ = m.generate_greedy(np.array([sp.bos_id()] + sp.Encode(prompt), np.uint32), 8)
+    m.close()
+    assert ids == [int(t) for t in want]
+    assert "\n".join(lines[1:]) == sp.Decode(ids)
+
+
+@pytest.mark.gpu
 def test_cpp_llama2_infer_program(model_file):
     """The C++ command-line program (the reference's app/llama2_infer.cpp flow
     on the drop-in classes) prints the same greedy ids."""
