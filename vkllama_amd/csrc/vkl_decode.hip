@@ -143,7 +143,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         {
-          const bool in = (threadIdx.x + j * kDecThreads) * 8 < K;
+          const bool in = (int)(threadIdx.x + j * kDecThreads) * 8 < K;
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -242,7 +242,7 @@ stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
       for (int j = 0; j < XCH; ++j)
         {
-          const bool in = (threadIdx.x + j * kDecThreads) * 8 < K;
+          const bool in = (int)(threadIdx.x + j * kDecThreads) * 8 < K;
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)

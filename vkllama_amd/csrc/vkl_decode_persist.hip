@@ -391,56 +391,6 @@ pconsume (const PBuf &b, int nch, int silu_out, int oi, int c, int sh0, int sh1,
     }
 }
 
-// RMSNorm of the row inside LDS by all threads, in the order of stage_row:
-// y = fp16(x * w * (1 / sqrt(mean(x^2) + eps))); nl holds the fp32 weights
-__device__ __forceinline__ void
-norm_row_lds (uint16_t *xl, const uint8_t *nl, int K, float eps, float *red)
-{
-  float s = 0.f;
-#pragma unroll 1
-  for (int j = 0; j < 4; ++j)
-    {
-      const int idx = threadIdx.x + j * kDecThreads;
-      if (idx * 8 < K)
-        {
-          const uint4 v = ((const uint4 *)xl)[idx];
-          const uint32_t w[4] = { v.x, v.y, v.z, v.w };
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            {
-              const float a = h2f ((uint16_t)(w[i] & 0xffff));
-              const float b = h2f ((uint16_t)(w[i] >> 16));
-              s += a * a;
-              s += b * b;
-            }
-        }
-    }
-  const float total = block_sum (s, red);
-  const float alpha = 1.0f / sqrtf (total / (float)K + eps);
-#pragma unroll 1
-  for (int j = 0; j < 4; ++j)
-    {
-      const int idx = threadIdx.x + j * kDecThreads;
-      if (idx * 8 < K)
-        {
-          const uint4 v = ((const uint4 *)xl)[idx];
-          const uint32_t w[4] = { v.x, v.y, v.z, v.w };
-          const uint4 g0 = ((const uint4 *)nl)[2 * idx], g1 = ((const uint4 *)nl)[2 * idx + 1];
-          const uint32_t g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
-          uint32_t r[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            {
-              const float a = h2f ((uint16_t)(w[i] & 0xffff));
-              const float b = h2f ((uint16_t)(w[i] >> 16));
-              r[i] = (uint32_t)f2h (a * __uint_as_float (g[2 * i]) * alpha)
-                     | ((uint32_t)f2h (b * __uint_as_float (g[2 * i + 1]) * alpha) << 16);
-            }
-          ((uint4 *)xl)[idx] = make_uint4 (r[0], r[1], r[2], r[3]);
-        }
-    }
-}
-
 // wave 0: `bytes` from global memory straight into LDS, 1 KiB per request
 // (lane l delivers 16 bytes at offset 16 l of the request's KiB); what lies
 // past `bytes` arrives as zeros

@@ -62,14 +62,6 @@ ldg16 (const void *p)
   return ldg4 (p);
 }
 
-// v or zero, component by component (a select between two aggregates would
-// take their addresses and push the tile registers out to scratch memory)
-__device__ __forceinline__ uint4
-keep_if (bool c, const uint4 v)
-{
-  return make_uint4 (c ? v.x : 0u, c ? v.y : 0u, c ? v.z : 0u, c ? v.w : 0u);
-}
-
 __device__ __align__ (16) const uint32_t g_zero_chunk[4] = { 0, 0, 0, 0 };
 
 template <int BM, int WT>
