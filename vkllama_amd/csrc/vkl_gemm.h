@@ -49,6 +49,11 @@ bool gemm_mfma_supported (const GemmArgs &a);
 int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
 // bytes of fp32 scratch gemm_mfma_launch will use for this problem (0: none)
 size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
+// Many token rows against dense fp16 weights: 256-row tiles staged by
+// direct-to-LDS loads (vkl_gemm_wide.hip).  gemm_mfma_launch takes this form
+// where it applies; no workspace.
+bool gemm_wide_supported (const GemmArgs &a);
+int gemm_wide_launch (const GemmArgs &a, hipStream_t s);
 // frees the scratch buffer that launches on this stream allocated (the
 // stream must be idle); called when a stream is destroyed
 void gemm_release_workspace (hipStream_t s);

@@ -1286,6 +1286,8 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
       if (a.wtype == 8 ? launch_skinny2<8> (a, s, err) : launch_skinny2<1> (a, s, err))
         return err;
     }
+  if (gemm_wide_supported (a))
+    return gemm_wide_launch (a, s);
   const bool small = half_height_tiles (a);
   if (a.wtype == 8)
     return small ? launch_cfg<64, 8> (a, s) : launch_cfg<128, 8> (a, s);
@@ -1315,6 +1317,8 @@ gemm_mfma_workspace_bytes (const GemmArgs &a)
       if (need <= kSk2Workspace)
         return need;
     }
+  if (gemm_wide_supported (a))
+    return 0;
   const bool small = half_height_tiles (a);
   int ksplit;
   if (a.wtype == 8)
