@@ -41,7 +41,7 @@ constexpr int WROWB = WBK * 2;                  // bytes of a tile row
 constexpr int WSTAGE_BYTES = (WBM + WBN) * WROWB;
 constexpr int WGPW = (WBM + WBN) / 8 / WWAVES;  // 1 KiB load instructions per wave and k-step
 constexpr int WAG = WBM / 8 / WWAVES;           // of which rows of x
-constexpr size_t kWideLds = (size_t)WSTAGES * WSTAGE_BYTES;
+constexpr size_t kWideStagesF16 = (size_t)WSTAGES * WSTAGE_BYTES;
 
 // Issue order of one quarter of a k-step: after product Q one fragment read
 // (the first NR products) and an even share of the quarter's LQ loads.
@@ -65,6 +65,119 @@ template <int V> struct WideInt
 {
   static constexpr int value = V;
 };
+
+// Epilogue through LDS (the k loop's stages are free by then): every wave parks
+// its 128 x 64 fp32 block in a region of its own, then walks it row-wise so
+// that a lane handles 8 neighbouring columns: 16-byte loads and stores, whole
+// cache lines per row, and a short loop instead of 128 unrolled elements.
+// Accumulator register q of lane l is row 8 (q/4) + 4 (l/32) + q%4, column
+// l%32 of its 32 x 32 block.
+constexpr int kWideParkLd = 68; // floats per parked row: 16-byte aligned, rows 4 banks apart
+constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 128 fp32 in rows of 64
+
+template <bool UPGATE, int TM>
+__device__ __forceinline__ void
+wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_lds, int wave, int lane,
+               int m0, int n0, int zmat, int vec)
+{
+  // waves are numbered row block first: wave = 2 wm + wn, TM x 32 rows by 64 columns each
+  constexpr int ROWS = TM * 32;
+  const int wm = wave >> 1, wn = wave & 1;
+  __builtin_amdgcn_s_barrier (); // every wave has read its last fragments
+  constexpr int LD = kWideParkLd;
+  float *park = (float *)(wide_lds + wave * (ROWS * LD * 4));
+  {
+    float *pl = park + (lane >> 5) * 4 * LD + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jn = 0; jn < WTN; ++jn)
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+          pl[(i * 32 + (q >> 2) * 8 + (q & 3)) * LD + jn * 32] = acc[i][jn][q];
+  }
+  // (a wave reads back only what it wrote itself: no barrier)
+  uint16_t *y = a.y[UPGATE ? 0 : zmat];
+  constexpr int CPR = UPGATE ? 4 : 8;   // lanes per row
+  constexpr int RPI = 64 / CPR;         // rows per iteration
+  const int er = lane / CPR, ec = (lane % CPR) * 8;
+  const int ncol0 = n0 + (UPGATE ? wn * 32 : wn * 64) + ec;
+  const bool plain = a.nmat != 1;       // one of three fused outputs: no scale, activation, residual
+  for (int it = 0; it < ROWS / RPI; ++it)
+    {
+      const int row = it * RPI + er;
+      const int m = m0 + wm * ROWS + row;
+      const float4 p0 = *(const float4 *)(park + row * LD + ec);
+      const float4 p1 = *(const float4 *)(park + row * LD + ec + 4);
+      float v[8] = { p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w };
+      if (UPGATE)
+        {
+          const float4 g0 = *(const float4 *)(park + row * LD + 32 + ec);
+          const float4 g1 = *(const float4 *)(park + row * LD + 32 + ec + 4);
+          const float g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = silu (g[e]) * v[e];
+        }
+      else if (!plain)
+        {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = v[e] * a.scale + a.bias;
+          if (a.act == 1)
+            {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                v[e] = silu (v[e]);
+            }
+        }
+      if (m >= a.M || ncol0 >= a.N)
+        continue;
+      uint16_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        h[e] = f2h (v[e]);
+      const size_t o = (size_t)m * a.ys + ncol0;
+      const bool res = !UPGATE && !plain && a.residual;
+      float *y32 = !UPGATE && !plain && a.y32 ? a.y32 + (size_t)m * a.N + ncol0 : nullptr;
+      if (vec && ncol0 + 8 <= a.N)
+        {
+          if (res)
+            {
+              const uint4 rv = ldg4 (a.residual + o);
+              const uint32_t rw[4] = { rv.x, rv.y, rv.z, rv.w };
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                h[e] = f2h (h2f (h[e]) + h2f ((uint16_t)(rw[e >> 1] >> ((e & 1) * 16))));
+            }
+          vkl_u32x4 pk;
+          pk.x = h[0] | ((uint32_t)h[1] << 16), pk.y = h[2] | ((uint32_t)h[3] << 16);
+          pk.z = h[4] | ((uint32_t)h[5] << 16), pk.w = h[6] | ((uint32_t)h[7] << 16);
+          *(VKL_GLOBAL vkl_u32x4 *)(y + o) = pk;
+          if (y32)
+            {
+              typedef float f32x4 __attribute__ ((ext_vector_type (4)));
+              f32x4 w0 = { h2f (h[0]), h2f (h[1]), h2f (h[2]), h2f (h[3]) };
+              f32x4 w1 = { h2f (h[4]), h2f (h[5]), h2f (h[6]), h2f (h[7]) };
+              *(VKL_GLOBAL f32x4 *)y32 = w0;
+              *(VKL_GLOBAL f32x4 *)(y32 + 4) = w1;
+            }
+          continue;
+        }
+      // ragged end of a row, or operands that are not 16-byte aligned
+      for (int e = 0; e < 8 && ncol0 + e < a.N; ++e)
+        {
+          uint16_t he = h[e];
+          if (res)
+            he = f2h (h2f (he) + h2f (ldg (a.residual + o + e)));
+          y[o + e] = he;
+          if (y32)
+            y32[e] = h2f (he);
+        }
+    }
+}
+
+constexpr size_t kWideLdsF16 = kWideStagesF16 > kWideParkBytes ? kWideStagesF16 : kWideParkBytes;
 
 template <bool UPGATE>
 __global__ __launch_bounds__ (WWAVES * 64) void
@@ -221,104 +334,244 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
     step (kt + 1, WideInt<1> ());
   __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
 
-  // Epilogue through LDS (the k loop's stages are free now): every wave parks
-  // its 128 x 64 fp32 block in a region of its own, then walks it row-wise so
-  // that a lane handles 8 neighbouring columns: 16-byte loads and stores, whole
-  // cache lines per row, and a short loop instead of 128 unrolled elements.
-  // Accumulator register q of lane l is row 8 (q/4) + 4 (l/32) + q%4, column
-  // l%32 of its 32 x 32 block.
-  __builtin_amdgcn_s_barrier (); // every wave has read its last fragments
-  constexpr int LD = 68;         // floats per parked row: 16-byte aligned, rows 4 banks apart
-  float *park = (float *)(wide_lds + wave * (128 * LD * 4));
-  {
-    float *pl = park + (lane >> 5) * 4 * LD + (lane & 31);
+  wide_epilogue<UPGATE, WTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+}
+
+// ---------------------------------------------------------------------------
+// planar Q8_0 weights
+// ---------------------------------------------------------------------------
+// Same tile, same staging.  The weight tile enters LDS as it lies in memory:
+// 128 rows x 64 int8 (8 KiB, 16-byte chunks swizzled by (row >> 1) & 3) plus
+// the two fp16 block scales of every row.  A wave converts the int8 fragments
+// it reads to fp16 (exact integers) in registers, sums each block of 32 on the
+// matrix core from a zero accumulator and applies the block's scale in fp32
+// (acc = fma (part, d, acc)): the arithmetic of the tile kernel and of the
+// reference shader.  That scaling costs as many vector-ALU cycles as the
+// products cost matrix-core cycles, and it wants the block sums in ordinary
+// registers: a workgroup is therefore EIGHT waves (4 x 2, 64 x 64 each, two per
+// SIMD, at most 256 registers, where the compiler keeps MFMA results out of
+// the accumulation registers).  The unit of the schedule is a block (two MFMA
+// k-slices): while block b is multiplied, the fragments of block b + 1 are
+// read and converted.
+constexpr int QWAVES = 8;
+constexpr int QTM = WBM / 4 / 32;
+constexpr int QAG = WBM / 8 / QWAVES; // x load instructions per wave and k-step
+// Three stages, laid out by kind (x tiles, then quants, then scales).
+constexpr int QSTAGES = 3;
+constexpr int QA_BYTES = WBM * WROWB;
+constexpr int QB_BYTES = WBN * WBK;
+constexpr int QS_BYTES = WBN * 4; // two fp16 scales per row
+constexpr int QB_BASE = QSTAGES * QA_BYTES;
+constexpr int QS_BASE = QB_BASE + QSTAGES * QB_BYTES;
+constexpr int QLOADS = QAG + 1 + 1; // per wave and k-step: x, quants, scales
+constexpr size_t kWideStagesQ8 = (size_t)QS_BASE + QSTAGES * QS_BYTES;
+constexpr size_t kWideLdsQ8 = kWideStagesQ8 > kWideParkBytes ? kWideStagesQ8 : kWideParkBytes;
+
+// (a vector type, not HIP's uint2 struct: LDS reads of the struct type are
+// taken to alias the tiles in flight and made to wait for all of them)
+typedef uint32_t u32x2 __attribute__ ((ext_vector_type (2)));
+
+__device__ __forceinline__ half8
+q8_frag (u32x2 r)
+{
+  h16x2 a, b, c, d;
+  i8x4_to_h2x2 (r.x, a, b);
+  i8x4_to_h2x2 (r.y, c, d);
+  half8 o;
+  o[0] = a[0], o[1] = a[1], o[2] = b[0], o[3] = b[1];
+  o[4] = c[0], o[5] = c[1], o[6] = d[0], o[7] = d[1];
+  return o;
+}
+
+template <bool UPGATE>
+__global__ __launch_bounds__ (QWAVES * 64) void
+gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
+{
+  extern __shared__ __align__ (16) uint8_t wide_lds[];
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int tile = xcd * per_xcd + j;
+  if (j >= per_xcd || tile >= tiles_m * tiles_n)
+    return;
+  const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
+  const int bn_rows = UPGATE ? WBN / 2 : WBN;
+  const int m0 = tm * WBM, n0 = tn * bn_rows;
+  const int zmat = blockIdx.z;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane (threadIdx.x >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // load addresses: x as in the fp16 kernel, instruction i of a wave covering
+  // tile rows 8 g .. 8 g + 7 with g = wave + 8 i
+  const int lr = lane >> 3;
+  const int chunk = (lane & 7) ^ lr ^ (wave & 1);
+  const uint8_t *src[QLOADS];
 #pragma unroll
-    for (int i = 0; i < WTM; ++i)
+  for (int i = 0; i < QAG; ++i)
+    {
+      const int m = min (m0 + (wave + QWAVES * i) * 8 + lr, a.M - 1);
+      src[i] = (const uint8_t *)(a.x + (size_t)m * a.xs + chunk * 8);
+    }
+  // quants: a wave's one instruction covers weight-tile rows 16 wave .. + 15;
+  // lane l fetches chunk (l%4) ^ ((row >> 1) & 3) of row 16 wave + l/4
+  {
+    const int qr = lane >> 2;
+    const int v = wave * 16 + qr;
+    const int mat = UPGATE ? v >> 6 : zmat;
+    const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
+    const uint8_t *w = mat == 0 ? a.wq[0] : (mat == 1 ? a.wq[1] : a.wq[2]);
+    src[QAG] = w + (size_t)n * a.Kp + ((lane & 3) ^ ((qr >> 1) & 3)) * 16;
+  }
+  // scales: the two of a row are one dword; a wave fetches rows 64 (wave & 1)
+  // + lane (four waves write each half, all the same values), so that every
+  // wave counts the same number of loads
+  {
+    const int v = (wave & 1) * 64 + lane;
+    const int mat = UPGATE ? v >> 6 : zmat;
+    const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
+    const uint16_t *ds = mat == 0 ? a.wd[0] : (mat == 1 ? a.wd[1] : a.wd[2]);
+    src[QAG + 1] = (const uint8_t *)(ds + (size_t)n * (a.Kp >> 5));
+  }
+
+  // fragment reads
+  const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
+  const int brow = (UPGATE ? wn * 32 : wn * 64) + (lane & 31);
+  const int qsw = (lane >> 1) & 3;
+  uint32_t aoff[4], qoff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+    {
+      aoff[ks] = (wm * (QTM * 32) + (lane & 31)) * WROWB + (((2 * ks + (lane >> 5)) ^ fsw) << 4);
+      qoff[ks] = QB_BASE + brow * WBK + ((ks ^ qsw) << 4) + (lane >> 5) * 8;
+    }
+  const uint32_t soff = QS_BASE + brow * 4;
+  constexpr int BJR = UPGATE ? 64 : 32; // rows from a wave's first to its second column block
+
+  float16v acc[QTM][WTN];
+#pragma unroll
+  for (int i = 0; i < QTM; ++i)
+#pragma unroll
+    for (int jn = 0; jn < WTN; ++jn)
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        acc[i][jn][q] = 0.f;
+
+  const int nk = a.K / WBK;
+  auto issue = [&] (int kt, int st) {
+#pragma unroll
+    for (int i = 0; i < QAG; ++i)
+      __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)(src[i] + (size_t)kt * WROWB),
+                                        (VKL_LDS void *)(wide_lds + st * QA_BYTES + (wave + QWAVES * i) * 1024), 16,
+                                        0, 0);
+    __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)(src[QAG] + (size_t)kt * WBK),
+                                      (VKL_LDS void *)(wide_lds + QB_BASE + st * QB_BYTES + wave * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)(src[QAG + 1] + (size_t)kt * 4),
+                                      (VKL_LDS void *)(wide_lds + QS_BASE + st * QS_BYTES + (wave & 1) * 256), 4,
+                                      0, 0);
+  };
+  issue (0, 0);
+  issue (nk > 1 ? 1 : 0, 1);
+
+  half8 af[2][2][QTM];  // [block buffer][k-slice of the block][row block]
+  u32x2 bq[2][2][WTN];  // weight fragments as read (int8)
+  float d[2][WTN];      // the scales of the tile's two blocks
+  auto read_block = [&] (int st, int blk, int buf) {
+    const int sa = st * QA_BYTES, sq = st * QB_BYTES;
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2)
+      {
+        const int ks = 2 * blk + k2;
+#pragma unroll
+        for (int jn = 0; jn < WTN; ++jn)
+          bq[buf][k2][jn] = *(const u32x2 *)(wide_lds + (qoff[ks] + sq) + jn * BJR * WBK);
+#pragma unroll
+        for (int i = 0; i < QTM; ++i)
+          af[buf][k2][i] = *(const half8 *)(wide_lds + (aoff[ks] + sa) + i * 32 * WROWB);
+      }
+  };
+  auto read_scales = [&] (int st) {
+#pragma unroll
+    for (int jn = 0; jn < WTN; ++jn)
+      {
+        const uint32_t sc = *(const uint32_t *)(wide_lds + (soff + st * QS_BYTES) + jn * BJR * 4);
+        d[0][jn] = h2f ((uint16_t)(sc & 0xffff));
+        d[1][jn] = h2f ((uint16_t)(sc >> 16));
+        // (keeps the conversion out of the scaling products: as fp16 operands
+        // they would become mixed-precision FMAs)
+        asm volatile ("" : "+v"(d[0][jn]), "+v"(d[1][jn]));
+      }
+  };
+  // The wave's four 32 x 32 blocks in turn, written so that the two MFMAs of one
+  // stand before the sixteen scaling FMAs of the one before; the order within
+  // a block is left to the compiler (pinned with scheduling barriers it ran
+  // 7 % slower).
+  auto multiply = [&] (int buf, const float (&dd)[WTN]) {
+    half8 bfc[2][WTN];
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int jn = 0; jn < WTN; ++jn)
+        bfc[k2][jn] = q8_frag (bq[buf][k2][jn]);
+    float16v part[2];
 #pragma unroll
-        for (int q = 0; q < 16; ++q)
-          pl[(i * 32 + (q >> 2) * 8 + (q & 3)) * LD + jn * 32] = acc[i][jn][q];
-  }
-  // (a wave reads back only what it wrote itself: no barrier)
-  uint16_t *y = a.y[UPGATE ? 0 : zmat];
-  constexpr int CPR = UPGATE ? 4 : 8;   // lanes per row
-  constexpr int RPI = 64 / CPR;         // rows per iteration
-  const int er = lane / CPR, ec = (lane % CPR) * 8;
-  const int ncol0 = n0 + (UPGATE ? wn * 32 : wn * 64) + ec;
-  const bool plain = a.nmat != 1;       // one of three fused outputs: no scale, activation, residual
-  for (int it = 0; it < 128 / RPI; ++it)
+    for (int p = 0; p <= QTM * WTN; ++p)
+      {
+        if (p < QTM * WTN)
+          {
+            const int i = p / WTN, jn = p % WTN;
+            float16v z;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              z[e] = 0.f;
+            z = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[buf][0][i], bfc[0][jn], z, 0, 0, 0);
+            part[p & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[buf][1][i], bfc[1][jn], z, 0, 0, 0);
+          }
+        if (p > 0)
+          {
+            const int i = (p - 1) / WTN, jn = (p - 1) % WTN;
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              acc[i][jn][e] = __builtin_fmaf (part[(p - 1) & 1][e], dd[jn], acc[i][jn][e]);
+          }
+      }
+  };
+  // s_waitcnt: the loads of the newest tile may stay in flight; the one in the
+  // loop also waits for the wave's own LDS reads
+  constexpr int WAITVM = 0x0f70 | (QLOADS & 15) | ((QLOADS >> 4) << 14);
+  __builtin_amdgcn_s_waitcnt (WAITVM);
+  __builtin_amdgcn_s_barrier ();
+  issue (nk > 2 ? 2 : nk - 1, 2);
+  read_block (0, 0, 0);
+  read_scales (0);
+  __builtin_amdgcn_sched_barrier (0);
+  // One k-step per turn.  On entry the fragments of block 0 of tile kt (stage
+  // st = kt % 3) are in buffer 0, the scales of both its blocks in d, and the
+  // loads of tiles kt + 1 and kt + 2 are in flight or done.  (One copy of the
+  // step with the stage as a variable: unrolled by the stages, the
+  // accumulators wander between sets of registers and the kernel spills.  Two
+  // stages, i.e. loads that have one k-step to arrive, ran 1.5 times slower.)
+  int st = 0;
+  for (int kt = 0; kt < nk; ++kt)
     {
-      const int row = it * RPI + er;
-      const int m = m0 + wm * (WBM / 2) + row;
-      const float4 p0 = *(const float4 *)(park + row * LD + ec);
-      const float4 p1 = *(const float4 *)(park + row * LD + ec + 4);
-      float v[8] = { p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w };
-      if (UPGATE)
-        {
-          const float4 g0 = *(const float4 *)(park + row * LD + 32 + ec);
-          const float4 g1 = *(const float4 *)(park + row * LD + 32 + ec + 4);
-          const float g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            v[e] = silu (g[e]) * v[e];
-        }
-      else if (!plain)
-        {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            v[e] = v[e] * a.scale + a.bias;
-          if (a.act == 1)
-            {
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                v[e] = silu (v[e]);
-            }
-        }
-      if (m >= a.M || ncol0 >= a.N)
-        continue;
-      uint16_t h[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        h[e] = f2h (v[e]);
-      const size_t o = (size_t)m * a.ys + ncol0;
-      const bool res = !UPGATE && !plain && a.residual;
-      float *y32 = !UPGATE && !plain && a.y32 ? a.y32 + (size_t)m * a.N + ncol0 : nullptr;
-      if (vec && ncol0 + 8 <= a.N)
-        {
-          if (res)
-            {
-              const uint4 rv = ldg4 (a.residual + o);
-              const uint32_t rw[4] = { rv.x, rv.y, rv.z, rv.w };
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                h[e] = f2h (h2f (h[e]) + h2f ((uint16_t)(rw[e >> 1] >> ((e & 1) * 16))));
-            }
-          vkl_u32x4 pk;
-          pk.x = h[0] | ((uint32_t)h[1] << 16), pk.y = h[2] | ((uint32_t)h[3] << 16);
-          pk.z = h[4] | ((uint32_t)h[5] << 16), pk.w = h[6] | ((uint32_t)h[7] << 16);
-          *(VKL_GLOBAL vkl_u32x4 *)(y + o) = pk;
-          if (y32)
-            {
-              typedef float f32x4 __attribute__ ((ext_vector_type (4)));
-              f32x4 w0 = { h2f (h[0]), h2f (h[1]), h2f (h[2]), h2f (h[3]) };
-              f32x4 w1 = { h2f (h[4]), h2f (h[5]), h2f (h[6]), h2f (h[7]) };
-              *(VKL_GLOBAL f32x4 *)y32 = w0;
-              *(VKL_GLOBAL f32x4 *)(y32 + 4) = w1;
-            }
-          continue;
-        }
-      // ragged end of a row, or operands that are not 16-byte aligned
-      for (int e = 0; e < 8 && ncol0 + e < a.N; ++e)
-        {
-          uint16_t he = h[e];
-          if (res)
-            he = f2h (h2f (he) + h2f (ldg (a.residual + o + e)));
-          y[o + e] = he;
-          if (y32)
-            y32[e] = h2f (he);
-        }
+      const int s1 = st == QSTAGES - 1 ? 0 : st + 1;
+      const float d1[WTN] = { d[1][0], d[1][1] };
+      read_block (st, 1, 1);
+      multiply (0, d[0]);
+      __builtin_amdgcn_sched_barrier (0);
+      // tile kt + 1 has landed (this wave's part; the barrier covers the
+      // others') and this wave has read the last of tile kt: its stage takes
+      // tile kt + 3 (past the end the last tile again, which nothing reads)
+      __builtin_amdgcn_s_waitcnt (WAITVM & ~0x0f00);
+      __builtin_amdgcn_s_barrier ();
+      __builtin_amdgcn_sched_barrier (0);
+      issue (kt + 3 < nk ? kt + 3 : nk - 1, st);
+      read_block (s1, 0, 0);
+      read_scales (s1);
+      multiply (1, d1);
+      __builtin_amdgcn_sched_barrier (0);
+      st = s1;
     }
+  __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
+  wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
 }
 
 // fewest tiles for which this form is used: below, too many of the 256 compute
@@ -329,8 +582,17 @@ constexpr int kWideMinTiles = 192;
 bool
 gemm_wide_supported (const GemmArgs &a)
 {
-  if (a.wtype != 1 || a.batch > 1 || (a.K % WBK) != 0 || a.M < WBM)
+  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < WBM)
     return false;
+  if (a.wtype == 8)
+    {
+      // whole k-steps of quants and scale pairs, aligned for 16- and 4-byte loads
+      if (a.Kp != a.K)
+        return false;
+      for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
+        if (((uintptr_t)a.wq[t] % 16) != 0 || ((uintptr_t)a.wd[t] % 4) != 0)
+          return false;
+    }
   const long tiles = (long)((a.M + WBM - 1) / WBM) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
                      * (a.upgate ? 1 : a.nmat);
   return tiles >= kWideMinTiles;
@@ -346,24 +608,36 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
   if (!lds_set[dev])
     {
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLds));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsF16));
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLds));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsF16));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
       lds_set[dev] = true;
     }
   const int tiles_m = (a.M + WBM - 1) / WBM;
   const int tiles_n = (a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128);
   const int per_xcd = (tiles_m * tiles_n + 7) / 8;
   const dim3 grid ((unsigned)(per_xcd * 8), 1, (unsigned)(a.upgate ? 1 : a.nmat));
+  const dim3 block ((a.wtype == 8 ? QWAVES : WWAVES) * 64);
   // 16-byte accesses to the outputs (and the residual) where their rows allow it
   int vec = (a.ys % 8) == 0 && (!a.residual || ((uintptr_t)a.residual % 16) == 0)
             && (!a.y32 || ((a.N % 4) == 0 && ((uintptr_t)a.y32 % 16) == 0));
   for (int t = 0; t < (a.upgate ? 1 : a.nmat); ++t)
     vec = vec && ((uintptr_t)a.y[t] % 16) == 0;
-  if (a.upgate)
-    gemm_wide_f16_kernel<true><<<grid, dim3 (WWAVES * 64), kWideLds, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+  if (a.wtype == 8)
+    {
+      if (a.upgate)
+        gemm_wide_q8_kernel<true><<<grid, block, kWideLdsQ8, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+      else
+        gemm_wide_q8_kernel<false><<<grid, block, kWideLdsQ8, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    }
+  else if (a.upgate)
+    gemm_wide_f16_kernel<true><<<grid, block, kWideLdsF16, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
   else
-    gemm_wide_f16_kernel<false><<<grid, dim3 (WWAVES * 64), kWideLds, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    gemm_wide_f16_kernel<false><<<grid, block, kWideLdsF16, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
   return (int)hipGetLastError ();
 }
 } // namespace vkl
