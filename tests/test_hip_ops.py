@@ -253,11 +253,12 @@ def test_matmul_f16_tb(dev, rng, C, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512),
                                    (512, 12800, 64), (600, 13000, 96), (600, 13000, 128), (777, 8200, 320),
-                                   (256, 24576, 192), (1030, 6144, 448)])
+                                   (256, 24576, 192), (1030, 6144, 448), (300, 6144, 128), (130, 12000, 192)])
 def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     """FP16 weights, many token rows: the matrix-core paths (from about two
-    hundred 256 x 128 output tiles on, with K a multiple of 64, the form that
-    loads its tiles straight into LDS; ragged M and N included)."""
+    hundred 256 x 128 output tiles on, or half as many 128 x 128 ones, with K a
+    multiple of 64, the form that loads its tiles straight into LDS; ragged M
+    and N included)."""
     a = rng.standard_normal((1, M, K)).astype(np.float16)
     b = (rng.standard_normal((1, N, K)) * 0.05).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
@@ -279,7 +280,7 @@ def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     assert np.array_equal(d32.read(np.float32, (M, N)), got.astype(np.float32))
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (130, 96, 4096), (600, 6500, 128), (257, 12300, 256)])
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (130, 96, 4096), (600, 6500, 128), (257, 12300, 256), (200, 6000, 128)])
 def test_ffn_upgate_f16_many_rows(dev, rng, M, N, K):
     x = rng.standard_normal((M, K)).astype(np.float16)
     up = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)

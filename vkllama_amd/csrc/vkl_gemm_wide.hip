@@ -36,12 +36,9 @@ typedef float float16v __attribute__ ((ext_vector_type (16)));
 constexpr int WBM = 256, WBN = 128, WBK = 64;
 constexpr int WSTAGES = 3;
 constexpr int WWAVES = 4;                       // 2 x 2
-constexpr int WTM = WBM / 2 / 32, WTN = WBN / 2 / 32;
+constexpr int WTN = WBN / 2 / 32;
 constexpr int WROWB = WBK * 2;                  // bytes of a tile row
-constexpr int WSTAGE_BYTES = (WBM + WBN) * WROWB;
-constexpr int WGPW = (WBM + WBN) / 8 / WWAVES;  // 1 KiB load instructions per wave and k-step
-constexpr int WAG = WBM / 8 / WWAVES;           // of which rows of x
-constexpr size_t kWideStagesF16 = (size_t)WSTAGES * WSTAGE_BYTES;
+
 
 // Issue order of one quarter of a k-step: after product Q one fragment read
 // (the first NR products) and an even share of the quarter's LQ loads.
@@ -73,7 +70,7 @@ template <int V> struct WideInt
 // Accumulator register q of lane l is row 8 (q/4) + 4 (l/32) + q%4, column
 // l%32 of its 32 x 32 block.
 constexpr int kWideParkLd = 68; // floats per parked row: 16-byte aligned, rows 4 banks apart
-constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 128 fp32 in rows of 64
+constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 128 fp32 in rows of 64 (Q8_0 kernel)
 
 template <bool UPGATE, int TM>
 __device__ __forceinline__ void
@@ -177,12 +174,24 @@ wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_
     }
 }
 
-constexpr size_t kWideLdsF16 = kWideStagesF16 > kWideParkBytes ? kWideStagesF16 : kWideParkBytes;
+template <int BM>
+constexpr size_t
+wide_lds_f16 ()
+{
+  const size_t stages = (size_t)WSTAGES * (BM + WBN) * WROWB, park = (size_t)BM * 2 * kWideParkLd * 4;
+  return stages > park ? stages : park;
+}
 
-template <bool UPGATE>
+// BM: token rows of a tile, 256 or (where 256-row tiles would be too few to
+// occupy the compute units) 128, i.e. 64 x 64 per wave.
+template <int BM, bool UPGATE>
 __global__ __launch_bounds__ (WWAVES * 64) void
 gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
 {
+  constexpr int TM = BM / 2 / 32;                    // 32-row accumulators per wave
+  constexpr int STAGE_BYTES = (BM + WBN) * WROWB;
+  constexpr int GPW = (BM + WBN) / 8 / WWAVES;       // 1 KiB load instructions per wave and k-step
+  constexpr int AG = BM / 8 / WWAVES;                // of which rows of x
   extern __shared__ __align__ (16) uint8_t wide_lds[];
   // workgroups go to the XCDs in turn: each XCD gets a contiguous range of
   // tiles, token-row tile fastest, so the weight tiles it shares stay in its L2
@@ -192,30 +201,30 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
     return;
   const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
   const int bn_rows = UPGATE ? WBN / 2 : WBN; // weight rows per matrix and tile
-  const int m0 = tm * WBM, n0 = tn * bn_rows;
+  const int m0 = tm * BM, n0 = tn * bn_rows;
   const int zmat = blockIdx.z;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane (threadIdx.x >> 6);
   const int wm = wave >> 1, wn = wave & 1;
 
   // Load addresses.  Instruction i of a wave covers tile rows 8g .. 8g+7 with
-  // g = wave + 4 i (x for i < WAG, then W); lane l fetches row 8g + l/8, and
+  // g = wave + 4 i (x for i < AG, then W); lane l fetches row 8g + l/8, and
   // LDS slot l%8 of that row receives chunk (l%8) ^ f(row), f(row) = (row & 7)
   // ^ ((row >> 3) & 1): 8 or 16 consecutive rows then hit different banks at
   // the same chunk.  Rows beyond M or N repeat the last row (never stored).
   const int lr = lane >> 3;
   const int chunk = (lane & 7) ^ lr ^ (wave & 1);
-  const uint16_t *src[WGPW];
+  const uint16_t *src[GPW];
 #pragma unroll
-  for (int i = 0; i < WAG; ++i)
+  for (int i = 0; i < AG; ++i)
     {
       const int m = min (m0 + (wave + WWAVES * i) * 8 + lr, a.M - 1);
       src[i] = a.x + (size_t)m * a.xs + chunk * 8;
     }
 #pragma unroll
-  for (int i = WAG; i < WGPW; ++i)
+  for (int i = AG; i < GPW; ++i)
     {
-      const int v = (wave + WWAVES * (i - WAG)) * 8 + lr; // row of the weight tile
+      const int v = (wave + WWAVES * (i - AG)) * 8 + lr; // row of the weight tile
       const int mat = UPGATE ? v >> 6 : zmat;
       const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
       const uint16_t *w = mat == 0 ? a.wh[0] : (mat == 1 ? a.wh[1] : a.wh[2]);
@@ -229,14 +238,14 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
   for (int ks = 0; ks < 4; ++ks)
     {
       const int ko = ((2 * ks + (lane >> 5)) ^ fsw) << 4;
-      aoff[ks] = (wm * (WBM / 2) + (lane & 31)) * WROWB + ko;
-      boff[ks] = WBM * WROWB + ((UPGATE ? wn * 32 : wn * 64) + (lane & 31)) * WROWB + ko;
+      aoff[ks] = (wm * (BM / 2) + (lane & 31)) * WROWB + ko;
+      boff[ks] = BM * WROWB + ((UPGATE ? wn * 32 : wn * 64) + (lane & 31)) * WROWB + ko;
     }
   constexpr int BJ = (UPGATE ? 64 : 32) * WROWB; // from a wave's first to its second column block
 
-  float16v acc[WTM][WTN];
+  float16v acc[TM][WTN];
 #pragma unroll
-  for (int i = 0; i < WTM; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int jn = 0; jn < WTN; ++jn)
 #pragma unroll
@@ -248,33 +257,33 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
 #pragma unroll
     for (int i = i0; i < i1; ++i)
       {
-        const int g = i < WAG ? wave + WWAVES * i : WBM / 8 + wave + WWAVES * (i - WAG);
+        const int g = i < AG ? wave + WWAVES * i : BM / 8 + wave + WWAVES * (i - AG);
         __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)(src[i] + (size_t)kt * WBK),
-                                          (VKL_LDS void *)(wide_lds + st * WSTAGE_BYTES + g * 1024), 16, 0, 0);
+                                          (VKL_LDS void *)(wide_lds + st * STAGE_BYTES + g * 1024), 16, 0, 0);
       }
   };
 #pragma unroll
   for (int p = 0; p < WSTAGES - 1; ++p)
-    issue_part (p < nk ? p : nk - 1, p, 0, WGPW);
+    issue_part (p < nk ? p : nk - 1, p, 0, GPW);
 
-  half8 af[2][WTM], bf[2][WTN];
+  half8 af[2][TM], bf[2][WTN];
   // in the order the products need them
   auto read_frags = [&] (int st, int ks, int buf) {
-    const uint8_t *sb = wide_lds + st * WSTAGE_BYTES;
+    const uint8_t *sb = wide_lds + st * STAGE_BYTES;
     af[buf][0] = *(const half8 *)(sb + aoff[ks]);
 #pragma unroll
     for (int jn = 0; jn < WTN; ++jn)
       bf[buf][jn] = *(const half8 *)(sb + boff[ks] + jn * BJ);
 #pragma unroll
-    for (int i = 1; i < WTM; ++i)
+    for (int i = 1; i < TM; ++i)
       af[buf][i] = *(const half8 *)(sb + aoff[ks] + i * 32 * WROWB);
   };
   // s_waitcnt immediates: vmcnt = the loads of the newest k-step may stay in
   // flight; the second one also waits for the wave's own LDS reads
-  constexpr int VMW = (WSTAGES - 2) * WGPW;
+  constexpr int VMW = (WSTAGES - 2) * GPW;
   constexpr int WAITVM = 0x0f70 | (VMW & 15) | ((VMW >> 4) << 14);
-  constexpr int LB1 = WGPW / 3, LB2 = 2 * WGPW / 3;
-  constexpr int NR = WTM + WTN, NP = WTM * WTN;
+  constexpr int LB1 = GPW / 3, LB2 = 2 * GPW / 3;
+  constexpr int NR = TM + WTN, NP = TM * WTN;
   // One k-step.  On entry tile kt is in stage ST and the fragments of its
   // first quarter are on their way into buffer 0.
   auto step = [&] (int kt, auto stc) {
@@ -290,7 +299,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
         if (ks < 3)
           {
             read_frags (ST, ks + 1, (ks + 1) & 1);
-            issue_part (kn, SN, ks == 0 ? 0 : ks == 1 ? LB1 : LB2, ks == 0 ? LB1 : ks == 1 ? LB2 : WGPW);
+            issue_part (kn, SN, ks == 0 ? 0 : ks == 1 ? LB1 : LB2, ks == 0 ? LB1 : ks == 1 ? LB2 : GPW);
           }
         else
           {
@@ -302,7 +311,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
             read_frags (S1, 0, 0);
           }
 #pragma unroll
-        for (int i = 0; i < WTM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int jn = 0; jn < WTN; ++jn)
             acc[i][jn] = __builtin_amdgcn_mfma_f32_32x32x16_f16 (af[ks & 1][i], bf[ks & 1][jn], acc[i][jn], 0, 0, 0);
@@ -311,7 +320,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
         else if (ks == 1)
           WideOrder<0, NP, NR, LB2 - LB1>::run ();
         else if (ks == 2)
-          WideOrder<0, NP, NR, WGPW - LB2>::run ();
+          WideOrder<0, NP, NR, GPW - LB2>::run ();
         else
           WideOrder<0, NP, NR, 0>::run ();
         __builtin_amdgcn_sched_barrier (0);
@@ -334,7 +343,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
     step (kt + 1, WideInt<1> ());
   __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
 
-  wide_epilogue<UPGATE, WTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+  wide_epilogue<UPGATE, TM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
 }
 
 // ---------------------------------------------------------------------------
@@ -574,28 +583,52 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
 }
 
-// fewest tiles for which this form is used: below, too many of the 256 compute
-// units would idle and the tile kernel with its k-split does better
-constexpr int kWideMinTiles = 192;
+// Fewest tiles for which this form is used: below, too many of the 256 compute
+// units would idle and the tile kernel with its k-split does better (measured
+// on the 7B shapes, 256 to 2048 rows).
+constexpr int kWideMinTilesQ8 = 160;
+constexpr int kWideMinHalfTiles = 88;
+// time of a round of 128-row tiles relative to one of 256-row tiles (31-38 us
+// against 46-51 us at K = 4096)
+constexpr double kWideHalfRound = 0.68;
+
+long
+wide_tiles (const GemmArgs &a, int bm)
+{
+  return (long)((a.M + bm - 1) / bm) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
+         * (a.upgate ? 1 : a.nmat);
+}
+
+// token rows of the tile to use, 0: this form does not apply
+int
+wide_tile_rows (const GemmArgs &a)
+{
+  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0)
+    return 0;
+  if (a.wtype == 8)
+    {
+      // whole k-steps of quants and scale pairs, aligned for 16- and 4-byte loads
+      if (a.Kp != a.K || a.M < WBM)
+        return 0;
+      for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
+        if (((uintptr_t)a.wq[t] % 16) != 0 || ((uintptr_t)a.wd[t] % 4) != 0)
+          return 0;
+      return wide_tiles (a, WBM) >= kWideMinTilesQ8 ? WBM : 0;
+    }
+  // fp16 weights: the tile height whose rounds over the 256 compute units
+  // take less time
+  const long t128 = wide_tiles (a, 128), t256 = wide_tiles (a, WBM);
+  if (a.M < 128 || t128 < kWideMinHalfTiles)
+    return 0;
+  const double c256 = (double)((t256 + 255) / 256), c128 = (double)((t128 + 255) / 256) * kWideHalfRound;
+  return a.M >= WBM && c256 <= c128 ? WBM : 128;
+}
 } // namespace
 
 bool
 gemm_wide_supported (const GemmArgs &a)
 {
-  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < WBM)
-    return false;
-  if (a.wtype == 8)
-    {
-      // whole k-steps of quants and scale pairs, aligned for 16- and 4-byte loads
-      if (a.Kp != a.K)
-        return false;
-      for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
-        if (((uintptr_t)a.wq[t] % 16) != 0 || ((uintptr_t)a.wd[t] % 4) != 0)
-          return false;
-    }
-  const long tiles = (long)((a.M + WBM - 1) / WBM) * ((a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128))
-                     * (a.upgate ? 1 : a.nmat);
-  return tiles >= kWideMinTiles;
+  return wide_tile_rows (a) != 0;
 }
 
 int
@@ -605,19 +638,27 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
   int dev = 0;
   if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
     return (int)hipErrorInvalidDevice;
+  constexpr size_t lds256 = wide_lds_f16<256> (), lds128 = wide_lds_f16<128> ();
   if (!lds_set[dev])
     {
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsF16));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsF16));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<256, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds256));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<256, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds256));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<false>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
       lds_set[dev] = true;
     }
-  const int tiles_m = (a.M + WBM - 1) / WBM;
+  const int bm = wide_tile_rows (a);
+  if (!bm)
+    return (int)hipErrorInvalidValue;
+  const int tiles_m = (a.M + bm - 1) / bm;
   const int tiles_n = (a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128);
   const int per_xcd = (tiles_m * tiles_n + 7) / 8;
   const dim3 grid ((unsigned)(per_xcd * 8), 1, (unsigned)(a.upgate ? 1 : a.nmat));
@@ -634,10 +675,17 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
       else
         gemm_wide_q8_kernel<false><<<grid, block, kWideLdsQ8, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
     }
+  else if (bm == 256)
+    {
+      if (a.upgate)
+        gemm_wide_f16_kernel<256, true><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+      else
+        gemm_wide_f16_kernel<256, false><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    }
   else if (a.upgate)
-    gemm_wide_f16_kernel<true><<<grid, block, kWideLdsF16, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    gemm_wide_f16_kernel<128, true><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
   else
-    gemm_wide_f16_kernel<false><<<grid, block, kWideLdsF16, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    gemm_wide_f16_kernel<128, false><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
   return (int)hipGetLastError ();
 }
 } // namespace vkl
