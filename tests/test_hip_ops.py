@@ -140,15 +140,17 @@ def test_matmul_q8_0_epilogue(dev, rng):
 @pytest.mark.parametrize("M,N,K", [(9, 128, 32), (16, 130, 512), (64, 256, 4096), (100, 200, 1376), (300, 1376, 512),
                                    (129, 64, 11008), (65, 32000, 512),
                                    (7, 200, 1376), (32, 129, 768), (5, 64, 256), (31, 300, 11008), (2, 1000, 5120),
-                                   (270, 12300, 64), (600, 13000, 192), (1030, 6144, 448), (777, 8200, 320)])
+                                   (270, 12300, 64), (600, 13000, 192), (1030, 6144, 448), (777, 8200, 320),
+                                   (300, 8192, 64)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
     few-row kernels (K a multiple of 256 or not, a last slice that is half
     empty, row counts that do not fill the last workgroup), half- and
-    full-height tiles, the k-split, and (the last four: about two hundred
-    256 x 128 tiles and more, K a multiple of 64) the form that loads its tiles
-    straight into LDS, with ragged M and N, one to seven k-steps."""
+    full-height tiles, the k-split, and (the last five: about two hundred
+    256 x 128 tiles and more, or half as many 128 x 128 ones, K a multiple of
+    64) the form that loads its tiles straight into LDS, with ragged M and N,
+    one to seven k-steps."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
@@ -188,7 +190,7 @@ def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     assert not yw[:, N:].any()
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376), (258, 4200, 64)])
+@pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376), (258, 4200, 64), (130, 5200, 64)])
 def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
     ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
     x = rng.standard_normal((M, K)).astype(np.float16)
@@ -202,7 +204,7 @@ def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
         assert rel_err(f16(o, (M, N)), w) < F16_REL_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128)])
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128), (200, 7800, 64)])
 def test_ffn_upgate_q8_0_many_rows(dev, rng, M, N, K):
     up, _ = q8_weights(rng, N, K)
     gate, _ = q8_weights(rng, N, K)

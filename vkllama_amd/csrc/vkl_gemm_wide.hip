@@ -363,18 +363,18 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
 // k-slices): while block b is multiplied, the fragments of block b + 1 are
 // read and converted.
 constexpr int QWAVES = 8;
-constexpr int QTM = WBM / 4 / 32;
-constexpr int QAG = WBM / 8 / QWAVES; // x load instructions per wave and k-step
 // Three stages, laid out by kind (x tiles, then quants, then scales).
 constexpr int QSTAGES = 3;
-constexpr int QA_BYTES = WBM * WROWB;
 constexpr int QB_BYTES = WBN * WBK;
 constexpr int QS_BYTES = WBN * 4; // two fp16 scales per row
-constexpr int QB_BASE = QSTAGES * QA_BYTES;
-constexpr int QS_BASE = QB_BASE + QSTAGES * QB_BYTES;
-constexpr int QLOADS = QAG + 1 + 1; // per wave and k-step: x, quants, scales
-constexpr size_t kWideStagesQ8 = (size_t)QS_BASE + QSTAGES * QS_BYTES;
-constexpr size_t kWideLdsQ8 = kWideStagesQ8 > kWideParkBytes ? kWideStagesQ8 : kWideParkBytes;
+
+template <int BM>
+constexpr size_t
+wide_lds_q8 ()
+{
+  const size_t stages = (size_t)QSTAGES * (BM * WROWB + QB_BYTES + QS_BYTES), park = (size_t)BM * 2 * kWideParkLd * 4;
+  return stages > park ? stages : park;
+}
 
 // (a vector type, not HIP's uint2 struct: LDS reads of the struct type are
 // taken to alias the tiles in flight and made to wait for all of them)
@@ -392,10 +392,16 @@ q8_frag (u32x2 r)
   return o;
 }
 
-template <bool UPGATE>
+template <int BM, bool UPGATE>
 __global__ __launch_bounds__ (QWAVES * 64) void
 gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
 {
+  constexpr int QTM = BM / 4 / 32;           // 32-row accumulators per wave
+  constexpr int QAG = BM / 8 / QWAVES;       // x load instructions per wave and k-step
+  constexpr int QA_BYTES = BM * WROWB;
+  constexpr int QB_BASE = QSTAGES * QA_BYTES;
+  constexpr int QS_BASE = QB_BASE + QSTAGES * QB_BYTES;
+  constexpr int QLOADS = QAG + 1 + 1;        // per wave and k-step: x, quants, scales
   extern __shared__ __align__ (16) uint8_t wide_lds[];
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int tile = xcd * per_xcd + j;
@@ -403,7 +409,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
     return;
   const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
   const int bn_rows = UPGATE ? WBN / 2 : WBN;
-  const int m0 = tm * WBM, n0 = tn * bn_rows;
+  const int m0 = tm * BM, n0 = tn * bn_rows;
   const int zmat = blockIdx.z;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane (threadIdx.x >> 6);
@@ -586,8 +592,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
 // Fewest tiles for which this form is used: below, too many of the 256 compute
 // units would idle and the tile kernel with its k-split does better (measured
 // on the 7B shapes, 256 to 2048 rows).
-constexpr int kWideMinTilesQ8 = 160;
-constexpr int kWideMinHalfTiles = 88;
+constexpr int kWideMinHalfTiles = 88, kWideMinHalfTilesQ8 = 160;
 // time of a round of 128-row tiles relative to one of 256-row tiles (31-38 us
 // against 46-51 us at K = 4096)
 constexpr double kWideHalfRound = 0.68;
@@ -608,17 +613,15 @@ wide_tile_rows (const GemmArgs &a)
   if (a.wtype == 8)
     {
       // whole k-steps of quants and scale pairs, aligned for 16- and 4-byte loads
-      if (a.Kp != a.K || a.M < WBM)
+      if (a.Kp != a.K)
         return 0;
       for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
         if (((uintptr_t)a.wq[t] % 16) != 0 || ((uintptr_t)a.wd[t] % 4) != 0)
           return 0;
-      return wide_tiles (a, WBM) >= kWideMinTilesQ8 ? WBM : 0;
     }
-  // fp16 weights: the tile height whose rounds over the 256 compute units
-  // take less time
+  // the tile height whose rounds over the 256 compute units take less time
   const long t128 = wide_tiles (a, 128), t256 = wide_tiles (a, WBM);
-  if (a.M < 128 || t128 < kWideMinHalfTiles)
+  if (a.M < 128 || t128 < (a.wtype == 8 ? kWideMinHalfTilesQ8 : kWideMinHalfTiles))
     return 0;
   const double c256 = (double)((t256 + 255) / 256), c128 = (double)((t128 + 255) / 256) * kWideHalfRound;
   return a.M >= WBM && c256 <= c128 ? WBM : 128;
@@ -639,6 +642,7 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
   if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
     return (int)hipErrorInvalidDevice;
   constexpr size_t lds256 = wide_lds_f16<256> (), lds128 = wide_lds_f16<128> ();
+  constexpr size_t q256 = wide_lds_q8<256> (), q128 = wide_lds_q8<128> ();
   if (!lds_set[dev])
     {
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<256, false>,
@@ -649,10 +653,14 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsQ8));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, false>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, true>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
       lds_set[dev] = true;
     }
   const int bm = wide_tile_rows (a);
@@ -668,12 +676,19 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
             && (!a.y32 || ((a.N % 4) == 0 && ((uintptr_t)a.y32 % 16) == 0));
   for (int t = 0; t < (a.upgate ? 1 : a.nmat); ++t)
     vec = vec && ((uintptr_t)a.y[t] % 16) == 0;
-  if (a.wtype == 8)
+  if (a.wtype == 8 && bm == 256)
     {
       if (a.upgate)
-        gemm_wide_q8_kernel<true><<<grid, block, kWideLdsQ8, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, true><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
       else
-        gemm_wide_q8_kernel<false><<<grid, block, kWideLdsQ8, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, false><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    }
+  else if (a.wtype == 8)
+    {
+      if (a.upgate)
+        gemm_wide_q8_kernel<128, true><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+      else
+        gemm_wide_q8_kernel<128, false><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
     }
   else if (bm == 256)
     {
