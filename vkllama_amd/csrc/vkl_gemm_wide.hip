@@ -72,6 +72,78 @@ template <int V> struct WideInt
 constexpr int kWideParkLd = 68; // floats per parked row: 16-byte aligned, rows 4 banks apart
 constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 128 fp32 in rows of 64 (Q8_0 kernel)
 
+// Eight neighbouring outputs of row m from column ncol0 on: v the fp32 sums (for
+// the fused pair: up; g: gate), then scale, bias, activation, rounding,
+// residual, the stores.
+template <bool UPGATE>
+__device__ __forceinline__ void
+wide_finish8 (const GemmArgs &a, float (&v)[8], const float (&g)[8], int m, int ncol0, int zmat, int vec)
+{
+  uint16_t *y = a.y[UPGATE ? 0 : zmat];
+  const bool plain = a.nmat != 1; // one of three fused outputs: no scale, activation, residual
+  if (UPGATE)
+    {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v[e] = silu (g[e]) * v[e];
+    }
+  else if (!plain)
+    {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v[e] = v[e] * a.scale + a.bias;
+      if (a.act == 1)
+        {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = silu (v[e]);
+        }
+    }
+  if (m >= a.M || ncol0 >= a.N)
+    return;
+  uint16_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    h[e] = f2h (v[e]);
+  const size_t o = (size_t)m * a.ys + ncol0;
+  const bool res = !UPGATE && !plain && a.residual;
+  float *y32 = !UPGATE && !plain && a.y32 ? a.y32 + (size_t)m * a.N + ncol0 : nullptr;
+  if (vec && ncol0 + 8 <= a.N)
+    {
+      if (res)
+        {
+          const uint4 rv = ldg4 (a.residual + o);
+          const uint32_t rw[4] = { rv.x, rv.y, rv.z, rv.w };
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            h[e] = f2h (h2f (h[e]) + h2f ((uint16_t)(rw[e >> 1] >> ((e & 1) * 16))));
+        }
+      vkl_u32x4 pk;
+      pk.x = h[0] | ((uint32_t)h[1] << 16), pk.y = h[2] | ((uint32_t)h[3] << 16);
+      pk.z = h[4] | ((uint32_t)h[5] << 16), pk.w = h[6] | ((uint32_t)h[7] << 16);
+      *(VKL_GLOBAL vkl_u32x4 *)(y + o) = pk;
+      if (y32)
+        {
+          typedef float f32x4 __attribute__ ((ext_vector_type (4)));
+          f32x4 w0 = { h2f (h[0]), h2f (h[1]), h2f (h[2]), h2f (h[3]) };
+          f32x4 w1 = { h2f (h[4]), h2f (h[5]), h2f (h[6]), h2f (h[7]) };
+          *(VKL_GLOBAL f32x4 *)y32 = w0;
+          *(VKL_GLOBAL f32x4 *)(y32 + 4) = w1;
+        }
+      return;
+    }
+  // ragged end of a row, or operands that are not 16-byte aligned
+  for (int e = 0; e < 8 && ncol0 + e < a.N; ++e)
+    {
+      uint16_t he = h[e];
+      if (res)
+        he = f2h (h2f (he) + h2f (ldg (a.residual + o + e)));
+      y[o + e] = he;
+      if (y32)
+        y32[e] = h2f (he);
+    }
+}
+
 template <bool UPGATE, int TM>
 __device__ __forceinline__ void
 wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_lds, int wave, int lane,
@@ -94,83 +166,67 @@ wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_
           pl[(i * 32 + (q >> 2) * 8 + (q & 3)) * LD + jn * 32] = acc[i][jn][q];
   }
   // (a wave reads back only what it wrote itself: no barrier)
-  uint16_t *y = a.y[UPGATE ? 0 : zmat];
   constexpr int CPR = UPGATE ? 4 : 8;   // lanes per row
   constexpr int RPI = 64 / CPR;         // rows per iteration
   const int er = lane / CPR, ec = (lane % CPR) * 8;
   const int ncol0 = n0 + (UPGATE ? wn * 32 : wn * 64) + ec;
-  const bool plain = a.nmat != 1;       // one of three fused outputs: no scale, activation, residual
   for (int it = 0; it < ROWS / RPI; ++it)
     {
       const int row = it * RPI + er;
-      const int m = m0 + wm * ROWS + row;
       const float4 p0 = *(const float4 *)(park + row * LD + ec);
       const float4 p1 = *(const float4 *)(park + row * LD + ec + 4);
       float v[8] = { p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w };
+      float g[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
       if (UPGATE)
         {
           const float4 g0 = *(const float4 *)(park + row * LD + 32 + ec);
           const float4 g1 = *(const float4 *)(park + row * LD + 32 + ec + 4);
-          const float g[8] = { g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w };
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            v[e] = silu (g[e]) * v[e];
+          g[0] = g0.x, g[1] = g0.y, g[2] = g0.z, g[3] = g0.w, g[4] = g1.x, g[5] = g1.y, g[6] = g1.z, g[7] = g1.w;
         }
-      else if (!plain)
+      wide_finish8<UPGATE> (a, v, g, m0 + wm * ROWS + row, ncol0, zmat, vec);
+    }
+}
+
+// The same for waves in a 2 x 4 grid (TM x 32 rows by 32 columns each; of the
+// fused pair the waves 0, 1 of a row block hold up, 2, 3 gate): the whole
+// BM x 128 tile is parked, and after a barrier all threads walk it row-wise.
+constexpr int kWideTileLd = 132;
+
+template <int BM, bool UPGATE, int TM>
+__device__ __forceinline__ void
+wide_epilogue_tile (const GemmArgs &a, const float16v (&acc)[TM][1], uint8_t *wide_lds, int wave, int lane,
+                    int m0, int n0, int zmat, int vec)
+{
+  constexpr int LD = kWideTileLd;
+  const int wm = wave >> 2, wn = wave & 3;
+  __builtin_amdgcn_s_barrier (); // every wave has read its last fragments
+  float *park = (float *)wide_lds;
+  {
+    float *pl = park + (wm * TM * 32 + (lane >> 5) * 4) * LD + wn * 32 + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        pl[(i * 32 + (q >> 2) * 8 + (q & 3)) * LD] = acc[i][0][q];
+  }
+  __syncthreads ();
+  constexpr int LPR = UPGATE ? 8 : 16;        // lanes per row
+  constexpr int RPI = 8 * 64 / LPR;           // rows per iteration of the workgroup
+  const int er = threadIdx.x / LPR, ec = (threadIdx.x % LPR) * 8;
+  for (int it = 0; it < BM / RPI; ++it)
+    {
+      const int row = it * RPI + er;
+      const float4 p0 = *(const float4 *)(park + row * LD + ec);
+      const float4 p1 = *(const float4 *)(park + row * LD + ec + 4);
+      float v[8] = { p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w };
+      float g[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
+      if (UPGATE)
         {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            v[e] = v[e] * a.scale + a.bias;
-          if (a.act == 1)
-            {
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                v[e] = silu (v[e]);
-            }
+          const float4 g0 = *(const float4 *)(park + row * LD + 64 + ec);
+          const float4 g1 = *(const float4 *)(park + row * LD + 64 + ec + 4);
+          g[0] = g0.x, g[1] = g0.y, g[2] = g0.z, g[3] = g0.w, g[4] = g1.x, g[5] = g1.y, g[6] = g1.z, g[7] = g1.w;
         }
-      if (m >= a.M || ncol0 >= a.N)
-        continue;
-      uint16_t h[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        h[e] = f2h (v[e]);
-      const size_t o = (size_t)m * a.ys + ncol0;
-      const bool res = !UPGATE && !plain && a.residual;
-      float *y32 = !UPGATE && !plain && a.y32 ? a.y32 + (size_t)m * a.N + ncol0 : nullptr;
-      if (vec && ncol0 + 8 <= a.N)
-        {
-          if (res)
-            {
-              const uint4 rv = ldg4 (a.residual + o);
-              const uint32_t rw[4] = { rv.x, rv.y, rv.z, rv.w };
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                h[e] = f2h (h2f (h[e]) + h2f ((uint16_t)(rw[e >> 1] >> ((e & 1) * 16))));
-            }
-          vkl_u32x4 pk;
-          pk.x = h[0] | ((uint32_t)h[1] << 16), pk.y = h[2] | ((uint32_t)h[3] << 16);
-          pk.z = h[4] | ((uint32_t)h[5] << 16), pk.w = h[6] | ((uint32_t)h[7] << 16);
-          *(VKL_GLOBAL vkl_u32x4 *)(y + o) = pk;
-          if (y32)
-            {
-              typedef float f32x4 __attribute__ ((ext_vector_type (4)));
-              f32x4 w0 = { h2f (h[0]), h2f (h[1]), h2f (h[2]), h2f (h[3]) };
-              f32x4 w1 = { h2f (h[4]), h2f (h[5]), h2f (h[6]), h2f (h[7]) };
-              *(VKL_GLOBAL f32x4 *)y32 = w0;
-              *(VKL_GLOBAL f32x4 *)(y32 + 4) = w1;
-            }
-          continue;
-        }
-      // ragged end of a row, or operands that are not 16-byte aligned
-      for (int e = 0; e < 8 && ncol0 + e < a.N; ++e)
-        {
-          uint16_t he = h[e];
-          if (res)
-            he = f2h (h2f (he) + h2f (ldg (a.residual + o + e)));
-          y[o + e] = he;
-          if (y32)
-            y32[e] = h2f (he);
-        }
+      wide_finish8<UPGATE> (a, v, g, m0 + row, n0 + ec, zmat, vec);
     }
 }
 
@@ -357,12 +413,17 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
 // (acc = fma (part, d, acc)): the arithmetic of the tile kernel and of the
 // reference shader.  That scaling costs as many vector-ALU cycles as the
 // products cost matrix-core cycles, and it wants the block sums in ordinary
-// registers: a workgroup is therefore EIGHT waves (4 x 2, 64 x 64 each, two per
-// SIMD, at most 256 registers, where the compiler keeps MFMA results out of
-// the accumulation registers).  The unit of the schedule is a block (two MFMA
+// registers: a workgroup is therefore EIGHT waves (two per SIMD, at most 256
+// registers each, where the compiler keeps MFMA results out of the
+// accumulation registers).  The unit of the schedule is a block (two MFMA
 // k-slices): while block b is multiplied, the fragments of block b + 1 are
-// read and converted.
+// read.  (LDS reads must not go through HIP's uint2/uint4 struct types here:
+// the compiler takes reads of a struct type to alias the tiles that the
+// direct-to-LDS loads still have in flight and waits for all of them.)
 constexpr int QWAVES = 8;
+// waves along N: 4 (2 x 4 waves, 128 x 32 each) measured 5-12 % faster than 2
+// (4 x 2 waves, 64 x 64 each) on the 7B and 13B shapes
+constexpr int QGRID = 4;
 // Three stages, laid out by kind (x tiles, then quants, then scales).
 constexpr int QSTAGES = 3;
 constexpr int QB_BYTES = WBN * WBK;
@@ -372,7 +433,7 @@ template <int BM>
 constexpr size_t
 wide_lds_q8 ()
 {
-  const size_t stages = (size_t)QSTAGES * (BM * WROWB + QB_BYTES + QS_BYTES), park = (size_t)BM * 2 * kWideParkLd * 4;
+  const size_t stages = (size_t)QSTAGES * (BM * WROWB + QB_BYTES + QS_BYTES), park = (size_t)BM * 2 * kWideParkLd * 4; // (>= BM * kWideTileLd * 4)
   return stages > park ? stages : park;
 }
 
@@ -392,11 +453,15 @@ q8_frag (u32x2 r)
   return o;
 }
 
-template <int BM, bool UPGATE>
+// WGN: waves along N, 2 (4 x 2 waves of 64 columns) or 4 (2 x 4 waves of 32
+// columns and twice the rows: every weight fragment is converted by two waves
+// instead of four).
+template <int BM, int WGN, bool UPGATE>
 __global__ __launch_bounds__ (QWAVES * 64) void
 gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
 {
-  constexpr int QTM = BM / 4 / 32;           // 32-row accumulators per wave
+  constexpr int QTM = BM / (QWAVES / WGN) / 32; // 32-row accumulators per wave
+  constexpr int QTN = 4 / WGN;                  // 32-column accumulators per wave
   constexpr int QAG = BM / 8 / QWAVES;       // x load instructions per wave and k-step
   constexpr int QA_BYTES = BM * WROWB;
   constexpr int QB_BASE = QSTAGES * QA_BYTES;
@@ -413,7 +478,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   const int zmat = blockIdx.z;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane (threadIdx.x >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
 
   // load addresses: x as in the fp16 kernel, instruction i of a wave covering
   // tile rows 8 g .. 8 g + 7 with g = wave + 8 i
@@ -449,7 +514,8 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
 
   // fragment reads
   const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
-  const int brow = (UPGATE ? wn * 32 : wn * 64) + (lane & 31);
+  // (rows of the weight tile: for the fused pair 0 .. 63 are up, 64 .. 127 gate)
+  const int brow = (WGN == 4 ? wn * 32 : UPGATE ? wn * 32 : wn * 64) + (lane & 31);
   const int qsw = (lane >> 1) & 3;
   uint32_t aoff[4], qoff[4];
 #pragma unroll
@@ -461,11 +527,11 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   const uint32_t soff = QS_BASE + brow * 4;
   constexpr int BJR = UPGATE ? 64 : 32; // rows from a wave's first to its second column block
 
-  float16v acc[QTM][WTN];
+  float16v acc[QTM][QTN];
 #pragma unroll
   for (int i = 0; i < QTM; ++i)
 #pragma unroll
-    for (int jn = 0; jn < WTN; ++jn)
+    for (int jn = 0; jn < QTN; ++jn)
 #pragma unroll
       for (int q = 0; q < 16; ++q)
         acc[i][jn][q] = 0.f;
@@ -487,8 +553,8 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   issue (nk > 1 ? 1 : 0, 1);
 
   half8 af[2][2][QTM];  // [block buffer][k-slice of the block][row block]
-  u32x2 bq[2][2][WTN];  // weight fragments as read (int8)
-  float d[2][WTN];      // the scales of the tile's two blocks
+  u32x2 bq[2][2][QTN];  // weight fragments as read (int8)
+  float d[2][QTN];      // the scales of the tile's two blocks
   auto read_block = [&] (int st, int blk, int buf) {
     const int sa = st * QA_BYTES, sq = st * QB_BYTES;
 #pragma unroll
@@ -496,7 +562,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
       {
         const int ks = 2 * blk + k2;
 #pragma unroll
-        for (int jn = 0; jn < WTN; ++jn)
+        for (int jn = 0; jn < QTN; ++jn)
           bq[buf][k2][jn] = *(const u32x2 *)(wide_lds + (qoff[ks] + sq) + jn * BJR * WBK);
 #pragma unroll
         for (int i = 0; i < QTM; ++i)
@@ -505,7 +571,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   };
   auto read_scales = [&] (int st) {
 #pragma unroll
-    for (int jn = 0; jn < WTN; ++jn)
+    for (int jn = 0; jn < QTN; ++jn)
       {
         const uint32_t sc = *(const uint32_t *)(wide_lds + (soff + st * QS_BYTES) + jn * BJR * 4);
         d[0][jn] = h2f ((uint16_t)(sc & 0xffff));
@@ -519,20 +585,20 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   // stand before the sixteen scaling FMAs of the one before; the order within
   // a block is left to the compiler (pinned with scheduling barriers it ran
   // 7 % slower).
-  auto multiply = [&] (int buf, const float (&dd)[WTN]) {
-    half8 bfc[2][WTN];
+  auto multiply = [&] (int buf, const float (&dd)[QTN]) {
+    half8 bfc[2][QTN];
 #pragma unroll
     for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
-      for (int jn = 0; jn < WTN; ++jn)
+      for (int jn = 0; jn < QTN; ++jn)
         bfc[k2][jn] = q8_frag (bq[buf][k2][jn]);
     float16v part[2];
 #pragma unroll
-    for (int p = 0; p <= QTM * WTN; ++p)
+    for (int p = 0; p <= QTM * QTN; ++p)
       {
-        if (p < QTM * WTN)
+        if (p < QTM * QTN)
           {
-            const int i = p / WTN, jn = p % WTN;
+            const int i = p / QTN, jn = p % QTN;
             float16v z;
 #pragma unroll
             for (int e = 0; e < 16; ++e)
@@ -542,7 +608,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
           }
         if (p > 0)
           {
-            const int i = (p - 1) / WTN, jn = (p - 1) % WTN;
+            const int i = (p - 1) / QTN, jn = (p - 1) % QTN;
 #pragma unroll
             for (int e = 0; e < 16; ++e)
               acc[i][jn][e] = __builtin_fmaf (part[(p - 1) & 1][e], dd[jn], acc[i][jn][e]);
@@ -562,13 +628,15 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   // st = kt % 3) are in buffer 0, the scales of both its blocks in d, and the
   // loads of tiles kt + 1 and kt + 2 are in flight or done.  (One copy of the
   // step with the stage as a variable: unrolled by the stages, the
-  // accumulators wander between sets of registers and the kernel spills.  Two
-  // stages, i.e. loads that have one k-step to arrive, ran 1.5 times slower.)
+  // accumulators wander between sets of registers and the kernel spills.)
   int st = 0;
   for (int kt = 0; kt < nk; ++kt)
     {
       const int s1 = st == QSTAGES - 1 ? 0 : st + 1;
-      const float d1[WTN] = { d[1][0], d[1][1] };
+      float d1[QTN];
+#pragma unroll
+      for (int jn = 0; jn < QTN; ++jn)
+        d1[jn] = d[1][jn];
       read_block (st, 1, 1);
       multiply (0, d[0]);
       __builtin_amdgcn_sched_barrier (0);
@@ -586,7 +654,10 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
       st = s1;
     }
   __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
-  wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+  if constexpr (WGN == 4)
+    wide_epilogue_tile<BM, UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+  else
+    wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
 }
 
 // Fewest tiles for which this form is used: below, too many of the 256 compute
@@ -653,13 +724,13 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
       VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, false>,
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, QGRID, false>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, true>,
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, QGRID, true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, false>,
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, QGRID, false>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, true>,
+      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, QGRID, true>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
       lds_set[dev] = true;
     }
@@ -679,16 +750,16 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
   if (a.wtype == 8 && bm == 256)
     {
       if (a.upgate)
-        gemm_wide_q8_kernel<256, true><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, QGRID, true><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
       else
-        gemm_wide_q8_kernel<256, false><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, QGRID, false><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
     }
   else if (a.wtype == 8)
     {
       if (a.upgate)
-        gemm_wide_q8_kernel<128, true><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<128, QGRID, true><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
       else
-        gemm_wide_q8_kernel<128, false><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<128, QGRID, false><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
     }
   else if (bm == 256)
     {
