@@ -2,15 +2,19 @@
 // call: scores, masked softmax and the product with V without the [H, S, L]
 // score and probability tensors ever reaching memory.
 //
-// The values rounded to fp16 are the ones the separate operators round:
-// score = fp16(scale * q.k), probability = fp16(exp(score - max) / sum), the
-// output sum_l p[l] v[l] in fp32 and rounded once.  To know max and sum before
-// the first probability is formed, the keys are walked twice: pass 1 computes
-// the scores and keeps a running maximum and a running sum of exponentials per
-// query, pass 2 computes the scores again, turns them into probabilities and
-// accumulates P V.  (The maximum is taken over the keys a query may see; it
-// cancels in the quotient, so taking it over masked keys as well, as the
-// separate softmax operator does, changes the result by fp32 rounding only.)
+// One pass over the keys with a running maximum (online softmax): per tile of
+// 64 keys the scores are formed (rounded to fp16 like the stand-alone product:
+// score = fp16(scale * q.k)), the maximum m is raised if needed - the products
+// accumulated so far and the sum of exponentials are then multiplied by
+// exp(m_old - m_new) -, the weights fp16(exp(score - m)) go into the second
+// product as they are, and the division by the sum of exponentials comes last,
+// in fp32, before the one rounding of the output.  The separate operators round
+// the NORMALISED probability to fp16 instead (p = fp16(exp(score - max) / sum));
+// the two differ by at most two half-ulp roundings of a weight, i.e. by
+// 2 * 2^-12 * sum_l p[l] |v[l]|, inside the 1e-2 the outputs are held to.  (A first
+// version walked the keys twice - maximum and sum first, then the very
+// probabilities of the operators - and took twice as long: two exponentials
+// per score and the scores computed twice.)
 //
 // Workgroup = 4 waves = 128 query rows of one head, 32 per wave; the keys come
 // through LDS in tiles of 64.  Both products run on v_mfma_f32_32x32x16_f16 in
@@ -21,7 +25,7 @@
 // Lane l of a wave owns query l % 32.  Of a 32-key block its 16 accumulator
 // registers hold the keys 8*(r/4) + 4*(l/32) + r%4, so maximum and sum over
 // keys are sums over a lane's own registers (the two lane halves are merged
-// once, after pass 1), and the probabilities it forms are, as they lie, the B
+// after every tile), and the weights it forms are, as they lie, the B
 // operand of the second product: registers 8t .. 8t+7 are the eight k values
 // of lane half l/32 in k-step t.  The V tile is written to LDS transposed and
 // with its keys permuted to that same order (slot 16t + 8h + j holds key
@@ -190,9 +194,13 @@ attn_prefill_kernel (const AttnArgs a)
   int head, qt;
   if ((a.H & 7) == 0)
     {
+      // j: position in the XCD's queue.  Its 32 compute units take the first
+      // 32 workgroups, then the next 32 beside them, and so on: every other
+      // such layer runs the tiles in the opposite order, so that a heavy tile
+      // and a light one share a compute unit.
       const int j = b >> 3;
       head = (b & 7) + 8 * (j / a.ntq);
-      qt = a.ntq - 1 - (j % a.ntq);
+      qt = ((j >> 5) & 1) ? j % a.ntq : a.ntq - 1 - (j % a.ntq);
     }
   else
     {
@@ -219,54 +227,10 @@ attn_prefill_kernel (const AttnArgs a)
   }
 
   Tile<HD> tl;
-  // ---- pass 1: maximum and sum of exponentials per query ---------------------
+  // One pass over the keys with a running maximum: the accumulated products
+  // and the sum of exponentials are rescaled whenever the maximum grows, and
+  // the division by the sum comes last.
   float m = kNeg, sum = 0.f;
-  load_k<HD> (a, kb, 0, tl);
-  for (int t = 0; t < ntile; ++t)
-    {
-      __syncthreads ();
-      store_k<HD> (tl, Ks);
-      __syncthreads ();
-      if (t + 1 < ntile)
-        load_k<HD> (a, kb, t + 1, tl);
-      if (t * kBKey > wave_last)
-        continue;
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
-        {
-          const float16v acc = score_block<HD> (Ks, blk, qf, lane);
-          const int key0 = t * kBKey + 32 * blk + 4 * hh;
-          float sv[16];
-          float bm = kNeg;
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            {
-              const int key = key0 + 8 * (r >> 2) + (r & 3);
-              const float s = vkl::h2f (vkl::f2h (acc[r] * a.scale));
-              sv[r] = key <= qrow + shift ? s : kNeg;
-              bm = fmaxf (bm, sv[r]);
-            }
-          const float mn = fmaxf (m, bm);
-          float add = 0.f;
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            add += sv[r] > 0.5f * kNeg ? fast_exp (sv[r] - mn) : 0.f;
-          sum = sum * fast_exp (m - mn) + add;
-          m = mn;
-        }
-    }
-  // the other half of the lanes holds the other keys of the same query
-  {
-    const float mo = __shfl_xor (m, 32, 64), so = __shfl_xor (sum, 32, 64);
-    const float M = fmaxf (m, mo);
-    sum = sum * fast_exp (m - M) + so * fast_exp (mo - M);
-    m = M;
-  }
-
-  // ---- pass 2: probabilities and P V -----------------------------------------
-  // exp(s - max) * (1 / sum) instead of a division per key: the two differ by
-  // one rounding of an fp32 value that is rounded to fp16 next
-  const float inv = 1.0f / sum;
   float16v oacc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -288,7 +252,11 @@ attn_prefill_kernel (const AttnArgs a)
         }
       if (t * kBKey > wave_last)
         continue;
-      half8 pf[2][2];
+      // scores of the tile's 64 keys, rounded to fp16 like the stand-alone
+      // product; a key the query must not see counts as "never seen"
+      float sv[2][16];
+      float bm = kNeg;
+      const bool inner = t * kBKey + kBKey - 1 <= q0 + wave * 32 + shift; // every key visible to every query of the wave
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
         {
@@ -298,11 +266,36 @@ attn_prefill_kernel (const AttnArgs a)
           for (int r = 0; r < 16; ++r)
             {
               const int key = key0 + 8 * (r >> 2) + (r & 3);
-              const float s = vkl::h2f (vkl::f2h (acc[r] * a.scale));
-              const float p = key <= qrow + shift ? fast_exp (s - m) * inv : 0.f;
-              pf[blk][r >> 3][r & 7] = (_Float16)p;
+              const float sc = vkl::h2f (vkl::f2h (acc[r] * a.scale));
+              sv[blk][r] = inner || key <= qrow + shift ? sc : kNeg;
+              bm = fmaxf (bm, sv[blk][r]);
             }
         }
+      // the two halves of the lanes hold different keys of the same query and
+      // feed one product: they need the same maximum
+      bm = fmaxf (bm, __shfl_xor (bm, 32, 64));
+      const float mn = fmaxf (m, bm);
+      if (__builtin_amdgcn_ballot_w64 (mn != m) != 0)
+        {
+          const float alpha = fast_exp (m - mn); // 0 before the first key, 1 where the maximum stays
+          sum *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              oacc[db][r] *= alpha;
+          m = mn;
+        }
+      half8 pf[2][2];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          {
+            const float e = fast_exp (sv[blk][r] - m); // exp (kNeg - m) = 0
+            sum += e;
+            pf[blk][r >> 3][r & 7] = (_Float16)e;
+          }
 #pragma unroll
       for (int db = 0; db < DB; ++db)
         {
@@ -315,6 +308,14 @@ attn_prefill_kernel (const AttnArgs a)
                   *(const half8 *)(vp + 32 * blk + 16 * t2), pf[blk][t2], oacc[db], 0, 0, 0);
         }
     }
+  // the other half of the lanes has summed the other keys of the same query
+  sum += __shfl_xor (sum, 32, 64);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      oacc[db][r] *= inv;
 
   if (qrow >= a.S)
     return;
