@@ -51,9 +51,16 @@ int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
 size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
 // Many token rows against dense fp16 weights: 256-row tiles staged by
 // direct-to-LDS loads (vkl_gemm_wide.hip).  gemm_mfma_launch takes this form
-// where it applies; no workspace.
+// where it applies.
 bool gemm_wide_supported (const GemmArgs &a);
 int gemm_wide_launch (const GemmArgs &a, hipStream_t s);
+size_t gemm_wide_workspace_bytes (const GemmArgs &a); // fp32 scratch of its k-split (0: none)
+// The k-split forms' fp32 scratch of a stream (allocated on first use; null if
+// that fails), its size, and the kernel that adds `parts` partial results of
+// `rows` rows each in order and applies the epilogue.
+float *gemm_stream_workspace (hipStream_t s);
+size_t gemm_stream_workspace_bytes ();
+int gemm_reduce_parts (const GemmArgs &a, const float *ws, int parts, int rows, hipStream_t s);
 // frees the scratch buffer that launches on this stream allocated (the
 // stream must be idle); called when a stream is destroyed
 void gemm_release_workspace (hipStream_t s);

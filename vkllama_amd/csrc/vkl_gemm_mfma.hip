@@ -1222,6 +1222,26 @@ launch_cfg (const GemmArgs &a, hipStream_t s)
 }
 } // namespace
 
+float *
+gemm_stream_workspace (hipStream_t s)
+{
+  return skinny2_workspace (s);
+}
+
+size_t
+gemm_stream_workspace_bytes ()
+{
+  return kSk2Workspace;
+}
+
+int
+gemm_reduce_parts (const GemmArgs &a, const float *ws, int parts, int rows, hipStream_t s)
+{
+  const size_t total = (size_t)a.M * a.N;
+  skinny2_reduce_kernel<<<dim3 ((unsigned)((total + 255) / 256)), dim3 (256), 0, s>>> (a, ws, parts, rows);
+  return (int)hipGetLastError ();
+}
+
 bool
 gemm_mfma_supported (const GemmArgs &a)
 {
@@ -1318,7 +1338,7 @@ gemm_mfma_workspace_bytes (const GemmArgs &a)
         return need;
     }
   if (gemm_wide_supported (a))
-    return 0;
+    return gemm_wide_workspace_bytes (a);
   const bool small = half_height_tiles (a);
   int ksplit;
   if (a.wtype == 8)

@@ -1,6 +1,7 @@
-// y[M,N] = x[M,K] W[N,K]^T for many token rows (prompt passes of a thousand
-// tokens and more), fp16 activations and dense fp16 weights, fp32 accumulation
-// on the matrix cores (v_mfma_f32_32x32x16_f16).
+// y[M,N] = x[M,K] W[N,K]^T for many token rows (prompt passes of 128 tokens
+// and more), fp16 activations and dense fp16 or planar Q8_0 weights, fp32
+// accumulation on the matrix cores (v_mfma_f32_32x32x16_f16).  First the
+// kernel for fp16 weights; the one for Q8_0 weights follows it.
 //
 // One workgroup of four waves per compute unit owns a 256 x 128 output tile;
 // each wave a 128 x 64 quarter (4 x 2 accumulators of 32 x 32).  A k-step is 64
@@ -77,8 +78,28 @@ constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 12
 // residual, the stores.
 template <bool UPGATE>
 __device__ __forceinline__ void
-wide_finish8 (const GemmArgs &a, float (&v)[8], const float (&g)[8], int m, int ncol0, int zmat, int vec)
+wide_finish8 (const GemmArgs &a, float (&v)[8], const float (&g)[8], int m, int ncol0, int zmat, int vec,
+              float *part)
 {
+  if (!UPGATE && part)
+    {
+      // one part of a split k range: the raw sums, dense [M, N] fp32; the
+      // reduction kernel adds the parts in order and applies the rest
+      if (m >= a.M || ncol0 >= a.N)
+        return;
+      float *dst = part + (size_t)m * a.N + ncol0;
+      if ((a.N % 4) == 0 && ncol0 + 8 <= a.N)
+        {
+          typedef float f32x4 __attribute__ ((ext_vector_type (4)));
+          f32x4 w0 = { v[0], v[1], v[2], v[3] }, w1 = { v[4], v[5], v[6], v[7] };
+          *(VKL_GLOBAL f32x4 *)dst = w0;
+          *(VKL_GLOBAL f32x4 *)(dst + 4) = w1;
+        }
+      else
+        for (int e = 0; e < 8 && ncol0 + e < a.N; ++e)
+          dst[e] = v[e];
+      return;
+    }
   uint16_t *y = a.y[UPGATE ? 0 : zmat];
   const bool plain = a.nmat != 1; // one of three fused outputs: no scale, activation, residual
   if (UPGATE)
@@ -147,7 +168,7 @@ wide_finish8 (const GemmArgs &a, float (&v)[8], const float (&g)[8], int m, int 
 template <bool UPGATE, int TM>
 __device__ __forceinline__ void
 wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_lds, int wave, int lane,
-               int m0, int n0, int zmat, int vec)
+               int m0, int n0, int zmat, int vec, float *part)
 {
   // waves are numbered row block first: wave = 2 wm + wn, TM x 32 rows by 64 columns each
   constexpr int ROWS = TM * 32;
@@ -183,7 +204,7 @@ wide_epilogue (const GemmArgs &a, const float16v (&acc)[TM][WTN], uint8_t *wide_
           const float4 g1 = *(const float4 *)(park + row * LD + 32 + ec + 4);
           g[0] = g0.x, g[1] = g0.y, g[2] = g0.z, g[3] = g0.w, g[4] = g1.x, g[5] = g1.y, g[6] = g1.z, g[7] = g1.w;
         }
-      wide_finish8<UPGATE> (a, v, g, m0 + wm * ROWS + row, ncol0, zmat, vec);
+      wide_finish8<UPGATE> (a, v, g, m0 + wm * ROWS + row, ncol0, zmat, vec, part);
     }
 }
 
@@ -195,7 +216,7 @@ constexpr int kWideTileLd = 132;
 template <int BM, bool UPGATE, int TM>
 __device__ __forceinline__ void
 wide_epilogue_tile (const GemmArgs &a, const float16v (&acc)[TM][1], uint8_t *wide_lds, int wave, int lane,
-                    int m0, int n0, int zmat, int vec)
+                    int m0, int n0, int zmat, int vec, float *part)
 {
   constexpr int LD = kWideTileLd;
   const int wm = wave >> 2, wn = wave & 3;
@@ -226,7 +247,7 @@ wide_epilogue_tile (const GemmArgs &a, const float16v (&acc)[TM][1], uint8_t *wi
           const float4 g1 = *(const float4 *)(park + row * LD + 64 + ec + 4);
           g[0] = g0.x, g[1] = g0.y, g[2] = g0.z, g[3] = g0.w, g[4] = g1.x, g[5] = g1.y, g[6] = g1.z, g[7] = g1.w;
         }
-      wide_finish8<UPGATE> (a, v, g, m0 + row, n0 + ec, zmat, vec);
+      wide_finish8<UPGATE> (a, v, g, m0 + row, n0 + ec, zmat, vec, part);
     }
 }
 
@@ -242,7 +263,7 @@ wide_lds_f16 ()
 // occupy the compute units) 128, i.e. 64 x 64 per wave.
 template <int BM, bool UPGATE>
 __global__ __launch_bounds__ (WWAVES * 64) void
-gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
+gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec, int ksplit, float *ws)
 {
   constexpr int TM = BM / 2 / 32;                    // 32-row accumulators per wave
   constexpr int STAGE_BYTES = (BM + WBN) * WROWB;
@@ -253,9 +274,17 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
   // tiles, token-row tile fastest, so the weight tiles it shares stay in its L2
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int tile = xcd * per_xcd + j;
-  if (j >= per_xcd || tile >= tiles_m * tiles_n)
+  // ksplit > 1: the k range is divided among ksplit workgroups per output
+  // tile; each writes its fp32 sums to the workspace, a second kernel adds them
+  const int plane = tiles_m * tiles_n;
+  if (j >= per_xcd || tile >= plane * ksplit)
     return;
-  const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
+  const int ks = tile / plane, t2 = tile - ks * plane;
+  const int tn = t2 / tiles_m, tm = t2 - tn * tiles_m;
+  const int nk_all = a.K / WBK;
+  const int kbase = (int)((long)nk_all * ks / ksplit);
+  const int nk = (int)((long)nk_all * (ks + 1) / ksplit) - kbase; // k-steps of this workgroup
+  float *part = ksplit > 1 ? ws + (size_t)ks * a.M * a.N : nullptr;
   const int bn_rows = UPGATE ? WBN / 2 : WBN; // weight rows per matrix and tile
   const int m0 = tm * BM, n0 = tn * bn_rows;
   const int zmat = blockIdx.z;
@@ -275,7 +304,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
   for (int i = 0; i < AG; ++i)
     {
       const int m = min (m0 + (wave + WWAVES * i) * 8 + lr, a.M - 1);
-      src[i] = a.x + (size_t)m * a.xs + chunk * 8;
+      src[i] = a.x + (size_t)m * a.xs + chunk * 8 + (size_t)kbase * WBK;
     }
 #pragma unroll
   for (int i = AG; i < GPW; ++i)
@@ -284,7 +313,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
       const int mat = UPGATE ? v >> 6 : zmat;
       const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
       const uint16_t *w = mat == 0 ? a.wh[0] : (mat == 1 ? a.wh[1] : a.wh[2]);
-      src[i] = w + (size_t)n * a.ws + chunk * 8;
+      src[i] = w + (size_t)n * a.ws + chunk * 8 + (size_t)kbase * WBK;
     }
 
   // fragment reads: lane l holds row l%32 of a 32-row block, k = 16 ks + 8 (l/32) .. +7
@@ -308,7 +337,6 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
       for (int q = 0; q < 16; ++q)
         acc[i][jn][q] = 0.f;
 
-  const int nk = a.K / WBK;
   auto issue_part = [&] (int kt, int st, int i0, int i1) {
 #pragma unroll
     for (int i = i0; i < i1; ++i)
@@ -399,7 +427,7 @@ gemm_wide_f16_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, i
     step (kt + 1, WideInt<1> ());
   __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
 
-  wide_epilogue<UPGATE, TM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+  wide_epilogue<UPGATE, TM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec, part);
 }
 
 // ---------------------------------------------------------------------------
@@ -458,7 +486,7 @@ q8_frag (u32x2 r)
 // instead of four).
 template <int BM, int WGN, bool UPGATE>
 __global__ __launch_bounds__ (QWAVES * 64) void
-gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec)
+gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, int vec, int ksplit, float *ws)
 {
   constexpr int QTM = BM / (QWAVES / WGN) / 32; // 32-row accumulators per wave
   constexpr int QTN = 4 / WGN;                  // 32-column accumulators per wave
@@ -470,9 +498,17 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   extern __shared__ __align__ (16) uint8_t wide_lds[];
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int tile = xcd * per_xcd + j;
-  if (j >= per_xcd || tile >= tiles_m * tiles_n)
+  // ksplit > 1: the k range is divided among ksplit workgroups per output
+  // tile; each writes its fp32 sums to the workspace, a second kernel adds them
+  const int plane = tiles_m * tiles_n;
+  if (j >= per_xcd || tile >= plane * ksplit)
     return;
-  const int tn = tile / tiles_m, tm = tile - tn * tiles_m;
+  const int ks = tile / plane, t2 = tile - ks * plane;
+  const int tn = t2 / tiles_m, tm = t2 - tn * tiles_m;
+  const int nk_all = a.K / WBK;
+  const int kbase = (int)((long)nk_all * ks / ksplit);
+  const int nk = (int)((long)nk_all * (ks + 1) / ksplit) - kbase; // k-steps of this workgroup
+  float *part = ksplit > 1 ? ws + (size_t)ks * a.M * a.N : nullptr;
   const int bn_rows = UPGATE ? WBN / 2 : WBN;
   const int m0 = tm * BM, n0 = tn * bn_rows;
   const int zmat = blockIdx.z;
@@ -489,7 +525,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
   for (int i = 0; i < QAG; ++i)
     {
       const int m = min (m0 + (wave + QWAVES * i) * 8 + lr, a.M - 1);
-      src[i] = (const uint8_t *)(a.x + (size_t)m * a.xs + chunk * 8);
+      src[i] = (const uint8_t *)(a.x + (size_t)m * a.xs + chunk * 8 + (size_t)kbase * WBK);
     }
   // quants: a wave's one instruction covers weight-tile rows 16 wave .. + 15;
   // lane l fetches chunk (l%4) ^ ((row >> 1) & 3) of row 16 wave + l/4
@@ -499,7 +535,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
     const int mat = UPGATE ? v >> 6 : zmat;
     const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
     const uint8_t *w = mat == 0 ? a.wq[0] : (mat == 1 ? a.wq[1] : a.wq[2]);
-    src[QAG] = w + (size_t)n * a.Kp + ((lane & 3) ^ ((qr >> 1) & 3)) * 16;
+    src[QAG] = w + (size_t)n * a.Kp + ((lane & 3) ^ ((qr >> 1) & 3)) * 16 + (size_t)kbase * WBK;
   }
   // scales: the two of a row are one dword; a wave fetches rows 64 (wave & 1)
   // + lane (four waves write each half, all the same values), so that every
@@ -509,7 +545,7 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
     const int mat = UPGATE ? v >> 6 : zmat;
     const int n = min (UPGATE ? n0 + (v & 63) : n0 + v, a.N - 1);
     const uint16_t *ds = mat == 0 ? a.wd[0] : (mat == 1 ? a.wd[1] : a.wd[2]);
-    src[QAG + 1] = (const uint8_t *)(ds + (size_t)n * (a.Kp >> 5));
+    src[QAG + 1] = (const uint8_t *)(ds + (size_t)n * (a.Kp >> 5) + (size_t)kbase * 2);
   }
 
   // fragment reads
@@ -536,7 +572,6 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
       for (int q = 0; q < 16; ++q)
         acc[i][jn][q] = 0.f;
 
-  const int nk = a.K / WBK;
   auto issue = [&] (int kt, int st) {
 #pragma unroll
     for (int i = 0; i < QAG; ++i)
@@ -655,18 +690,28 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
     }
   __builtin_amdgcn_s_waitcnt (0x0f70); // no load may outlive the workgroup's LDS
   if constexpr (WGN == 4)
-    wide_epilogue_tile<BM, UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+    wide_epilogue_tile<BM, UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec, part);
   else
-    wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec);
+    wide_epilogue<UPGATE, QTM> (a, acc, wide_lds, wave, lane, m0, n0, zmat, vec, part);
 }
 
-// Fewest tiles for which this form is used: below, too many of the 256 compute
-// units would idle and the tile kernel with its k-split does better (measured
-// on the 7B shapes, 256 to 2048 rows).
-constexpr int kWideMinHalfTiles = 88, kWideMinHalfTilesQ8 = 160;
-// time of a round of 128-row tiles relative to one of 256-row tiles (31-38 us
-// against 46-51 us at K = 4096)
-constexpr double kWideHalfRound = 0.68;
+// Which tile height and how many parts of the k range: the pair with the
+// lowest estimated time, from a model fitted to measurements on the 7B shapes
+// (microseconds: a round of 256-row tiles over the 256 compute units takes
+// about 0.95 per k-step + 8, one of 128-row tiles 0.55 per k-step + 6, Q8_0
+// weights 1.6 times that; a reduction launch 5 + its bytes at 2.5 TB/s).
+// Below kWideMinGroups workgroups the tile kernel of vkl_gemm_mfma.hip does
+// better.
+#ifndef VKL_WIDE_MIN_GROUPS
+#define VKL_WIDE_MIN_GROUPS 88
+#endif
+constexpr int kWideMinGroups = VKL_WIDE_MIN_GROUPS, kWideMinGroupsQ8 = VKL_WIDE_MIN_GROUPS > 128 ? VKL_WIDE_MIN_GROUPS : 128;
+
+struct WidePlan
+{
+  int bm;     // token rows of a tile, 0: this form does not apply
+  int ksplit; // parts of the k range
+};
 
 long
 wide_tiles (const GemmArgs &a, int bm)
@@ -675,34 +720,59 @@ wide_tiles (const GemmArgs &a, int bm)
          * (a.upgate ? 1 : a.nmat);
 }
 
-// token rows of the tile to use, 0: this form does not apply
-int
-wide_tile_rows (const GemmArgs &a)
+WidePlan
+wide_plan (const GemmArgs &a)
 {
-  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0)
-    return 0;
+  WidePlan none = { 0, 1 }, best = none;
+  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < 128)
+    return none;
   if (a.wtype == 8)
     {
       // whole k-steps of quants and scale pairs, aligned for 16- and 4-byte loads
       if (a.Kp != a.K)
-        return 0;
+        return none;
       for (int t = 0; t < (a.upgate ? 2 : a.nmat); ++t)
         if (((uintptr_t)a.wq[t] % 16) != 0 || ((uintptr_t)a.wd[t] % 4) != 0)
-          return 0;
+          return none;
     }
-  // the tile height whose rounds over the 256 compute units take less time
-  const long t128 = wide_tiles (a, 128), t256 = wide_tiles (a, WBM);
-  if (a.M < 128 || t128 < (a.wtype == 8 ? kWideMinHalfTilesQ8 : kWideMinHalfTiles))
-    return 0;
-  const double c256 = (double)((t256 + 255) / 256), c128 = (double)((t128 + 255) / 256) * kWideHalfRound;
-  return a.M >= WBM && c256 <= c128 ? WBM : 128;
+  const int nk = a.K / WBK;
+  const double wq = a.wtype == 8 ? 1.6 : 1.0;
+  const size_t ws_bytes = a.workspace ? a.workspace_bytes : gemm_stream_workspace_bytes ();
+  double best_cost = 0;
+  for (int bm = 128; bm <= WBM; bm *= 2)
+    for (int ks = 1; ks <= 4; ks *= 2)
+      {
+        if (a.M < bm)
+          continue;
+        // parts only for one matrix with the plain epilogue, of at least 16
+        // k-steps each, and as far as the scratch holds them
+        if (ks > 1
+            && (a.upgate || a.nmat != 1 || nk / ks < 16 || (size_t)ks * a.M * a.N * sizeof (float) > ws_bytes))
+          continue;
+        const long groups = wide_tiles (a, bm) * ks;
+        if (groups < (a.wtype == 8 ? kWideMinGroupsQ8 : kWideMinGroups))
+          continue;
+        const double round = wq * (bm == WBM ? 0.95 * nk / ks + 8 : 0.55 * nk / ks + 6);
+        const double reduce = ks > 1 ? 5 + (double)ks * a.M * a.N * sizeof (float) / 2.5e6 : 0;
+        const double cost = (double)((groups + 255) / 256) * round + reduce;
+        if (!best.bm || cost < best_cost)
+          best = { bm, ks }, best_cost = cost;
+      }
+  return best;
 }
 } // namespace
 
 bool
 gemm_wide_supported (const GemmArgs &a)
 {
-  return wide_tile_rows (a) != 0;
+  return wide_plan (a).bm != 0;
+}
+
+size_t
+gemm_wide_workspace_bytes (const GemmArgs &a)
+{
+  const WidePlan p = wide_plan (a);
+  return p.bm && p.ksplit > 1 ? (size_t)p.ksplit * a.M * a.N * sizeof (float) : 0;
 }
 
 int
@@ -734,12 +804,17 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
       lds_set[dev] = true;
     }
-  const int bm = wide_tile_rows (a);
+  const WidePlan plan = wide_plan (a);
+  const int bm = plan.bm;
+  int ksplit = plan.ksplit;
   if (!bm)
     return (int)hipErrorInvalidValue;
+  float *ws = nullptr;
+  if (ksplit > 1 && !(ws = a.workspace ? a.workspace : gemm_stream_workspace (s)))
+    ksplit = 1;
   const int tiles_m = (a.M + bm - 1) / bm;
   const int tiles_n = (a.N + (a.upgate ? 63 : 127)) / (a.upgate ? 64 : 128);
-  const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+  const int per_xcd = (tiles_m * tiles_n * ksplit + 7) / 8;
   const dim3 grid ((unsigned)(per_xcd * 8), 1, (unsigned)(a.upgate ? 1 : a.nmat));
   const dim3 block ((a.wtype == 8 ? QWAVES : WWAVES) * 64);
   // 16-byte accesses to the outputs (and the residual) where their rows allow it
@@ -750,28 +825,30 @@ gemm_wide_launch (const GemmArgs &a, hipStream_t s)
   if (a.wtype == 8 && bm == 256)
     {
       if (a.upgate)
-        gemm_wide_q8_kernel<256, QGRID, true><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, QGRID, true><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
       else
-        gemm_wide_q8_kernel<256, QGRID, false><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<256, QGRID, false><<<grid, block, q256, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
     }
   else if (a.wtype == 8)
     {
       if (a.upgate)
-        gemm_wide_q8_kernel<128, QGRID, true><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<128, QGRID, true><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
       else
-        gemm_wide_q8_kernel<128, QGRID, false><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_q8_kernel<128, QGRID, false><<<grid, block, q128, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
     }
   else if (bm == 256)
     {
       if (a.upgate)
-        gemm_wide_f16_kernel<256, true><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_f16_kernel<256, true><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
       else
-        gemm_wide_f16_kernel<256, false><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+        gemm_wide_f16_kernel<256, false><<<grid, block, lds256, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
     }
   else if (a.upgate)
-    gemm_wide_f16_kernel<128, true><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    gemm_wide_f16_kernel<128, true><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
   else
-    gemm_wide_f16_kernel<128, false><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec);
+    gemm_wide_f16_kernel<128, false><<<grid, block, lds128, s>>> (a, tiles_m, tiles_n, per_xcd, vec, ksplit, ws);
+  if (ksplit > 1)
+    return gemm_reduce_parts (a, ws, ksplit, a.M, s);
   return (int)hipGetLastError ();
 }
 } // namespace vkl
