@@ -141,7 +141,7 @@ def test_matmul_q8_0_epilogue(dev, rng):
                                    (129, 64, 11008), (65, 32000, 512),
                                    (7, 200, 1376), (32, 129, 768), (5, 64, 256), (31, 300, 11008), (2, 1000, 5120),
                                    (270, 12300, 64), (600, 13000, 192), (1030, 6144, 448), (777, 8200, 320),
-                                   (300, 8192, 64)])
+                                   (300, 8192, 64), (256, 4096, 2048)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
@@ -150,24 +150,26 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     full-height tiles, the k-split, and (the last five: about two hundred
     256 x 128 tiles and more, or half as many 128 x 128 ones, K a multiple of
     64) the form that loads its tiles straight into LDS, with ragged M and N,
-    one to seven k-steps."""
+    one to seven k-steps, and (the last) its k range split in two."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
-    if M * N * K <= 3e8:
+    if M * N * K <= 3e8 or K == 2048:
         want = O.matmul_q8_0(x, raw, K)
         assert rel_err(got, want) < F16_REL_TOL
     exact = x.astype(np.float64) @ deq[:, :K].T
     assert rel_err(got, exact) < 2e-3
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 200, 512), (72, 200, 2048), (20, 200, 2048), (260, 12300, 64)])
+@pytest.mark.parametrize("M,N,K", [(40, 200, 512), (72, 200, 2048), (20, 200, 2048), (260, 12300, 64),
+                                   (260, 4096, 2048)])
 def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     """scale / bias / activation, residual, widened copy and row strides: on
     the tile kernel without (K 512) and with the k-split, on the few-row
     kernel (20 rows; these two finish in the reduction kernel) and on the
     256-row tiles (260 rows: 16-byte stores, and single ones where the output
-    rows are not 16-byte aligned)"""
+    rows are not 16-byte aligned; with K 2048 the k range split in two, which
+    finishes in the reduction kernel as well)"""
     raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
     x = rng.standard_normal((M, K)).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
@@ -255,12 +257,12 @@ def test_matmul_f16_tb(dev, rng, C, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512),
                                    (512, 12800, 64), (600, 13000, 96), (600, 13000, 128), (777, 8200, 320),
-                                   (256, 24576, 192), (1030, 6144, 448), (300, 6144, 128), (130, 12000, 192)])
+                                   (256, 24576, 192), (1030, 6144, 448), (300, 6144, 128), (130, 12000, 192), (200, 4096, 2048)])
 def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     """FP16 weights, many token rows: the matrix-core paths (from about two
     hundred 256 x 128 output tiles on, or half as many 128 x 128 ones, with K a
     multiple of 64, the form that loads its tiles straight into LDS; ragged M
-    and N included)."""
+    and N included; the last shape with its k range split in two)."""
     a = rng.standard_normal((1, M, K)).astype(np.float16)
     b = (rng.standard_normal((1, N, K)) * 0.05).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
