@@ -170,8 +170,13 @@ int vkl_rope_kvwrite_f16 (void *q, const void *k, const void *v, int S, int H,
 /* The attention core of src/ops/multiheadattention_v2.cpp:290-309 in one
  * launch for many query rows: matmul_b0_tb_fp16_v2.comp (scores = fp16(scale
  * q.k)), softmax_fp16.comp with seq_mask (key l is masked iff l > s + (L - S))
- * and matmul_broadcast0_fp16_v2.comp (P V), with the same fp16 rounding points
- * and neither scores nor probabilities stored.  q [H,S,hd] with strides (qcs,
+ * and matmul_broadcast0_fp16_v2.comp (P V), with neither scores nor
+ * probabilities stored.  Scores and output are rounded to fp16 where the
+ * shaders round them; the softmax runs with a running maximum and the
+ * division by the sum of exponentials last, so the fp16 weights of the second
+ * product are exp(score - max) instead of the normalised probabilities
+ * (outputs within 5e-3 of the three shaders' relative to the size of the terms
+ * summed; the operators' bar is 1e-2).  q [H,S,hd] with strides (qcs,
  * qhs); k, v [H,L,hd] views with strides (kcs, khs), (vcs, vhs), e.g. the
  * first L rows of a [H,maxlen,hd] cache; out[s*ors + h*ohs + d] (ors = H*hd,
  * ohs = hd gives the [S, H*hd] layout the output projection reads; ors = hd,
