@@ -184,8 +184,10 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
   // launches on the projection outputs as they lie ([S, heads*dim]): RoPE of
   // Q and K + cache write, then scores / masked softmax / P V.  Reshapes,
   // transposes, the clip of Q to its last row and the cache views of the
-  // operator-by-operator form below become index arithmetic; the values and
-  // their fp16 rounding points are the same.
+  // operator-by-operator form below become index arithmetic.  RoPE and the
+  // cache rows are bit-identical to that form; the attention kernel rounds
+  // scores and outputs where the operators do but forms its softmax with a
+  // running maximum (see vkl_attn_prefill_causal_f16).
   attn_fused_last_ = false;
   if (use_kvcache_ && dtype_ == FP16 && (dim_ == 64 || dim_ == 128)
       && k.dtype () == FP16 && q.dtype () == FP16 && v.dtype () == FP16)
@@ -269,8 +271,9 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
     }
 
   // scores, masked softmax and P V in one launch, written as [seqlen,
-  // heads*dim]: same rounding points as the three operators below, without
-  // the [heads, seqlen, read_len] tensors in memory
+  // heads*dim]: the three operators below without the [heads, seqlen,
+  // read_len] tensors in memory (online softmax: outputs within 5e-3 of
+  // theirs relative to the size of the terms summed)
   if (dtype_ == FP16 && (dim_ == 64 || dim_ == 128) && roped_q->dtype () == FP16
       && roped_k->dtype () == FP16 && transposed_v->dtype () == FP16)
     {
