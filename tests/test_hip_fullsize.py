@@ -71,13 +71,15 @@ def test_c3_llama2_7b_q8_0_against_oracle():
     assert logit_err(got, want) < 1e-2
     assert margin_ok(got, want)
     ids = [int(np.argmax(want))]
-    same = int(np.argmax(got)) == ids[0]
+    gpu_ids = [int(np.argmax(got))]  # the GPU's choice at each step of the oracle's sequence
+    same = gpu_ids[0] == ids[0]
     pos = 32
     for _ in range(31):
         got, want = m.forward([ids[-1]], pos), om.forward([ids[-1]], pos)
         assert logit_err(got, want) < 1e-2, pos
         assert margin_ok(got, want), pos
         same += int(np.argmax(got)) == int(np.argmax(want))
+        gpu_ids.append(int(np.argmax(got)))
         ids.append(int(np.argmax(want)))
         pos += 1
     # the committed fixture is the oracle's sequence
@@ -85,7 +87,8 @@ def test_c3_llama2_7b_q8_0_against_oracle():
     assert same >= 30
     # the greedy loop: replayed from a graph (bench.py's form), launched step
     # by step, and as one persistent launch per token give one sequence, which
-    # follows the oracle's up to the first near-tie
+    # follows the oracle's up to the first near-tie (where margin_ok above has
+    # already accepted the GPU's choice) and takes the GPU's choice there
     ids1, _, _ = m.generate_greedy(prompt, 32)
     m.set_option("decode_graph", 0)
     ids2, _, _ = m.generate_greedy(prompt, 32)
@@ -93,7 +96,8 @@ def test_c3_llama2_7b_q8_0_against_oracle():
     m.set_option("decode_mode", 1)
     ids3, _, _ = m.generate_greedy(prompt, 32)
     assert list(ids3) == list(ids1)
-    assert [int(t) for t in ids1[:6]] == gold["oracle_ids"][:6]
+    n = next((i for i in range(32) if int(ids1[i]) != ids[i]), 32)
+    assert [int(t) for t in ids1[:n + 1]] == gpu_ids[:n + 1]
     m.close()
 
 

@@ -141,7 +141,8 @@ def test_matmul_q8_0_epilogue(dev, rng):
                                    (129, 64, 11008), (65, 32000, 512),
                                    (7, 200, 1376), (32, 129, 768), (5, 64, 256), (31, 300, 11008), (2, 1000, 5120),
                                    (270, 12300, 64), (600, 13000, 192), (1030, 6144, 448), (777, 8200, 320),
-                                   (300, 8192, 64), (256, 4096, 2048)])
+                                   (300, 8192, 64), (256, 4096, 2048),
+                                   (9, 6416, 1024), (32, 12288, 768), (3, 16368, 1280)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
@@ -150,11 +151,14 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     full-height tiles, the k-split, and (the last five: about two hundred
     256 x 128 tiles and more, or half as many 128 x 128 ones, K a multiple of
     64) the form that loads its tiles straight into LDS, with ragged M and N,
-    one to seven k-steps, and (the last) its k range split in two."""
+    one to seven k-steps, and its k range split in two; the last three: at
+    most 32 token rows against 512 and more groups of 16 weight rows, K a
+    multiple of 256: workgroups that run over the whole of K (2, 3 and 4
+    groups each, the last workgroup not full)."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
-    if M * N * K <= 3e8 or K == 2048:
+    if M * N * K <= 3e8 or K == 2048 or M <= 32:
         want = O.matmul_q8_0(x, raw, K)
         assert rel_err(got, want) < F16_REL_TOL
     exact = x.astype(np.float64) @ deq[:, :K].T
@@ -162,14 +166,15 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(40, 200, 512), (72, 200, 2048), (20, 200, 2048), (260, 12300, 64),
-                                   (260, 4096, 2048)])
+                                   (260, 4096, 2048), (20, 8224, 1024)])
 def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     """scale / bias / activation, residual, widened copy and row strides: on
     the tile kernel without (K 512) and with the k-split, on the few-row
     kernel (20 rows; these two finish in the reduction kernel) and on the
     256-row tiles (260 rows: 16-byte stores, and single ones where the output
     rows are not 16-byte aligned; with K 2048 the k range split in two, which
-    finishes in the reduction kernel as well)"""
+    finishes in the reduction kernel as well), and on the few-row kernel whose
+    workgroups run over the whole of K (20 rows x 8224)"""
     raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
     x = rng.standard_normal((M, K)).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
@@ -192,8 +197,12 @@ def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     assert not yw[:, N:].any()
 
 
-@pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376), (258, 4200, 64), (130, 5200, 64)])
+@pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376), (258, 4200, 64), (130, 5200, 64),
+                                   (32, 4096, 4096), (7, 4112, 768), (17, 5120, 1024), (2, 2736, 1024)])
 def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
+    """(the last four: at most 32 token rows and 512 and more groups of 16
+    weight rows over the three matrices: workgroups over the whole of K, 3, 4, 4
+    and 3 consecutive groups each, also across the end of a matrix)"""
     ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
     x = rng.standard_normal((M, K)).astype(np.float16)
     dx = dev.upload(x)
@@ -206,8 +215,12 @@ def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
         assert rel_err(f16(o, (M, N)), w) < F16_REL_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128), (200, 7800, 64)])
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128), (200, 7800, 64),
+                                   (32, 11008, 4096), (5, 2064, 768), (20, 4112, 1024), (32, 13824, 1280)])
 def test_ffn_upgate_q8_0_many_rows(dev, rng, M, N, K):
+    """(the last four: at most 32 token rows against 128 and more groups of
+    16 row pairs: workgroups over the whole of K with 3, 1, 2 and 4 groups of
+    each matrix)"""
     up, _ = q8_weights(rng, N, K)
     gate, _ = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)

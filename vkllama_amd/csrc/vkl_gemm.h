@@ -55,6 +55,10 @@ size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
 bool gemm_wide_supported (const GemmArgs &a);
 int gemm_wide_launch (const GemmArgs &a, hipStream_t s);
 size_t gemm_wide_workspace_bytes (const GemmArgs &a); // fp32 scratch of its k-split (0: none)
+// At most 32 token rows against many rows of Q8_0 weights, each workgroup over
+// the whole of K: no partial sums (vkl_gemm_rowsfull.hip).
+bool gemm_rowsfull_supported (const GemmArgs &a);
+int gemm_rowsfull_launch (const GemmArgs &a, hipStream_t s);
 // The k-split forms' fp32 scratch of a stream (allocated on first use; null if
 // that fails), its size, and the kernel that adds `parts` partial results of
 // `rows` rows each in order and applies the epilogue.
