@@ -11,9 +11,10 @@
 // one block scale: sum = fma (block sum, d, sum), blocks in order.
 //
 // K is walked in steps of 256 (8 blocks).  A workgroup is alone on its compute
-// unit (it takes nearly all of the LDS), so the loads it keeps in flight are
-// all that hides the memory latency, about 3 us for the weights under load:
-// the step's int8 tiles (16 G x 256 bytes) and scales (16 G x 16 bytes) go
+// unit, so the loads it keeps in flight are all that hides the memory latency
+// (2.5-3 us for the weights under load; a compute unit gets about 45 KiB of
+// requests served per round trip, so rings deeper than that only queue): the
+// step's int8 tiles (16 G x 256 bytes) and scales (16 G x 16 bytes) go
 // straight into an LDS ring DW steps deep (global_load_lds_dwordx4, 1 KiB per
 // instruction: 8 rows x 128 bytes, stored XOR-swizzled by the choice of which
 // chunk a lane fetches, or 64 rows of scales), issued by NL waves that do

@@ -72,7 +72,6 @@ template <int V> struct WideInt
 // Accumulator register q of lane l is row 8 (q/4) + 4 (l/32) + q%4, column
 // l%32 of its 32 x 32 block.
 constexpr int kWideParkLd = 68; // floats per parked row: 16-byte aligned, rows 4 banks apart
-constexpr size_t kWideParkBytes = (size_t)WBM * 2 * kWideParkLd * 4; // 256 x 128 fp32 in rows of 64 (Q8_0 kernel)
 
 template <bool UPGATE, int TM>
 __device__ __forceinline__ void
@@ -607,8 +606,10 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
 // Which tile height and how many parts of the k range: the pair with the
 // lowest estimated time, from a model fitted to measurements on the 7B shapes
 // (microseconds: a round of 256-row tiles over the 256 compute units takes
-// about 0.95 per k-step + 8, one of 128-row tiles 0.55 per k-step + 6, Q8_0
-// weights 1.6 times that; a reduction launch 5 + its bytes at 2.5 TB/s).
+// about 0.95 per k-step + 8, one of 128-row tiles 0.55 per k-step + 6; with Q8_0
+// weights 1.35 and 0.90 per k-step, fitted on the 13B shapes at 3968 rows as
+// well: every tile converts its weight fragments anew, so short tiles gain
+// less there; a reduction launch 5 + its bytes at 2.5 TB/s).
 // Below kWideMinGroups workgroups the tile kernel of vkl_gemm_mfma.hip does
 // better.
 // (Below 128 token rows the two are about even: 64 x 4096 x 11008 takes 28 us
@@ -645,7 +646,6 @@ wide_plan (const GemmArgs &a)
           return none;
     }
   const int nk = a.K / WBK;
-  const double wq = a.wtype == 8 ? 1.6 : 1.0;
   const size_t ws_bytes = a.workspace ? a.workspace_bytes : gemm_stream_workspace_bytes ();
   double best_cost = 0;
   for (int bm = 128; bm <= WBM; bm *= 2)
@@ -661,7 +661,8 @@ wide_plan (const GemmArgs &a)
         const long groups = wide_tiles (a, bm) * ks;
         if (groups < (a.wtype == 8 ? kWideMinGroupsQ8 : kWideMinGroups))
           continue;
-        const double round = wq * (bm == WBM ? 0.95 * nk / ks + 8 : 0.55 * nk / ks + 6);
+        const double per_step = a.wtype == 8 ? (bm == WBM ? 1.35 : 0.90) : (bm == WBM ? 0.95 : 0.55);
+        const double round = per_step * nk / ks + (bm == WBM ? 8 : 6);
         const double reduce = ks > 1 ? 5 + (double)ks * a.M * a.N * sizeof (float) / 2.5e6 : 0;
         const double cost = (double)((groups + 255) / 256) * round + reduce;
         if (!best.bm || cost < best_cost)
