@@ -142,7 +142,9 @@ def test_matmul_q8_0_epilogue(dev, rng):
                                    (7, 200, 1376), (32, 129, 768), (5, 64, 256), (31, 300, 11008), (2, 1000, 5120),
                                    (270, 12300, 64), (600, 13000, 192), (1030, 6144, 448), (777, 8200, 320),
                                    (300, 8192, 64), (256, 4096, 2048),
-                                   (9, 6416, 1024), (32, 12288, 768), (3, 16368, 1280)])
+                                   (9, 6416, 1024), (32, 12288, 768), (3, 16368, 1280),
+                                   (64, 12288, 768), (33, 6416, 1024), (50, 16368, 1280),
+                                   (96, 12288, 768), (65, 6416, 1024), (80, 16368, 1280), (128, 12288, 768), (110, 6416, 1024)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
@@ -154,11 +156,13 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     one to seven k-steps, and its k range split in two; the last three: at
     most 32 token rows against 512 and more groups of 16 weight rows, K a
     multiple of 256: workgroups that run over the whole of K (2, 3 and 4
-    groups each, the last workgroup not full)."""
+    groups each, the last workgroup not full), and the same with 33 to 96
+    token rows (two and three blocks of 32 rows per workgroup) and with 97 to 128 (a
+    second launch for the rows past 96)."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)
-    if M * N * K <= 3e8 or K == 2048 or M <= 32:
+    if M * N * K <= 3e8 or K == 2048 or M <= 128:
         want = O.matmul_q8_0(x, raw, K)
         assert rel_err(got, want) < F16_REL_TOL
     exact = x.astype(np.float64) @ deq[:, :K].T
@@ -166,7 +170,7 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(40, 200, 512), (72, 200, 2048), (20, 200, 2048), (260, 12300, 64),
-                                   (260, 4096, 2048), (20, 8224, 1024)])
+                                   (260, 4096, 2048), (20, 8224, 1024), (40, 8224, 1024), (100, 8224, 1024)])
 def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     """scale / bias / activation, residual, widened copy and row strides: on
     the tile kernel without (K 512) and with the k-split, on the few-row
@@ -174,7 +178,7 @@ def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     256-row tiles (260 rows: 16-byte stores, and single ones where the output
     rows are not 16-byte aligned; with K 2048 the k range split in two, which
     finishes in the reduction kernel as well), and on the few-row kernel whose
-    workgroups run over the whole of K (20 rows x 8224)"""
+    workgroups run over the whole of K (20, 40 and, in two launches, 100 rows x 8224)"""
     raw, _ = q8_weights(rng, N, K, 0.01, 0.03)
     x = rng.standard_normal((M, K)).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
@@ -195,14 +199,25 @@ def test_gemm_q8_0_epilogue_and_strides(dev, rng, M, N, K):
     yw = f16(dy, (M, ys))
     assert rel_err(yw[:, :N], O.matmul_q8_0(x, raw, K)) < F16_REL_TOL
     assert not yw[:, N:].any()
+    # output rows that are not 16-byte aligned: single stores, the same values
+    ys2 = N + 4 if N % 8 == 0 else N + 3
+    dy2 = dev.alloc(M * ys2 * 2)
+    dy2.zero()
+    capi.check(L().vkl_matmul_q8_0(dx.ptr, dw.ptr, M, N, K, xs, ys2, 1.0, 0.0, 0, None, dy2.ptr, None, dev.stream))
+    yw2 = f16(dy2, (M, ys2))
+    assert np.array_equal(yw2[:, :N].view(np.uint16), yw[:, :N].view(np.uint16))
+    assert not yw2[:, N:].any()
 
 
 @pytest.mark.parametrize("M,N,K", [(40, 512, 512), (130, 96, 1376), (258, 4200, 64), (130, 5200, 64),
-                                   (32, 4096, 4096), (7, 4112, 768), (17, 5120, 1024), (2, 2736, 1024)])
+                                   (32, 4096, 4096), (7, 4112, 768), (17, 5120, 1024), (2, 2736, 1024),
+                                   (64, 4096, 4096), (45, 4112, 768), (96, 4096, 4096), (70, 4112, 768), (128, 4096, 4096),
+                                   (100, 4112, 768)])
 def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
     """(the last four: at most 32 token rows and 512 and more groups of 16
     weight rows over the three matrices: workgroups over the whole of K, 3, 4, 4
-    and 3 consecutive groups each, also across the end of a matrix)"""
+    and 3 consecutive groups each, also across the end of a matrix; then the same
+    form with 64, 45, 96 and 70 token rows, and 128 and 100 in two launches)"""
     ws = [q8_weights(rng, N, K)[0] for _ in range(3)]
     x = rng.standard_normal((M, K)).astype(np.float16)
     dx = dev.upload(x)
@@ -216,11 +231,14 @@ def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128), (200, 7800, 64),
-                                   (32, 11008, 4096), (5, 2064, 768), (20, 4112, 1024), (32, 13824, 1280)])
+                                   (32, 11008, 4096), (5, 2064, 768), (20, 4112, 1024), (32, 13824, 1280),
+                                   (64, 11008, 4096), (40, 2064, 768), (33, 4112, 1024), (48, 13824, 1280), (96, 11008, 4096),
+                                   (70, 2064, 768)])
 def test_ffn_upgate_q8_0_many_rows(dev, rng, M, N, K):
     """(the last four: at most 32 token rows against 128 and more groups of
     16 row pairs: workgroups over the whole of K with 3, 1, 2 and 4 groups of
-    each matrix)"""
+    each matrix; then 33 to 64 token rows on the same form with 3, 1 and 2
+    groups, on the tile kernel where it would take 4, and 96 and 70 rows in two launches)"""
     up, _ = q8_weights(rng, N, K)
     gate, _ = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)

@@ -55,7 +55,7 @@ size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
 bool gemm_wide_supported (const GemmArgs &a);
 int gemm_wide_launch (const GemmArgs &a, hipStream_t s);
 size_t gemm_wide_workspace_bytes (const GemmArgs &a); // fp32 scratch of its k-split (0: none)
-// At most 32 token rows against many rows of Q8_0 weights, each workgroup over
+// At most 96 token rows against many rows of Q8_0 weights, each workgroup over
 // the whole of K: no partial sums (vkl_gemm_rowsfull.hip).
 bool gemm_rowsfull_supported (const GemmArgs &a);
 int gemm_rowsfull_launch (const GemmArgs &a, hipStream_t s);

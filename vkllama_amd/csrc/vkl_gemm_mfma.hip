@@ -1297,11 +1297,12 @@ gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
 {
   if (!gemm_mfma_supported (a))
     return (int)hipErrorInvalidValue;
+  // up to 96 token rows against many weight rows: workgroups that run over the
+  // whole of K
+  if (gemm_rowsfull_supported (a))
+    return gemm_rowsfull_launch (a, s);
   if (few_rows_form (a))
     {
-      // many weight rows: workgroups that run over the whole of K
-      if (gemm_rowsfull_supported (a))
-        return gemm_rowsfull_launch (a, s);
       int err = 0;
       if (launch_rows64_q8 (a, s, err))
         return err;
@@ -1325,10 +1326,10 @@ gemm_mfma_workspace_bytes (const GemmArgs &a)
   if (!gemm_mfma_supported (a))
     return 0;
   const size_t nm = a.upgate ? 2 : a.nmat;
+  if (gemm_rowsfull_supported (a))
+    return 0;
   if (few_rows_form (a))
     {
-      if (gemm_rowsfull_supported (a))
-        return 0;
       // Q8_0: the whole-line form with slices of 512 if its sums fit, else
       // the form with slices of 1024
       if (a.wtype == 8)
