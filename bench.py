@@ -46,7 +46,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of a kernel from hardware counters (FETCH_SIZE +
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
-TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96185914}
+TRAFFIC = {("llama2-7b-q8_0", "upgate"): 96197201}
 TRAFFIC_SOURCE = "profiles/decode_phase_kernels_llama2-7b-q8_0_hbm_traffic.txt"
 
 
@@ -243,19 +243,32 @@ def main():
             per_phase[name] = {"launches_per_step": n // steps, "avg_us": round(ms * 1e3 / n, 3),
                                "us_per_step": round(ms * 1e3 / steps, 1),
                                "bytes_per_launch": m.phase_bytes(name, L_mid)}
+    if "attention" in per_phase and "wo" not in per_phase and phases.get("wo", (0, 0))[1] == 0:
+        # short contexts: the attention phase and the Wo projection are one launch
+        fused = per_phase.pop("attention")
+        fused["bytes_per_launch"] += m.phase_bytes("wo", L_mid)
+        per_phase = {"kqv": per_phase.pop("kqv"), "attention+wo": fused, **per_phase} if "kqv" in per_phase \
+            else {"attention+wo": fused, **per_phase}
     if per_phase:
         dom = max(per_phase, key=lambda k: per_phase[k]["us_per_step"])
         # the dominant kernel again, launched back to back (every layer's weights
         # in turn) between ONE event pair: its duration without a pair's own cost
         rounds = max(2, steps // 8)
-        m.phase_replay(dom, L_mid - 1, 1)
-        dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
+        if dom == "attention+wo":
+            # (no stand-alone replay of the fused launch: its average between event pairs)
+            dom_us, dom_n = per_phase[dom]["avg_us"], phases["attention"][1]
+        else:
+            m.phase_replay(dom, L_mid - 1, 1)
+            dom_us, dom_n = m.phase_replay(dom, L_mid - 1, rounds)
         dom_bytes = per_phase[dom]["bytes_per_launch"]
         # the kernel's name as a profiler prints it: phase number, weight type,
         # 4096-value chunks of the staged activation row
-        phase_no = {"kqv": 0, "attention": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5}[dom]
+        phase_no = {"kqv": 0, "attention": 1, "attention+wo": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5}[dom]
         kstage = cfg["ffn"] if dom == "down" else cfg["dim"]
-        if dom == "attention":
+        if dom == "attention+wo":
+            dom_kernel = "decode_attn_wo_kernel<%d, %d> (attention + Wo)" % (8 if cfg["wtype"] == 8 else 1,
+                                                                            min(4, (cfg["dim"] + 4095) // 4096))
+        elif dom == "attention":
             dom_kernel = "decode_phase_kernel<1, %d> (attention)" % (8 if cfg["wtype"] == 8 else 1)
         else:
             # last argument: weights of a step beyond what the caches hold are

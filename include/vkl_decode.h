@@ -85,6 +85,16 @@ int vkl_decode_status (const vkl_decode_model *m, void *stream);
  * captured with. */
 int vkl_decode_set_attn_split (int min_len);
 
+/* Whether mode 0 runs the attention phase (one workgroup per head, i.e. below
+ * the split length above) and the Wo projection in one launch: the projection's
+ * workgroups request their weights while the heads are computed and start
+ * once every head has counted itself in (a bounded wait; one that gives up is
+ * reported by vkl_decode_status).  Results are bit for bit those of the two
+ * launches.  On by default; process-wide; a measuring and testing aid without
+ * counterpart in the reference.  Graphs captured by vkl_decode_loop hold the
+ * form they were captured with. */
+int vkl_decode_set_fuse_attn_wo (int on);
+
 /* n_steps greedy tokens without a host round trip per token: step i reads
  * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
  * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the

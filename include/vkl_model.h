@@ -74,7 +74,8 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
 /* options: fused one-token decode on/off, decode launch mode (0 = one launch
  * per phase, 1 = one persistent launch per token), replay of the greedy loop
  * from a HIP graph on/off, the context length from which attention is split
- * over several workgroups per head, the reference's last-block RoPE position
+ * over several workgroups per head, attention and the Wo projection in one
+ * launch on/off ("fuse_attn_wo"), the reference's last-block RoPE position
  * quirk */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);
 /* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */

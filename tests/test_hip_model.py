@@ -331,6 +331,36 @@ def test_graph_replayed_loop_equals_stepwise_and_oracle(n_prompt, n_gen):
     m.close()
 
 
+@pytest.mark.parametrize("cfg", [TINY, dict(dim=5120, n_layers=2, n_heads=40, ffn=1376, vocab=1024, maxlen=256, eps=1e-5,
+                                              wtype=8),
+                                 dict(dim=4096, n_layers=2, n_heads=32, ffn=1376, vocab=1024, maxlen=256, eps=1e-5,
+                                      wtype=1)])
+def test_attention_and_wo_in_one_launch_equals_two_launches(cfg):
+    """Below the split length the decode step runs the attention phase and the
+    Wo projection in one launch (option "fuse_attn_wo", on by default): the
+    projection's workgroups wait inside the launch for the heads.  Ids and
+    logits must equal those of the two separate launches bit for bit, replayed
+    from a graph and launched step by step (the two-launch form is what the
+    other tests of this file hold against the oracle)."""
+    w = M.synth_weights(cfg, seed=5)
+    prompt = np.random.default_rng(5).integers(3, cfg["vocab"], 9).astype(np.uint32)
+    m = M.Llama2(cfg, w)
+    runs = {}
+    for fuse in (1, 0):
+        m.set_option("fuse_attn_wo", fuse)
+        for graph in (1, 0):
+            m.set_option("decode_graph", graph)
+            ids, _, _ = m.generate_greedy(prompt, 48)
+            logits = m.forward([int(ids[-1])], 9 + 47)
+            runs[(fuse, graph)] = (list(ids), logits.copy())
+    m.set_option("fuse_attn_wo", 1)
+    m.close()
+    ref_ids, ref_logits = runs[(0, 0)]
+    for key, (ids, logits) in runs.items():
+        assert ids == ref_ids, key
+        assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
+
+
 @pytest.mark.parametrize("fused", [0, 1])
 def test_sampled_generation_on_the_device(small, fused):
     """generate_sampled: k = 1 is the greedy sequence; a seed reproduces a top-k

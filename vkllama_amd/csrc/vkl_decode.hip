@@ -33,6 +33,22 @@ namespace
 {
 // contexts from this length on run the split form of the attention phase
 int g_attn_split_min = kAttnSplitMinLen;
+int g_fuse_attn_wo = 1; // short contexts: attention and the Wo projection in one launch
+// words of the sync area for the fused attention + Wo launch: a counter of the
+// heads whose attention output is in memory, and eight flags (one per
+// workgroup index mod 8, i.e. per XCD) that the last head sets and the
+// projection's workgroups poll (polling the counter itself from every
+// workgroup held up the heads' atomics); all zeroed by the layer's K/Q/V phase
+constexpr int kSyncAttnDone = 800;
+constexpr int kSyncAttnFlag = 816; // + 16 * slot
+constexpr int kFuseSpinLimit = 1 << 13; // some 10 ms; a head takes microseconds
+
+__device__ __forceinline__ void
+reset_attn_done (const Params &p, int wg)
+{
+  if (wg == 0 && threadIdx.x < 9)
+    st_coherent_u32 (p.s.sync + (threadIdx.x == 8 ? kSyncAttnDone : kSyncAttnFlag + 16 * (int)threadIdx.x), 0u);
+}
 
 // The activation row (K fp16 values, K a multiple of 32, K <= 16384) is
 // fetched into registers first: thread t holds the 8-element chunks t,
@@ -743,6 +759,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         VKL_TR (2);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
         GV::run (ps, A, B, xl, e, red);
+        reset_attn_done (p, wg);
         break;
       }
     case PH_ATTN:
@@ -872,6 +889,7 @@ run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
         stage_row<true, XCH> (x, dim, xl, nw, m.eps, red, VKL_TRP);
         VKL_TR (2);
         e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
+        reset_attn_done (p, wg);
         break;
       }
     case PH_WO:
@@ -943,6 +961,85 @@ decode_phase_direct_kernel (const Params p, const vkl_layer_weights lw, int laye
 {
   extern __shared__ __align__ (16) uint8_t lds[];
   run_phase_direct<PHASE, WT, XCH, NT> (p, lw, layer, (int)blockIdx.x, G, lds);
+}
+
+// ---------------------------------------------------------------------------
+// short contexts: attention and the Wo projection in one launch
+// ---------------------------------------------------------------------------
+// The attention phase moves little data (a head's cache rows) but takes
+// 4-6 us of dependent steps on n_heads compute units, and the Wo projection
+// after it spends half of its 5 us waiting for its first weights.  In one
+// launch the first n_heads workgroups compute a head each while the G others
+// already have their Wo weights on the way; those then wait until every head
+// has counted itself in (the last one sets the flags they poll; the K/Q/V
+// phase of the layer has zeroed counter and flags), read the attention row
+// and multiply.  The row can be read with ordinary loads: no cache of this
+// launch has seen its lines before the wait (caches are invalidated between
+// launches), and the heads' stores went through to memory before they counted.  The head workgroups have the lowest indices, so
+// they are resident before any waiter; the wait is bounded all the same, and
+// one that gives up sets the error word that vkl_decode_status reports.
+// Results are those of the two separate launches bit for bit.
+template <int WT, int XCH>
+__global__ __launch_bounds__ (kDecThreads) void
+decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, int G)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  const vkl_decode_model &m = p.m;
+  const int nh = m.n_heads, dim = m.dim;
+  uint32_t *done = p.s.sync + kSyncAttnDone;
+  if ((int)blockIdx.x < nh)
+    {
+      if (m.head_dim == 128)
+        attention_head<128, true> (p, lw, (int)blockIdx.x, lds, nullptr);
+      else
+        attention_head<64, true> (p, lw, (int)blockIdx.x, lds, nullptr);
+      // count in once the head's output is in memory
+      __builtin_amdgcn_s_waitcnt (0x0f70);
+      __syncthreads ();
+      if (threadIdx.x < 64)
+        {
+          uint32_t old = 0;
+          if (threadIdx.x == 0)
+            old = __hip_atomic_fetch_add (done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
+          if (old + 1u == (uint32_t)nh && threadIdx.x < 8)
+            st_coherent_u32 (p.s.sync + kSyncAttnFlag + 16 * (int)threadIdx.x, 1u);
+        }
+      return;
+    }
+  const int wg = (int)blockIdx.x - nh;
+  typedef Gemv<WT, false, 1> GV;
+  uint16_t *xl = (uint16_t *)lds;
+  float *red = (float *)(lds + (size_t)dim * 2);
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
+  const QMat w = wmat<WT> (lw.wo, dim, dim);
+  // (both items of a wave: with one or two rows per wave that is all of them)
+  GV::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true);
+  if (threadIdx.x < 64)
+    {
+      const uint32_t *flag = p.s.sync + kSyncAttnFlag + 16 * ((int)blockIdx.x & 7);
+      bool ok = false;
+      for (int spin = 0; spin < kFuseSpinLimit; ++spin)
+        {
+          if (ld_coherent_u32 (flag) != 0u)
+            {
+              ok = true;
+              break;
+            }
+          __builtin_amdgcn_s_sleep (4);
+        }
+      if (!ok && threadIdx.x == 0)
+        st_coherent_u32 (p.s.sync + 1, 1u);
+    }
+  __syncthreads ();
+  load_row<XCH> (p.s.att, dim, x);
+  stage_row<false, XCH> (x, dim, xl, nw, 0.f, red, nullptr);
+  e.y[0] = p.s.x, e.residual = p.s.x;
+  GV::run (ps, A, B, xl, e, red);
 }
 
 // ---------------------------------------------------------------------------
@@ -1378,6 +1475,49 @@ launch_phase (const Params &p, const vkl_layer_weights &lw, int layer,
   return timer_mark (PHASE, true, s);
 }
 
+// attention of one head per workgroup + the Wo projection on G - n_heads more
+template <int WT, int XCH>
+int
+launch_attn_wo_xch (const Params &p, const vkl_layer_weights &lw, int layer, int G, size_t lds,
+                    hipStream_t s)
+{
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute ((const void *)decode_attn_wo_kernel<WT, XCH>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  decode_attn_wo_kernel<WT, XCH>
+      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G - p.m.n_heads);
+  return 0;
+}
+
+bool
+attn_wo_fused (const Params &p, const vkl_decode_model *m, int G)
+{
+  return g_fuse_attn_wo && (int)p.pos + 1 < g_attn_split_min 
+         && G >= 4 * m->n_heads && m->dim <= 8192 && (m->dim % 8) == 0;
+}
+
+int
+launch_attn_wo (const Params &p, const vkl_layer_weights &lw, int layer, int G, size_t lds,
+                hipStream_t s)
+{
+  if (int e = timer_mark (PH_ATTN, false, s))
+    return e;
+  int e;
+  if (p.m.dim <= 4096)
+    e = p.m.wtype == 8 ? launch_attn_wo_xch<8, 1> (p, lw, layer, G, lds, s)
+                       : launch_attn_wo_xch<1, 1> (p, lw, layer, G, lds, s);
+  else
+    e = p.m.wtype == 8 ? launch_attn_wo_xch<8, 2> (p, lw, layer, G, lds, s)
+                       : launch_attn_wo_xch<1, 2> (p, lw, layer, G, lds, s);
+  if (e)
+    return e;
+  return timer_mark (PH_ATTN, true, s);
+}
+
 // attention of one layer: one workgroup per head, or the split form for long
 // contexts
 int
@@ -1459,10 +1599,18 @@ launch_step (const Params &p, const vkl_decode_model *m, int n_cu, int G,
       const vkl_layer_weights &lw = m->layers_h[l];
       if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
         return e;
-      if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
-        return e;
-      if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
-        return e;
+      if (attn_wo_fused (p, m, G))
+        {
+          if (int e = launch_attn_wo (p, lw, l, G, lds, s))
+            return e;
+        }
+      else
+        {
+          if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
+            return e;
+          if (int e = launch_phase<PH_WO> (p, lw, l, G, G, lds, s))
+            return e;
+        }
       if (int e = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s))
         return e;
       if (int e = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s))
@@ -1583,6 +1731,13 @@ vkl_decode_set_attn_split (int min_len)
 }
 
 extern "C" int
+vkl_decode_set_fuse_attn_wo (int on)
+{
+  g_fuse_attn_wo = on ? 1 : 0;
+  return 0;
+}
+
+extern "C" int
 vkl_decode_status (const vkl_decode_model *m, void *stream)
 {
   VKL_CHECK_ARG (m != nullptr && m->scratch != nullptr);
@@ -1614,6 +1769,7 @@ struct StepGraph
   const void *scratch = nullptr, *ids = nullptr, *logits = nullptr;
   uint64_t model_hash = 0; // over every pointer and dimension the launches hold
   int long_ctx = 0;
+  int fused = 0; // the attention + Wo launch was enabled at capture
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   uint64_t used = 0;
@@ -1702,7 +1858,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
         {
           if (c.exec && c.scratch == m->scratch && c.ids == ids
               && c.logits == p.logits32 && c.model_hash == mh
-              && c.long_ctx == long_ctx)
+              && c.long_ctx == long_ctx && c.fused == g_fuse_attn_wo)
             g = &c;
           if (c.used < lru->used)
             lru = &c;
@@ -1737,7 +1893,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
               break;
             }
           g->scratch = m->scratch, g->ids = ids, g->logits = p.logits32;
-          g->model_hash = mh, g->long_ctx = long_ctx;
+          g->model_hash = mh, g->long_ctx = long_ctx, g->fused = g_fuse_attn_wo;
         }
       g->used = ++g_graph_clock;
       for (; done < upto && !err; ++done)

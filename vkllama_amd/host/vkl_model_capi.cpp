@@ -227,6 +227,8 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_decode_graph (value != 0);
   else if (n == "phase_timing")
     vkl_decode_phase_timing (value);
+  else if (n == "fuse_attn_wo")
+    vkl_decode_set_fuse_attn_wo (value);
   else if (n == "attn_split_min")
     {
       if (vkl_decode_set_attn_split (value))

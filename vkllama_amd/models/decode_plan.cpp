@@ -178,11 +178,12 @@ DecodePlan::loop (uint32_t *ids, size_t pos0, size_t n_steps)
 absl::Status
 DecodePlan::check ()
 {
-  if (!usable_ || mode_ != 1)
+  // (mode 0 waits between workgroups too, in its fused attention + Wo launch)
+  if (!usable_)
     return absl::OkStatus ();
   if (int e = vkl_decode_status (&desc_, gpu_->stream ()))
     return absl::InternalError (absl::StrFormat (
-        "persistent decode step: a wait between workgroups gave up (%s); the GPU must not be "
+        "decode step: a wait between workgroups gave up (%s); the GPU must not be "
         "shared while such a launch runs",
         vkl_error_string (e)));
   return absl::OkStatus ();
