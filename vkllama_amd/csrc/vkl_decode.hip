@@ -39,15 +39,16 @@ int g_fuse_attn_wo = 1; // short contexts: attention and the Wo projection in on
 // workgroup index mod 8, i.e. per XCD) that the last head sets and the
 // projection's workgroups poll (polling the counter itself from every
 // workgroup held up the heads' atomics); all zeroed by the layer's K/Q/V phase
-constexpr int kSyncAttnDone = 800;
-constexpr int kSyncAttnFlag = 816; // + 16 * slot
+// (each on a cache line of its own, clear of the words the persistent mode uses)
+constexpr int kSyncAttnDone = 32;
+constexpr int kSyncAttnFlag = 768; // + 32 * slot
 constexpr int kFuseSpinLimit = 1 << 13; // some 10 ms; a head takes microseconds
 
 __device__ __forceinline__ void
 reset_attn_done (const Params &p, int wg)
 {
   if (wg == 0 && threadIdx.x < 9)
-    st_coherent_u32 (p.s.sync + (threadIdx.x == 8 ? kSyncAttnDone : kSyncAttnFlag + 16 * (int)threadIdx.x), 0u);
+    st_coherent_u32 (p.s.sync + (threadIdx.x == 8 ? kSyncAttnDone : kSyncAttnFlag + 32 * (int)threadIdx.x), 0u);
 }
 
 // The activation row (K fp16 values, K a multiple of 32, K <= 16384) is
@@ -1003,7 +1004,7 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
             old = __hip_atomic_fetch_add (done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
           if (old + 1u == (uint32_t)nh && threadIdx.x < 8)
-            st_coherent_u32 (p.s.sync + kSyncAttnFlag + 16 * (int)threadIdx.x, 1u);
+            st_coherent_u32 (p.s.sync + kSyncAttnFlag + 32 * (int)threadIdx.x, 1u);
         }
       return;
     }
@@ -1021,7 +1022,7 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
   GV::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true);
   if (threadIdx.x < 64)
     {
-      const uint32_t *flag = p.s.sync + kSyncAttnFlag + 16 * ((int)blockIdx.x & 7);
+      const uint32_t *flag = p.s.sync + kSyncAttnFlag + 32 * ((int)blockIdx.x & 7);
       bool ok = false;
       for (int spin = 0; spin < kFuseSpinLimit; ++spin)
         {
