@@ -95,6 +95,14 @@ int vkl_decode_set_attn_split (int min_len);
  * form they were captured with. */
 int vkl_decode_set_fuse_attn_wo (int on);
 
+/* A testing aid without counterpart in the reference: after how many polls a
+ * wait inside the fused attention + Wo launch gives up (0 restores the
+ * default, some 10 ms), and whether the head workgroups leave the flags unset,
+ * which makes every such wait give up: the launches still end, the results
+ * are invalid and vkl_decode_status reports it.  Process-wide; drops the
+ * graphs cached by vkl_decode_loop, so no decode work may be in flight. */
+int vkl_decode_set_wait_limit (int polls, int silent_heads);
+
 /* n_steps greedy tokens without a host round trip per token: step i reads
  * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
  * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the

@@ -361,6 +361,35 @@ def test_attention_and_wo_in_one_launch_equals_two_launches(cfg):
         assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
 
 
+def test_wait_inside_the_fused_launch_is_bounded_and_reported():
+    """The projection's workgroups of the fused attention + Wo launch wait for the
+    heads with a bounded number of polls.  With the heads kept silent from the
+    host (option "fused_wait_test": the flags stay unset, 4 polls) every wait
+    gives up: all launches still end, and the status word turns the generation
+    and the logits read-back into errors instead of wrong tokens.  Afterwards
+    the same model generates the same ids as before."""
+    cfg = TINY
+    w = M.synth_weights(cfg, seed=9)
+    prompt = np.random.default_rng(9).integers(3, cfg["vocab"], 6).astype(np.uint32)
+    m = M.Llama2(cfg, w)
+    want, _, _ = m.generate_greedy(prompt, 24)
+    m.set_option("fused_wait_test", 4)
+    try:
+        for graph in (0, 1):
+            m.set_option("decode_graph", graph)
+            with pytest.raises(capi.VklError):
+                m.generate_greedy(prompt, 24)
+        with pytest.raises(capi.VklError):
+            m.forward([int(want[0])], 6)
+    finally:
+        m.set_option("fused_wait_test", 0)
+    for graph in (1, 0):
+        m.set_option("decode_graph", graph)
+        ids, _, _ = m.generate_greedy(prompt, 24)
+        assert list(ids) == list(want)
+    m.close()
+
+
 @pytest.mark.parametrize("fused", [0, 1])
 def test_sampled_generation_on_the_device(small, fused):
     """generate_sampled: k = 1 is the greedy sequence; a seed reproduces a top-k

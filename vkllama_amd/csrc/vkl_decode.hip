@@ -34,6 +34,7 @@ namespace
 // contexts from this length on run the split form of the attention phase
 int g_attn_split_min = kAttnSplitMinLen;
 int g_fuse_attn_wo = 1; // short contexts: attention and the Wo projection in one launch
+int g_fuse_wait = 0;    // polls before a wait inside that launch gives up (0: kFuseSpinLimit), bit 30: the heads stay silent (tests)
 // words of the sync area for the fused attention + Wo launch: a counter of the
 // heads whose attention output is in memory, and eight flags (one per
 // workgroup index mod 8, i.e. per XCD) that the last head sets and the
@@ -982,7 +983,7 @@ decode_phase_direct_kernel (const Params p, const vkl_layer_weights lw, int laye
 // Results are those of the two separate launches bit for bit.
 template <int WT, int XCH>
 __global__ __launch_bounds__ (kDecThreads) void
-decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, int G)
+decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, int G, int wait)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
   const vkl_decode_model &m = p.m;
@@ -1003,7 +1004,8 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
           if (threadIdx.x == 0)
             old = __hip_atomic_fetch_add (done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
-          if (old + 1u == (uint32_t)nh && threadIdx.x < 8)
+          // (wait bit 30: a test of the bounded wait; the flags then stay unset)
+          if (old + 1u == (uint32_t)nh && threadIdx.x < 8 && !(wait & (1 << 30)))
             st_coherent_u32 (p.s.sync + kSyncAttnFlag + 32 * (int)threadIdx.x, 1u);
         }
       return;
@@ -1024,7 +1026,8 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
     {
       const uint32_t *flag = p.s.sync + kSyncAttnFlag + 32 * ((int)blockIdx.x & 7);
       bool ok = false;
-      for (int spin = 0; spin < kFuseSpinLimit; ++spin)
+      const int limit = (wait & 0xffffff) ? (wait & 0xffffff) : kFuseSpinLimit;
+      for (int spin = 0; spin < limit; ++spin)
         {
           if (ld_coherent_u32 (flag) != 0u)
             {
@@ -1490,7 +1493,7 @@ launch_attn_wo_xch (const Params &p, const vkl_layer_weights &lw, int layer, int
       lds_set = lds;
     }
   decode_attn_wo_kernel<WT, XCH>
-      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G - p.m.n_heads);
+      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G - p.m.n_heads, g_fuse_wait);
   return 0;
 }
 
@@ -2082,4 +2085,15 @@ vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream)
   argmax_f32_kernel<<<dim3 (1), dim3 (1024), 0, (hipStream_t)stream>>> (x, n,
                                                                         out);
   return vkl_launch_status ();
+}
+
+extern "C" int
+vkl_decode_set_wait_limit (int polls, int silent_heads)
+{
+  VKL_CHECK_ARG (polls >= 0 && polls < (1 << 24));
+  g_fuse_wait = polls | (silent_heads ? 1 << 30 : 0);
+  // captured graphs hold the old value
+  for (StepGraph &g : g_graphs)
+    drop_graph (g);
+  return 0;
 }

@@ -229,6 +229,13 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     vkl_decode_phase_timing (value);
   else if (n == "fuse_attn_wo")
     vkl_decode_set_fuse_attn_wo (value);
+  else if (n == "fused_wait_test")
+    {
+      // value > 0: waits of the fused launch give up after `value` polls and
+      // the heads never signal; 0: back to normal
+      if (vkl_decode_set_wait_limit (value > 0 ? value : 0, value > 0))
+        return fail (m, absl::InvalidArgumentError ("fused_wait_test out of range"));
+    }
   else if (n == "attn_split_min")
     {
       if (vkl_decode_set_attn_split (value))
