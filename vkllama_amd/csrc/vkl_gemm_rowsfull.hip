@@ -352,6 +352,7 @@ gemm_rowsfull_q8_kernel (const GemmArgs a, int groups, int gpm, int vec)
 // G, KS, NL, DX, DW per number of groups.  Deeper rings do not pay: past some
 // 45 KiB of requests in flight per compute unit the memory system only queues
 // them (7B K/Q/V at 32 rows: 16.9 us with DX 3 / DW 4, 18.2 us with 4 / 7).
+#define RF_CFG1 1, 8, 1, 3, 6, 1
 #define RF_CFG2 2, 8, 2, 3, 5, 1
 #define RF_CFG3 3, 8, 2, 3, 4, 1
 #define RF_CFG4 4, 8, 2, 3, 4, 1
@@ -395,7 +396,9 @@ rowsfull_plan (const GemmArgs &a)
     }
   const int total = gpm * a.nmat;
   const int gq = (total + 255) / 256;
-  return gq > 4 || gq < 2 || total < 128 * gq ? 0 : gq;
+  if (gq == 1)
+    return a.M <= 32 && total >= 200 && a.K <= 4096 ? 1 : 0;
+  return gq > 4 || total < 128 * gq ? 0 : gq;
 }
 
 template <int G, int KS, int NL, int DX, int DW, int TB, bool UPGATE>
@@ -472,6 +475,7 @@ rowsfull_launch_rows (const GemmArgs &a, int g, int vec, hipStream_t s)
       }
   switch (g)
     {
+    case 1: return rowsfull_run<RF_CFG1, false> (a, total, gpm, vec, s);
     case 2: return rowsfull_run<RF_CFG2, false> (a, total, gpm, vec, s);
     case 3: return rowsfull_run<RF_CFG3, false> (a, total, gpm, vec, s);
     case 4: return rowsfull_run<RF_CFG4, false> (a, total, gpm, vec, s);
