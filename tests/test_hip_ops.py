@@ -145,7 +145,7 @@ def test_matmul_q8_0_epilogue(dev, rng):
                                    (9, 6416, 1024), (32, 12288, 768), (3, 16368, 1280),
                                    (64, 12288, 768), (33, 6416, 1024), (50, 16368, 1280),
                                    (96, 12288, 768), (65, 6416, 1024), (80, 16368, 1280), (128, 12288, 768), (110, 6416, 1024),
-                                   (24, 4000, 768)])
+                                   (24, 4000, 768), (64, 4000, 768), (90, 4000, 1024)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
@@ -159,8 +159,8 @@ def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     multiple of 256: workgroups that run over the whole of K (2, 3 and 4
     groups each, the last workgroup not full), and the same with 33 to 96
     token rows (two and three blocks of 32 rows per workgroup) and with 97 to 128 (a
-    second launch for the rows past 96); the last: one group per workgroup (the Wo
-    product of a short prompt)."""
+    second launch for the rows past 96); the last three: one group per workgroup
+    (the Wo product of a short prompt) with one, two and three blocks of 32 rows."""
     raw, deq = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)
     got = _run_matmul_q8(dev, x, raw, N, K)

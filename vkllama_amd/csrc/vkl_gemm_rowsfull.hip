@@ -359,11 +359,13 @@ gemm_rowsfull_q8_kernel (const GemmArgs a, int groups, int gpm, int vec)
 #define RF_CFG6 6, 8, 4, 3, 3, 1
 #define RF_CFG8 8, 8, 4, 3, 3, 1
 // 33 to 64 token rows: the x tile of a step is 32 KiB
+#define RF_CFG1W 1, 8, 1, 3, 6, 2
 #define RF_CFG2W 2, 8, 2, 3, 5, 2
 #define RF_CFG3W 3, 8, 2, 3, 4, 2
 #define RF_CFG4W 4, 8, 2, 3, 3, 2
 #define RF_CFG6W 6, 8, 4, 2, 3, 2
 // 65 to 96 token rows (single matrices and K/Q/V only): 48 KiB
+#define RF_CFG1X 1, 8, 1, 2, 6, 3
 #define RF_CFG2X 2, 8, 2, 2, 5, 3
 #define RF_CFG3X 3, 8, 2, 2, 4, 3
 #define RF_CFG4X 4, 8, 2, 2, 3, 3
@@ -397,7 +399,7 @@ rowsfull_plan (const GemmArgs &a)
   const int total = gpm * a.nmat;
   const int gq = (total + 255) / 256;
   if (gq == 1)
-    return a.M <= 32 && total >= 200 && a.K <= 4096 ? 1 : 0;
+    return a.M <= kRowsFullPlain && total >= 200 && a.K <= 4096 ? 1 : 0;
   return gq > 4 || total < 128 * gq ? 0 : gq;
 }
 
@@ -462,6 +464,7 @@ rowsfull_launch_rows (const GemmArgs &a, int g, int vec, hipStream_t s)
   if (a.M > 64)
     switch (g)
       {
+      case 1: return rowsfull_run<RF_CFG1X, false> (a, total, gpm, vec, s);
       case 2: return rowsfull_run<RF_CFG2X, false> (a, total, gpm, vec, s);
       case 3: return rowsfull_run<RF_CFG3X, false> (a, total, gpm, vec, s);
       case 4: return rowsfull_run<RF_CFG4X, false> (a, total, gpm, vec, s);
@@ -469,6 +472,7 @@ rowsfull_launch_rows (const GemmArgs &a, int g, int vec, hipStream_t s)
   if (a.M > 32)
     switch (g)
       {
+      case 1: return rowsfull_run<RF_CFG1W, false> (a, total, gpm, vec, s);
       case 2: return rowsfull_run<RF_CFG2W, false> (a, total, gpm, vec, s);
       case 3: return rowsfull_run<RF_CFG3W, false> (a, total, gpm, vec, s);
       case 4: return rowsfull_run<RF_CFG4W, false> (a, total, gpm, vec, s);
