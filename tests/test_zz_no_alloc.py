@@ -38,8 +38,9 @@ def _both(dev, rng, M, N, K, residual=False):
 
 
 def test_noalloc_equals_the_allocating_entry_point_on_two_calls_in_a_row(dev, rng):
-    # few-row kernel: 20 rows against a 4096 x 4096 matrix (4.2 MB of partial sums) ...
-    a, b = _both(dev, rng, 20, 4096, 4096)
+    # few-row kernel with K slices: 20 rows against a 2048 x 4096 matrix (2.1 MB of partial sums; with 4096 rows
+    # and more the workgroups run over the whole of K and need no scratch) ...
+    a, b = _both(dev, rng, 20, 2048, 4096)
     assert np.isfinite(a.astype(np.float32)).all() and a.any()
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
     # ... then a smaller problem over the same scratch, with the residual epilogue
@@ -48,8 +49,10 @@ def test_noalloc_equals_the_allocating_entry_point_on_two_calls_in_a_row(dev, rn
     # the tile kernel with its k range split (100 rows: 3.3 MB of partial tiles)
     a, b = _both(dev, rng, 100, 4096, 1024)
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
-    # one row needs no scratch
+    # one row needs no scratch, nor do few rows against many weight rows
     a, b = _both(dev, rng, 1, 4096, 4096)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    a, b = _both(dev, rng, 20, 4096, 4096, residual=True)
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
 
 
