@@ -235,12 +235,13 @@ def test_kqv_q8_0_many_rows(dev, rng, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (128, 160, 4096), (200, 64, 512), (300, 6200, 128), (200, 7800, 64),
                                    (32, 11008, 4096), (5, 2064, 768), (20, 4112, 1024), (32, 13824, 1280),
                                    (64, 11008, 4096), (40, 2064, 768), (33, 4112, 1024), (48, 13824, 1280), (96, 11008, 4096),
-                                   (70, 2064, 768)])
+                                   (70, 2064, 768), (100, 8256, 128), (66, 13824, 256), (127, 11008, 512)])
 def test_ffn_upgate_q8_0_many_rows(dev, rng, M, N, K):
     """(the last four: at most 32 token rows against 128 and more groups of
     16 row pairs: workgroups over the whole of K with 3, 1, 2 and 4 groups of
     each matrix; then 33 to 64 token rows on the same form with 3, 1 and 2
-    groups, on the tile kernel where it would take 4, and 96 and 70 rows in two launches)"""
+    groups, on the tile kernel where it would take 4, and 96 and 70 rows in two launches;
+    the last three: 65 to 127 rows in one partly empty row of 128-row tiles of the many-row kernel)"""
     up, _ = q8_weights(rng, N, K)
     gate, _ = q8_weights(rng, N, K)
     x = rng.standard_normal((M, K)).astype(np.float16)

@@ -615,6 +615,12 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
 // (Below 128 token rows the two are about even: 64 x 4096 x 11008 takes 28 us
 // there and 34 us here, 100 x 4096 x 4096 21 and 16.)
 constexpr int kWideMinRows = 128;
+// the fused up/gate pair (three times the weights of a square product) already
+// from 65 rows on (where the tile kernel needs a second row of 64-row tiles), in
+// one partly empty row of 128-row tiles: 13B 108 -> 92 us at 80 rows, 7B
+// 84 -> 66 us at 127; below (13B at 64 rows: 83 against 88 us), and for the other
+// products (down at 7B: 39 -> 42 us at 96 rows), the tile kernel does better
+constexpr int kWideMinRowsUpgate = 65;
 constexpr int kWideMinGroups = 88, kWideMinGroupsQ8 = 128;
 
 struct WidePlan
@@ -634,7 +640,8 @@ WidePlan
 wide_plan (const GemmArgs &a)
 {
   WidePlan none = { 0, 1 }, best = none;
-  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < kWideMinRows)
+  const int min_rows = a.upgate && a.wtype == 8 ? kWideMinRowsUpgate : kWideMinRows;
+  if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < min_rows)
     return none;
   if (a.wtype == 8)
     {
@@ -651,7 +658,8 @@ wide_plan (const GemmArgs &a)
   for (int bm = 128; bm <= WBM; bm *= 2)
     for (int ks = 1; ks <= 4; ks *= 2)
       {
-        if (a.M < bm)
+        // (a single row of 128-row tiles may be partly empty)
+        if (a.M < bm && !(bm == 128 && a.M >= min_rows))
           continue;
         // parts only for one matrix with the plain epilogue, of at least 16
         // k-steps each, and as far as the scratch holds them
