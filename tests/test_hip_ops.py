@@ -145,7 +145,7 @@ def test_matmul_q8_0_epilogue(dev, rng):
                                    (9, 6416, 1024), (32, 12288, 768), (3, 16368, 1280),
                                    (64, 12288, 768), (33, 6416, 1024), (50, 16368, 1280),
                                    (96, 12288, 768), (65, 6416, 1024), (80, 16368, 1280), (128, 12288, 768), (110, 6416, 1024),
-                                   (24, 4000, 768), (64, 4000, 768), (90, 4000, 1024)])
+                                   (24, 4000, 768), (64, 4000, 768), (90, 4000, 1024), (110, 16400, 64)])
 def test_gemm_q8_0_many_rows(dev, rng, M, N, K):
     """Several token rows run on the matrix cores (quants as exact fp16
     integers, block sums by MFMA, block scale in fp32); the shapes cover the
@@ -291,12 +291,14 @@ def test_matmul_f16_tb(dev, rng, C, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(16, 130, 512), (100, 200, 1376), (300, 96, 4096), (64, 1376, 512),
                                    (512, 12800, 64), (600, 13000, 96), (600, 13000, 128), (777, 8200, 320),
-                                   (256, 24576, 192), (1030, 6144, 448), (300, 6144, 128), (130, 12000, 192), (200, 4096, 2048)])
+                                   (256, 24576, 192), (1030, 6144, 448), (300, 6144, 128), (130, 12000, 192), (200, 4096, 2048),
+                                   (100, 11392, 128), (66, 12000, 192)])
 def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     """FP16 weights, many token rows: the matrix-core paths (from about two
     hundred 256 x 128 output tiles on, or half as many 128 x 128 ones, with K a
     multiple of 64, the form that loads its tiles straight into LDS; ragged M
-    and N included; the last shape with its k range split in two)."""
+    and N included; (200, 4096, 2048) with its k range split in two; the last
+    two: 65 to 127 rows in one partly empty row of 128-row tiles)."""
     a = rng.standard_normal((1, M, K)).astype(np.float16)
     b = (rng.standard_normal((1, N, K)) * 0.05).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
@@ -318,7 +320,8 @@ def test_matmul_f16_tb_many_rows(dev, rng, M, N, K):
     assert np.array_equal(d32.read(np.float32, (M, N)), got.astype(np.float32))
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (130, 96, 4096), (600, 6500, 128), (257, 12300, 256), (200, 6000, 128)])
+@pytest.mark.parametrize("M,N,K", [(33, 1376, 512), (130, 96, 4096), (600, 6500, 128), (257, 12300, 256), (200, 6000, 128),
+                                   (90, 6000, 128), (127, 11008, 256)])
 def test_ffn_upgate_f16_many_rows(dev, rng, M, N, K):
     x = rng.standard_normal((M, K)).astype(np.float16)
     up = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)

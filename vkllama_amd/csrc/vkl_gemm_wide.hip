@@ -612,15 +612,15 @@ gemm_wide_q8_kernel (const GemmArgs a, int tiles_m, int tiles_n, int per_xcd, in
 // less there; a reduction launch 5 + its bytes at 2.5 TB/s).
 // Below kWideMinGroups workgroups the tile kernel of vkl_gemm_mfma.hip does
 // better.
-// (Below 128 token rows the two are about even: 64 x 4096 x 11008 takes 28 us
-// there and 34 us here, 100 x 4096 x 4096 21 and 16.)
 constexpr int kWideMinRows = 128;
-// the fused up/gate pair (three times the weights of a square product) already
-// from 65 rows on (where the tile kernel needs a second row of 64-row tiles), in
-// one partly empty row of 128-row tiles: 13B 108 -> 92 us at 80 rows, 7B
-// 84 -> 66 us at 127; below (13B at 64 rows: 83 against 88 us), and for the other
-// products (down at 7B: 39 -> 42 us at 96 rows), the tile kernel does better
-constexpr int kWideMinRowsUpgate = 65;
+// From 65 rows on (where the tile kernel needs a second row of 64-row tiles) in
+// one partly empty row of 128-row tiles: fp16 weights, the fused up/gate pair,
+// and Q8_0 products with K up to 5120.  Measured at 80-127 rows: fp16 4096^2
+// 20-23 -> 16-17 us, 12288 x 4096 41-43 -> 35-39, up/gate 62-67 -> 47-50 (13B
+// 89-97 -> 65-70), down even; Q8_0 up/gate 84 -> 66 (13B 108 -> 92), 4096^2
+// 27 -> 24.  Not the Q8_0 down product (K = 11008: 39 -> 42 us), and nothing
+// below 65 rows (13B Q8_0 up/gate at 64 rows: 83 against 88 us).
+constexpr int kWideMinRowsPartial = 65;
 constexpr int kWideMinGroups = 88, kWideMinGroupsQ8 = 128;
 
 struct WidePlan
@@ -640,7 +640,7 @@ WidePlan
 wide_plan (const GemmArgs &a)
 {
   WidePlan none = { 0, 1 }, best = none;
-  const int min_rows = a.upgate && a.wtype == 8 ? kWideMinRowsUpgate : kWideMinRows;
+  const int min_rows = a.wtype == 1 || a.upgate || a.K <= 5120 ? kWideMinRowsPartial : kWideMinRows;
   if ((a.wtype != 1 && a.wtype != 8) || a.batch > 1 || (a.K % WBK) != 0 || a.M < min_rows)
     return none;
   if (a.wtype == 8)
