@@ -73,6 +73,26 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
  * counterpart in the reference, which has no persistent kernels. */
 int vkl_decode_status (const vkl_decode_model *m, void *stream);
 
+/* n_steps greedy tokens without a host round trip per token: step i reads
+ * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
+ * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the
+ * device.  The launches of one step are captured once in a HIP graph (per
+ * model / buffers / attention form) and replayed; results are identical to
+ * n_steps calls of vkl_decode_step in mode 0.  logits32 (optional) receives
+ * the logits of the last step.  The stream must not be capturing. */
+int vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
+                     int n_steps, float *logits32, void *stream);
+
+/* device pointer to the fp16 logits [vocab] of the last step inside scratch */
+const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
+/* arg-max over fp32 values (first maximum); out is device-visible */
+int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Measuring and testing aids.  None has a counterpart in the reference; the
+ * product path (vkl_decode_step / vkl_decode_loop above) does not need them.
+ * ------------------------------------------------------------------------ */
+
 /* From which context length on the attention phase runs in its split form
  * (each head's rows over several workgroups of one launch, whose parts
  * the last workgroup of the head to finish combines) instead of one workgroup
@@ -103,16 +123,6 @@ int vkl_decode_set_fuse_attn_wo (int on);
  * graphs cached by vkl_decode_loop, so no decode work may be in flight. */
 int vkl_decode_set_wait_limit (int polls, int silent_heads);
 
-/* n_steps greedy tokens without a host round trip per token: step i reads
- * ids[i] (device memory) at position pos0 + i and writes its arg-max id to
- * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the
- * device.  The launches of one step are captured once in a HIP graph (per
- * model / buffers / attention form) and replayed; results are identical to
- * n_steps calls of vkl_decode_step in mode 0.  logits32 (optional) receives
- * the logits of the last step.  The stream must not be capturing. */
-int vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
-                     int n_steps, float *logits32, void *stream);
-
 /* Phase timing (mode 0 only; a measuring aid without counterpart in the
  * reference, whose GPUDevice timestamps play this role in
  * src/core/gpu_device.cpp).  While enabled, vkl_decode_step brackets every
@@ -139,11 +149,6 @@ int vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
 /* algorithmic bytes one launch of phase `kind` moves at context length L
  * (weights + scales read once; activations, KV rows and results once) */
 size_t vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L);
-
-/* device pointer to the fp16 logits [vocab] of the last step inside scratch */
-const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
-/* arg-max over fp32 values (first maximum); out is device-visible */
-int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
 
 #ifdef __cplusplus
 }
