@@ -263,9 +263,19 @@ def main():
         dom_bytes = per_phase[dom]["bytes_per_launch"]
         # the kernel's name as a profiler prints it: phase number, weight type,
         # 4096-value chunks of the staged activation row
-        phase_no = {"kqv": 0, "attention": 1, "attention+wo": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5}[dom]
+        phase_no = {"kqv": 0, "attention": 1, "attention+wo": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5,
+                    "layer": 8}[dom]
         kstage = cfg["ffn"] if dom == "down" else cfg["dim"]
-        if dom == "attention+wo":
+        per = 34.0 / 32.0 if cfg["wtype"] == 8 else 2.0
+        wbytes = (cfg["n_layers"] * (4.0 * cfg["dim"] ** 2 + 3.0 * cfg["dim"] * cfg["ffn"])
+                  + cfg["vocab"] * cfg["dim"]) * per
+        if dom == "layer":
+            # (row chunks of 4096 values as the library picks them: see launch_layer_wt)
+            xd, xf = (cfg["dim"] + 4095) // 4096, (cfg["ffn"] + 4095) // 4096
+            xd, xf = (1, 1) if (xd, xf) == (1, 1) else ((1, 3) if xd == 1 and xf <= 3 else (2, 4))
+            dom_kernel = "decode_layer_kernel<%d, %d, %d, %s> (the five phases of a layer in one launch)" % (
+                8 if cfg["wtype"] == 8 else 1, xd, xf, "true" if wbytes > (288 << 20) else "false")
+        elif dom == "attention+wo":
             dom_kernel = "decode_attn_wo_kernel<%d, %d> (attention + Wo)" % (8 if cfg["wtype"] == 8 else 1,
                                                                             min(4, (cfg["dim"] + 4095) // 4096))
         elif dom == "attention":
@@ -273,17 +283,13 @@ def main():
         else:
             # last argument: weights of a step beyond what the caches hold are
             # requested with the non-temporal hint (same rule as the library's)
-            per = 34.0 / 32.0 if cfg["wtype"] == 8 else 2.0
-            wbytes = (cfg["n_layers"] * (4.0 * cfg["dim"] ** 2 + 3.0 * cfg["dim"] * cfg["ffn"])
-                      + cfg["vocab"] * cfg["dim"]) * per
             dom_kernel = "decode_phase_direct_kernel<%d, %d, %d, %s> (%s)" % (
                 phase_no, 8 if cfg["wtype"] == 8 else 1, min(4, (kstage + 4095) // 4096),
                 "true" if wbytes > (288 << 20) else "false", dom)
         dom_pair_us = per_phase[dom]["avg_us"]
     else:
-        # persistent mode: one launch per token, priced as a whole
         dom, dom_us, dom_n, dom_bytes = None, ms_per_step * 1e3, steps, step_bytes
-        dom_kernel, dom_pair_us = "decode step (all phases of one token)", None
+        dom_kernel, dom_pair_us = "decode step (all launches of one token)", None
     dom_gbs = dom_bytes / (dom_us * 1e-6) / 1e9
 
     # the same loop through Model::operator() (token id from the host, 128 KB of
@@ -312,8 +318,8 @@ def main():
         "data": "synthetic: random-init N(0,0.02) weights" + (" quantised to Q8_0" if cfg["wtype"] == 8 else " in FP16")
                 + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
-                   "decode_mode": ("launch-per-phase" + (", replayed from a HIP graph" if args.decode_graph else ""),
-                                   "persistent")[args.decode_mode],
+                   "decode_mode": ("one launch per phase", "one launch per layer")[args.decode_mode]
+                                  + (", replayed from a HIP graph" if args.decode_graph else ""),
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "decode_tokens_per_second_host_interface": round(host_tok_s, 1),
         "prefill_tokens_per_second": round(n_prompt / (prefill_ms * 1e-3), 1),

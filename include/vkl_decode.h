@@ -43,6 +43,25 @@ typedef struct
   const float *output_norm;        /* [dim] */
   const float *freqc, *freqs;      /* RoPE tables fp32 [maxlen, head_dim/2] */
   void *scratch; /* device, vkl_decode_scratch_bytes() bytes, zeroed once */
+  /* Options of this model's decode steps; all zero = the defaults.  They are
+   * part of the model, not of the process: two models in one process do not
+   * share them, and the graphs vkl_decode_loop caches are keyed by them. */
+  int attn_split_min;  /* context length from which the attention phase runs in
+                          its split form (each head's rows over several
+                          workgroups of one launch); 0 = 1024, the measured
+                          break-even; a value beyond maxlen never splits.  The
+                          split form weights the V rows with fp32
+                          probabilities, the one-workgroup form with
+                          probabilities rounded to fp16 as the reference's
+                          softmax stores them: outputs differ by at most one
+                          fp16 step */
+  int separate_attn_wo; /* mode 0: attention (one workgroup per head) and the Wo
+                          projection as two launches instead of one */
+  int wait_polls;      /* polls after which a wait between workgroups inside a
+                          launch gives up; 0 = the default (some 10 ms) */
+  int wait_test;       /* testing aid: the workgroups that others wait for
+                          never raise their flags, so every such wait gives
+                          up */
 } vkl_decode_model;
 
 /* bytes of device scratch a model of these dimensions needs */
@@ -50,12 +69,15 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
 
 /* One token at KV position `pos` (context length becomes pos + 1).
  *  tok      device-visible uint32: the input token id (ids >= vocab -> 0)
- *  mode     0 = one launch per phase; 1 = one persistent launch per step:
- *           the workgroups stay resident, hand activations over through
- *           memory with bounded waits for one another, and keep the next
- *           phase's weights streaming meanwhile (Q8_0 weights and contexts
- *           below 1024 positions; other steps run as mode 0).  The GPU must
- *           not be shared while a persistent launch runs: see
+ *  mode     0 = one launch per phase (attention and Wo share one below the
+ *           split length); 1 = one launch per layer: all workgroups stay
+ *           resident through the five phases, hand activations over through
+ *           memory with bounded waits for one another, and have the next
+ *           phase's weights on the way meanwhile (above the split length:
+ *           K/Q/V, split attention, then Wo + up/gate + down in one
+ *           launch).  Results are bit for bit those of mode 0.  Models whose
+ *           rows the one-launch form does not cover run as mode 0.  The GPU
+ *           must not be shared while such a launch runs: see
  *           vkl_decode_status
  *  logits32 optional device fp32 [vocab]: widened fp16 logits
  *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
@@ -65,12 +87,17 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
                      uint32_t pos, int mode, float *logits32,
                      uint32_t *next_tok, void *stream);
 
-/* Persistent launches (mode 1) need every workgroup resident at once; where
- * that does not hold (a GPU shared with other work) a bounded wait inside the
- * kernel gives up, the launch still ends, and its results are invalid.  This
- * call synchronises the stream and returns 0 if no wait gave up since the
- * last call, hipErrorLaunchFailure otherwise (the mark is cleared).  No
- * counterpart in the reference, which has no persistent kernels. */
+/* Launches in which workgroups wait for one another (mode 1; the attention +
+ * Wo launch of mode 0) need every workgroup resident at once and the
+ * workgroups dealt round-robin over the XCDs; where that does not hold (a GPU
+ * shared with other work, another dispatch order) a bounded wait inside the
+ * kernel gives up or the kernel notices the placement, the launch still ends,
+ * the workgroup concerned drops its results instead of storing them, and the
+ * step's results are invalid.  This call synchronises the stream and returns
+ * 0 if nothing of the kind happened since the last call,
+ * hipErrorLaunchFailure otherwise (the mark is cleared); the caller then
+ * repeats the step with mode 0 and separate_attn_wo = 1, which wait for
+ * nothing.  No counterpart in the reference, which has no such kernels. */
 int vkl_decode_status (const vkl_decode_model *m, void *stream);
 
 /* n_steps greedy tokens without a host round trip per token: step i reads
@@ -78,10 +105,10 @@ int vkl_decode_status (const vkl_decode_model *m, void *stream);
  * ids[i + 1], the loop of app/llama2_infer.cpp:140-177 with the sampler on the
  * device.  The launches of one step are captured once in a HIP graph (per
  * model / buffers / attention form) and replayed; results are identical to
- * n_steps calls of vkl_decode_step in mode 0.  logits32 (optional) receives
- * the logits of the last step.  The stream must not be capturing. */
+ * n_steps calls of vkl_decode_step in the same mode.  logits32 (optional)
+ * receives the logits of the last step.  The stream must not be capturing. */
 int vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
-                     int n_steps, float *logits32, void *stream);
+                     int n_steps, int mode, float *logits32, void *stream);
 
 /* device pointer to the fp16 logits [vocab] of the last step inside scratch */
 const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
@@ -93,49 +120,21 @@ int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
  * product path (vkl_decode_step / vkl_decode_loop above) does not need them.
  * ------------------------------------------------------------------------ */
 
-/* From which context length on the attention phase runs in its split form
- * (each head's rows over several workgroups of one launch, whose parts
- * the last workgroup of the head to finish combines) instead of one workgroup
- * per head.  The split form weights the V rows with fp32 probabilities, the
- * one-workgroup form with probabilities rounded to fp16 as the reference's
- * softmax stores them: outputs differ by at most one fp16 step.  0 restores the default (1024,
- * the measured break-even); a value beyond the context length never splits.
- * Process-wide; a testing and measuring aid without counterpart in the
- * reference.  Graphs captured by vkl_decode_loop hold the form they were
- * captured with. */
-int vkl_decode_set_attn_split (int min_len);
-
-/* Whether mode 0 runs the attention phase (one workgroup per head, i.e. below
- * the split length above) and the Wo projection in one launch: the projection's
- * workgroups request their weights while the heads are computed and start
- * once every head has counted itself in (a bounded wait; one that gives up is
- * reported by vkl_decode_status).  Results are bit for bit those of the two
- * launches.  On by default; process-wide; a measuring and testing aid without
- * counterpart in the reference.  Graphs captured by vkl_decode_loop hold the
- * form they were captured with. */
-int vkl_decode_set_fuse_attn_wo (int on);
-
-/* A testing aid without counterpart in the reference: after how many polls a
- * wait inside the fused attention + Wo launch gives up (0 restores the
- * default, some 10 ms), and whether the head workgroups leave the flags unset,
- * which makes every such wait give up: the launches still end, the results
- * are invalid and vkl_decode_status reports it.  Process-wide; drops the
- * graphs cached by vkl_decode_loop, so no decode work may be in flight. */
-int vkl_decode_set_wait_limit (int polls, int silent_heads);
-
-/* Phase timing (mode 0 only; a measuring aid without counterpart in the
+/* Phase timing (a measuring aid without counterpart in the
  * reference, whose GPUDevice timestamps play this role in
  * src/core/gpu_device.cpp).  While enabled, vkl_decode_step brackets every
  * phase launch with a pair of HIP events on the launch stream and
  * synchronises the stream before it returns.  vkl_decode_phase_times adds up,
  * per phase kind (0 K/Q/V, 1 attention, 2 Wo, 3 up/gate, 4 down, 5 lm_head,
- * 6 arg-max), the elapsed milliseconds and the number of launches since the
- * last call, and clears both. */
-#define VKL_DECODE_PHASES 7
+ * 6 arg-max, 8 a whole layer in one launch as mode 1 runs it; 7 is not
+ * used), the elapsed milliseconds and the number of launches since the last
+ * call, and clears both. */
+#define VKL_DECODE_PHASES 9
+#define VKL_DECODE_PHASE_LAYER 8
 int vkl_decode_phase_timing (int enable);
 int vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
                             uint64_t launches[VKL_DECODE_PHASES]);
-/* Launches phase `kind` (0..4: of every layer in turn; 5: lm_head) `rounds`
+/* Launches phase `kind` (0..4 and 8: of every layer in turn; 5: lm_head) `rounds`
  * times back to back on `stream` between ONE pair of events and returns the
  * average milliseconds per launch: the kernel's duration without the cost of
  * an event pair per launch.  The phase's outputs in scratch are overwritten

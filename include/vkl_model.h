@@ -71,13 +71,20 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
                                 float topp, uint64_t seed,
                                 uint32_t *out_ids_h, double *prefill_ms,
                                 double *decode_ms);
-/* options: fused one-token decode on/off, decode launch mode (0 = one launch
- * per phase, 1 = one persistent launch per token), replay of the greedy loop
- * from a HIP graph on/off, the context length from which attention is split
- * over several workgroups per head, attention and the Wo projection in one
- * launch on/off ("fuse_attn_wo"), the reference's last-block RoPE position
- * quirk */
+/* options, all per model: "fused_decode" (fused one-token decode on/off),
+ * "decode_mode" (0 = one launch per phase, 1 = one launch per layer),
+ * "decode_graph" (replay of the greedy loop from a HIP graph on/off),
+ * "attn_split_min" (the context length from which attention is split over
+ * several workgroups per head), "fuse_attn_wo" (mode 0: attention and the Wo
+ * projection in one launch on/off), "lastblock_rope_quirk" (the reference's
+ * last-block RoPE position), "wait_test" (a testing aid: waits between
+ * workgroups inside a launch give up after that many polls and are never
+ * answered; 0 = normal), "phase_timing" (process-wide measuring aid) */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);
+/* how often a decode step or a generation of this model was repeated, on the
+ * launches that wait for nothing, because a wait between workgroups inside a
+ * launch had given up (a shared GPU); 0 in normal operation */
+size_t vkl_model_decode_recoveries (const vkl_model *m);
 /* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */
 int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,
                              uint16_t *out_h, size_t n);
@@ -85,7 +92,7 @@ int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,
 size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
 /* per-phase measurements of the fused decode step: option "phase_timing"
  * switches them on; see vkl_decode_phase_times / vkl_decode_phase_bytes */
-int vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7]);
+int vkl_model_phase_times (vkl_model *m, double ms_sum[9], uint64_t launches[9]);
 size_t vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L);
 /* vkl_decode_phase_replay on this model's stream; overwrites decode scratch */
 int vkl_model_phase_replay (vkl_model *m, int kind, size_t pos, int rounds,

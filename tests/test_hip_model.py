@@ -261,11 +261,11 @@ def test_blocks_of_different_type_never_reach_the_fused_step():
 
 
 @pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5), (TINY, 1234)])
-def test_persistent_decode_matches_oracle(cfg, seed):
-    """decode_mode 1: one persistent launch per token; the workgroups hand the
-    activations over through memory and wait for one another.  Ids identical to
-    the oracle's, and logits bit-identical to the launch-per-phase step (both
-    keep the same order of every sum)."""
+def test_layer_launch_decode_matches_oracle(cfg, seed):
+    """decode_mode 1: one launch per layer; the workgroups stay for the five
+    phases, hand the activations over through memory and wait for one another.
+    Ids identical to the oracle's, and logits bit-identical to the
+    launch-per-phase step (both keep the same order of every sum)."""
     w = M.synth_weights(cfg, seed=seed)
     prompt = np.array([5, 17, 99, 3], np.uint32)
     m = M.Llama2(cfg, w)
@@ -277,10 +277,71 @@ def test_persistent_decode_matches_oracle(cfg, seed):
     got = m.forward([7], 4)
     assert logit_err(got, om.forward([7], 4)) < 1e-2
     assert np.array_equal(got, m0.forward([7], 4))
-    ids, _, t_dec = m.generate_greedy(prompt, 32)
     want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 32)
-    assert list(ids) == list(want)
+    for graph in (1, 0):
+        m.set_option("decode_graph", graph)
+        ids, _, t_dec = m.generate_greedy(prompt, 32)
+        assert list(ids) == list(want), graph
+    assert m.decode_recoveries() == 0
     m.close(), m0.close()
+
+
+@pytest.mark.parametrize("cfg", [dict(dim=4096, n_layers=2, n_heads=32, ffn=11008, vocab=1024, maxlen=256, eps=1e-5,
+                                      wtype=8),
+                                 dict(dim=5120, n_layers=1, n_heads=40, ffn=13824, vocab=640, maxlen=128, eps=1e-5,
+                                      wtype=8),
+                                 dict(dim=4096, n_layers=2, n_heads=32, ffn=11008, vocab=1024, maxlen=256, eps=1e-5,
+                                      wtype=1),
+                                 dict(dim=512, n_layers=3, n_heads=8, ffn=1376, vocab=2048, maxlen=128, eps=1e-5,
+                                      wtype=1)])
+def test_layer_launch_equals_phase_launches(cfg):
+    """One launch per layer against one launch per phase at the row widths of
+    the 7B and 13B shapes and with fp16 weights: greedy ids and the logits of a
+    further step bit for bit, replayed from a graph and launched step by step
+    (the launch-per-phase form is what the other tests hold against the
+    oracle)."""
+    w = M.synth_weights(cfg, seed=3)
+    prompt = np.random.default_rng(3).integers(3, cfg["vocab"], 7).astype(np.uint32)
+    m = M.Llama2(cfg, w)
+    runs = {}
+    for mode in (0, 1):
+        m.set_option("decode_mode", mode)
+        for graph in (1, 0):
+            m.set_option("decode_graph", graph)
+            ids, _, _ = m.generate_greedy(prompt, 40)
+            logits = m.forward([int(ids[-1])], 7 + 39)
+            runs[(mode, graph)] = (list(ids), logits.copy())
+    assert m.decode_recoveries() == 0
+    m.close()
+    ref_ids, ref_logits = runs[(0, 0)]
+    for key, (ids, logits) in runs.items():
+        assert ids == ref_ids, key
+        assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
+
+
+def test_layer_launch_long_context_equals_phase_launches():
+    """Above the split length mode 1 runs K/Q/V, the split attention and then
+    Wo + up/gate + down in one launch; ids and logits bit for bit those of the
+    launch-per-phase form, across the switch at the split length."""
+    cfg = dict(dim=256, n_layers=2, n_heads=4, ffn=352, vocab=640, maxlen=160, eps=1e-5, wtype=8)
+    w = M.synth_weights(cfg, seed=21)
+    prompt = np.random.default_rng(21).integers(3, cfg["vocab"], 90).astype(np.uint32)
+    m = M.Llama2(cfg, w)
+    m.set_option("attn_split_min", 100)
+    runs = {}
+    for mode in (0, 1):
+        m.set_option("decode_mode", mode)
+        for graph in (1, 0):
+            m.set_option("decode_graph", graph)
+            ids, _, _ = m.generate_greedy(prompt, 30)
+            logits = m.forward([int(ids[-1])], 90 + 29)
+            runs[(mode, graph)] = (list(ids), logits.copy())
+    assert m.decode_recoveries() == 0
+    m.close()
+    ref_ids, ref_logits = runs[(0, 0)]
+    for key, (ids, logits) in runs.items():
+        assert ids == ref_ids, key
+        assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
 
 
 @pytest.mark.parametrize("heads", [4, 2])
@@ -361,32 +422,46 @@ def test_attention_and_wo_in_one_launch_equals_two_launches(cfg):
         assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
 
 
-def test_wait_inside_the_fused_launch_is_bounded_and_reported():
-    """The projection's workgroups of the fused attention + Wo launch wait for the
-    heads with a bounded number of polls.  With the heads kept silent from the
-    host (option "fused_wait_test": the flags stay unset, 4 polls) every wait
-    gives up: all launches still end, and the status word turns the generation
-    and the logits read-back into errors instead of wrong tokens.  Afterwards
-    the same model generates the same ids as before."""
+@pytest.mark.parametrize("mode", [0, 1])
+def test_wait_inside_a_launch_is_bounded_and_recovered(mode):
+    """Workgroups that wait for others inside a launch (the Wo projection for
+    the attention heads, in the attention + Wo launch of mode 0 and in the
+    one-launch layer of mode 1) poll a bounded number of times.  With the heads
+    kept silent from the host (option "wait_test": the flags stay unset, 4
+    polls) every such wait gives up: all launches still end, the workgroups
+    concerned store nothing, the status word reports it, and the model repeats
+    the work on the launches that wait for nothing.  The ids are those of an
+    undisturbed run, and the repeat is counted."""
     cfg = TINY
     w = M.synth_weights(cfg, seed=9)
     prompt = np.random.default_rng(9).integers(3, cfg["vocab"], 6).astype(np.uint32)
     m = M.Llama2(cfg, w)
+    m.set_option("decode_mode", mode)
     want, _, _ = m.generate_greedy(prompt, 24)
-    m.set_option("fused_wait_test", 4)
+    want_logits = m.forward([int(want[0])], 6)
+    assert m.decode_recoveries() == 0
+    n = 0
     try:
         for graph in (0, 1):
+            m.set_option("decode_mode", mode), m.set_option("fuse_attn_wo", 1)
+            m.set_option("wait_test", 4)
             m.set_option("decode_graph", graph)
-            with pytest.raises(capi.VklError):
-                m.generate_greedy(prompt, 24)
-        with pytest.raises(capi.VklError):
-            m.forward([int(want[0])], 6)
+            ids, _, _ = m.generate_greedy(prompt, 24)
+            n += 1
+            assert m.decode_recoveries() == n
+            assert list(ids) == list(want)
+        m.set_option("decode_mode", mode), m.set_option("fuse_attn_wo", 1)
+        got = m.forward([int(want[0])], 6)
+        assert m.decode_recoveries() == n + 1
+        assert np.array_equal(got, want_logits)
     finally:
-        m.set_option("fused_wait_test", 0)
+        m.set_option("wait_test", 0)
+    m.set_option("decode_mode", mode), m.set_option("fuse_attn_wo", 1)
     for graph in (1, 0):
         m.set_option("decode_graph", graph)
         ids, _, _ = m.generate_greedy(prompt, 24)
         assert list(ids) == list(want)
+    assert m.decode_recoveries() == n + 1
     m.close()
 
 

@@ -1,0 +1,393 @@
+// One layer of the decode step as ONE launch.
+//
+// The launch-per-phase kernels stream at about 6 TB/s while they run, but
+// every kernel boundary costs 2.5-3.5 us in which the memory is idle (the end
+// of one kernel's tail, the launch gap, the way to the next kernel's first
+// bytes): five boundaries on a layer of some 50 us.  Here the G workgroups
+// (512 threads, two per compute unit, all resident at once) stay for the five
+// phases of a layer and keep the shape of the launch-per-phase kernels: every
+// wave computes, a workgroup normalises its own copy of the row with all of
+// its threads, two weight items per wave are in flight.  What changes is the
+// hand-over between phases:
+//
+//   results -> memory (stores written through, acknowledged)
+//   barrier, ONE arrival per workgroup at the counter of the XCD it runs
+//   on; the XCD's last arriver raises the XCD's flag
+//   NEXT phase: both weight items of every wave are requested first, so that
+//   the memory keeps streaming during everything that follows
+//   wave 0 polls the eight flags (bounded); barrier
+//   the row is read with ordinary loads, normalised, staged in LDS
+//
+// Ordinary loads of a row that was written inside the same launch are safe
+// because (a) caches are invalidated between launches and no buffer is read
+// before it is written inside one launch (the residual stream after the Wo
+// projection has a buffer of its own, xm), so no cache holds an older copy of
+// a line, and (b) the results are dealt so that every 128-byte line of a row
+// is written by workgroups of ONE XCD (see Deal): an L2 has either seen all
+// writes to a line or none.  Nothing is assumed about which XCD a workgroup
+// lands on: it reads the XCD's number from the hardware register and takes a
+// ticket at the XCD's counter, and (XCD, ticket) decide its role and share.
+//
+// Attention runs on n_heads workgroups (the first to have taken a ticket on
+// each XCD), one head each, while the others already hold their Wo weights;
+// the heads count in at one counter and the last one raises a flag per XCD.
+//
+// Flags carry the number of the launch (a word in the sync area that
+// workgroup 0 advances at the end of every launch), counters are zeroed by
+// their last arriver: nothing has to be cleared between launches.  Every wait
+// is bounded; a workgroup whose wait gave up marks the error word that
+// vkl_decode_status reports, keeps counting in (so that nobody else waits for
+// it in vain) and drops its results into a sink instead of storing them.  The
+// error word names the first cause: 0x100 | stage for a wait that gave
+// up, 0x200 | xcd for an XCD that was dealt more than its share of workgroups.
+#include "vkl_decode_gemv.h"
+#include "vkl_decode_shared.h"
+#include <algorithm>
+
+namespace vkl
+{
+namespace dec
+{
+namespace
+{
+// words of the layer-sync area (Scratch::lsync); every counter and flag on a
+// 128-byte line of its own
+constexpr int kLsLaunch = 0;              // launches completed so far
+constexpr int kLsCnt = 32;                // + (stage * 8 + slot) * 32
+constexpr int kLsFlag = 32 + 4 * 8 * 32;  // + (stage * 8 + slot) * 32
+constexpr int kLsTicket = kLsFlag + 4 * 8 * 32; // + slot * 32: workgroups of the XCD that have started
+static_assert ((kLsTicket + 8 * 32) * 4 <= kLayerSyncBytes, "layer-sync area too small");
+constexpr int kSyncErr = 1; // word of Scratch::sync: a wait gave up
+constexpr int kLayerSpinLimit = 1 << 14;
+
+enum Stage
+{
+  ST_KQV = 0,
+  ST_ATT,
+  ST_WO,
+  ST_UP
+};
+
+// the error word keeps the FIRST cause reported since the host last looked
+__device__ __forceinline__ void
+report (uint32_t *err, uint32_t code)
+{
+  uint32_t expected = 0u;
+  __hip_atomic_compare_exchange_strong (err, &expected, code, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// counts the workgroup in at `cnt` once its stores have been acknowledged;
+// the last of `n` arrivals zeroes the counter and raises `nflags` flags
+__device__ __forceinline__ void
+arrive (uint32_t *cnt, uint32_t n, uint32_t *flag, int nflags, uint32_t mark, bool silent)
+{
+  __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
+  __syncthreads ();
+  if (threadIdx.x < 64)
+    {
+      uint32_t old = 0;
+      if (threadIdx.x == 0)
+        old = __hip_atomic_fetch_add (cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
+      if (old + 1u == n)
+        {
+          if (threadIdx.x == 0)
+            st_coherent_u32 (cnt, 0u);
+          if ((int)threadIdx.x < nflags && !silent)
+            st_coherent_u32 (flag + 32 * (int)threadIdx.x, mark);
+        }
+    }
+}
+
+// Wave 0 polls `nflags` flags (1 or 8, 32 words apart) until all carry `mark`;
+// ends with a barrier.  False: the wait gave up (the error word is set).
+__device__ __forceinline__ bool
+wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t *err,
+            uint32_t *lds_word, uint32_t code)
+{
+  if (threadIdx.x < 64)
+    {
+      const uint32_t *f = flag + 32 * ((int)threadIdx.x & (nflags - 1));
+      bool ok = false;
+      for (int spin = 0; spin < limit; ++spin)
+        {
+          const bool up = ld_coherent_u32 (f) == mark;
+          if (__builtin_amdgcn_ballot_w64 (!up) == 0)
+            {
+              ok = true;
+              break;
+            }
+          __builtin_amdgcn_s_sleep (2);
+        }
+      if (threadIdx.x == 0)
+        {
+          *lds_word = ok ? 1u : 0u;
+          if (!ok)
+            report (err, code);
+        }
+    }
+  __syncthreads ();
+  return *lds_word != 0u;
+}
+
+// XD / XF: 4096-element chunks of a row of dim / ffn values
+template <int WT, int XD, int XF, bool NT>
+__global__ __launch_bounds__ (kDecThreads) __attribute__ ((amdgpu_waves_per_eu (4, 4))) void
+decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int first, int G,
+                     size_t lds_word_at)
+{
+  extern __shared__ __align__ (16) uint8_t lds[];
+  typedef Gemv<WT, NT, 2> GV2;    // K/Q/V, up/gate: two-row units
+  typedef Gemv<WT, false, 1> GVO; // Wo: one-row units, plain loads (short phase)
+  typedef Gemv<WT, NT, 1> GVD;    // down
+  const vkl_decode_model &m = p.m;
+  const int dim = m.dim, ffn = m.ffn, nh = first == 0 ? m.n_heads : 0;
+  const int wg = (int)blockIdx.x;
+  uint32_t *ls = p.s.lsync;
+  uint32_t *err = p.s.sync + kSyncErr;
+  uint32_t *word = (uint32_t *)(lds + lds_word_at); // [0] wait result, [1] XCD, [2] ticket
+  uint16_t *xl = (uint16_t *)lds;
+  const bool silent = m.wait_test != 0;
+  // the number of this launch; flags raised in it carry it
+  const uint32_t mark = ld_coherent_u32 (ls + kLsLaunch) + 1u;
+  // once a wait has given up the step is lost anyway: the launches that
+  // follow until the host has looked do not wait at all
+  const int limit
+      = ld_coherent_u32 (err) != 0u ? 1 : (m.wait_polls > 0 ? m.wait_polls : kLayerSpinLimit);
+  // Where this workgroup runs, and its number among the workgroups of that
+  // XCD in order of arrival: nothing is assumed about how the dispatcher
+  // deals workgroups to XCDs except that each gets G / 8 of them (if not, a
+  // counter below never fills up and the bounded waits report it).
+  const int n_slot = G >> 3;
+  uint32_t xcc = 0, ticket = 0;
+  if (threadIdx.x == 0)
+    {
+      xcc = __builtin_amdgcn_s_getreg (20 | (0 << 6) | (3 << 11)) & 7u;
+      ticket = __hip_atomic_fetch_add (ls + kLsTicket + 32 * xcc, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    }
+  auto cnt_of = [&] (int stage, int k) { return ls + kLsCnt + (stage * 8 + k) * 32; };
+  auto flag_of = [&] (int stage, int k) { return ls + kLsFlag + (stage * 8 + k) * 32; };
+  bool live = true; // false once a wait of this workgroup gave up
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
+  int slot = 0, idx = 0;
+  // (after a barrier that follows the store below)
+  auto place = [&] () {
+    slot = __builtin_amdgcn_readfirstlane ((int)word[1]);
+    idx = __builtin_amdgcn_readfirstlane ((int)word[2]);
+    if (idx >= n_slot && threadIdx.x == 0)
+      report (err, 0x200u | (uint32_t)slot);
+  };
+
+  if (first == 0)
+    {
+      // ---- RMSNorm + K/Q/V -------------------------------------------------
+      const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
+                 wv = wmat<WT> (lw.wv, dim, dim);
+      float *red = (float *)(lds + (size_t)dim * 2);
+      load_row<XD> (p.s.x, dim, x);
+      load_norm<XD> (lw.attn_norm, dim, nw);
+      __builtin_amdgcn_sched_barrier (0);
+      GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1, nullptr, true);
+      if (threadIdx.x == 0)
+        word[1] = xcc, word[2] = ticket;
+      stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+      place ();
+      e = Epilogue{};
+      e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
+      e.through = true;
+      GV2::run (ps, A, B, xl, e, red);
+      arrive (cnt_of (ST_KQV, slot), (uint32_t)n_slot, flag_of (ST_KQV, slot), 1, mark, false);
+    }
+  else
+    {
+      if (threadIdx.x == 0)
+        word[1] = xcc, word[2] = ticket;
+      __syncthreads ();
+      place ();
+    }
+  // heads h = slot, slot + 8, ... run on the first workgroups of XCD `slot`
+  const int n_heads_here = (nh - slot + 7) >> 3;
+  const bool is_head = idx < n_heads_here;
+  if (is_head)
+    {
+      // ---- one head of the attention ---------------------------------------
+      live = wait_flags (flag_of (ST_KQV, 0), 8, mark, limit, err, word, 0x100u | ST_KQV);
+      if (live)
+        {
+          if (m.head_dim == 128)
+            attention_head<128, true> (p, lw, idx * 8 + slot, lds, nullptr);
+          else
+            attention_head<64, true> (p, lw, idx * 8 + slot, lds, nullptr);
+        }
+      arrive (cnt_of (ST_ATT, 0), (uint32_t)nh, flag_of (ST_ATT, 0), 8, mark, silent);
+    }
+  else
+    {
+      // ---- Wo + residual -> xm ---------------------------------------------
+      const QMat w = wmat<WT> (lw.wo, dim, dim);
+      float *red = (float *)(lds + (size_t)dim * 2);
+      GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true,
+                  Deal{ 1, slot, idx - n_heads_here, n_slot - n_heads_here });
+      if (first == 0)
+        live = wait_flags (flag_of (ST_ATT, slot), 1, mark, limit, err, word, 0x100u | ST_ATT);
+      load_row<XD> (p.s.att, dim, x);
+      stage_row<false, XD> (x, dim, xl, nw, 0.f, red, nullptr);
+      e = Epilogue{};
+      e.y[0] = live ? p.s.xm : p.s.sink, e.residual = p.s.x;
+      e.through = true;
+      GVO::run (ps, A, B, xl, e, red);
+    }
+  arrive (cnt_of (ST_WO, slot), (uint32_t)n_slot, flag_of (ST_WO, slot), 1, mark, false);
+
+  // ---- RMSNorm + up/gate with SiLU -> t -------------------------------------
+  {
+    const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
+    float *red = (float *)(lds + (size_t)dim * 2);
+    load_norm<XD> (lw.ffn_norm, dim, nw);
+    __builtin_amdgcn_sched_barrier (0);
+    GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true,
+                Deal{ 1, slot, idx, n_slot });
+    live = wait_flags (flag_of (ST_WO, 0), 8, mark, limit, err, word, 0x100u | ST_WO) && live;
+    load_row<XD> (p.s.xm, dim, x);
+    stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+    e = Epilogue{};
+    e.y[0] = live ? p.s.t : p.s.sink;
+    e.through = true;
+    GV2::run (ps, A, B, xl, e, red);
+    arrive (cnt_of (ST_UP, slot), (uint32_t)n_slot, flag_of (ST_UP, slot), 1, mark, false);
+  }
+
+  // ---- down + residual -> x ---------------------------------------------------
+  {
+    const QMat w = wmat<WT> (lw.w_down, dim, ffn);
+    float *red = (float *)(lds + (size_t)ffn * 2);
+    GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, p.s.xm, true);
+    live = wait_flags (flag_of (ST_UP, 0), 8, mark, limit, err, word, 0x100u | ST_UP) && live;
+    load_row<XF> (p.s.t, ffn, x);
+    stage_row<false, XF> (x, ffn, xl, nw, 0.f, red, nullptr);
+    e = Epilogue{};
+    e.y[0] = live ? p.s.x : p.s.sink, e.residual = p.s.xm;
+    GVD::run (ps, A, B, xl, e, red);
+  }
+  // (every workgroup has read the launch number and taken its ticket before
+  // its first arrival, and this one has seen all of them arrive)
+  if (wg == 0 && threadIdx.x < 9)
+    st_coherent_u32 (threadIdx.x == 8 ? ls + kLsLaunch : ls + kLsTicket + 32 * (int)threadIdx.x,
+                     threadIdx.x == 8 ? mark : 0u);
+}
+
+// the token's embedding row as the start of the residual stream
+template <int WT>
+__global__ __launch_bounds__ (kDecThreads) void
+embed_row_kernel (const Params p)
+{
+  const int dim = p.m.dim;
+  uint32_t tok = ldg (step_tok (p));
+  if (tok >= (uint32_t)p.m.vocab)
+    tok = 0;
+  for (int i = (int)(blockIdx.x * kDecThreads + threadIdx.x) * 8; i < dim;
+       i += (int)(gridDim.x * kDecThreads) * 8)
+    {
+      uint32_t o[4];
+      if (WT == 8)
+        {
+          const QMat tab = qmat (p.m.tok_embd, p.m.vocab, dim);
+          const unsigned long long q
+              = ldg ((const unsigned long long *)(tab.q + (size_t)tok * dim + i));
+          const float sc = h2f (ldg (tab.d + (size_t)tok * (dim >> 5) + (i >> 5)));
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              const int8_t b0 = (int8_t)((q >> (16 * j)) & 0xff);
+              const int8_t b1 = (int8_t)((q >> (16 * j + 8)) & 0xff);
+              o[j] = (uint32_t)f2h ((float)b0 * sc) | ((uint32_t)f2h ((float)b1 * sc) << 16);
+            }
+        }
+      else
+        {
+          const uint4 v = ldg4 ((const uint16_t *)p.m.tok_embd + (size_t)tok * dim + i);
+          o[0] = v.x, o[1] = v.y, o[2] = v.z, o[3] = v.w;
+        }
+      uint32_t *dst = (uint32_t *)(p.s.x + i);
+      stg (dst, o[0]), stg (dst + 1, o[1]), stg (dst + 2, o[2]), stg (dst + 3, o[3]);
+    }
+}
+
+template <int WT, int XD, int XF, bool NT>
+int
+launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                hipStream_t s)
+{
+  const size_t at = (lds_bytes_needed (p.m.dim, p.m.ffn, p.m.maxlen, p.m.head_dim) + 15) & ~(size_t)15;
+  const size_t lds = at + 16;
+  static size_t lds_set = 0;
+  if (lds > lds_set)
+    {
+      VKL_HIP (hipFuncSetAttribute ((const void *)decode_layer_kernel<WT, XD, XF, NT>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      lds_set = lds;
+    }
+  decode_layer_kernel<WT, XD, XF, NT>
+      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, first, G, at);
+  return 0;
+}
+
+template <int WT, int XD, int XF>
+int
+launch_layer_x (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                hipStream_t s)
+{
+  return p.stream_once ? launch_layer_t<WT, XD, XF, true> (p, lw, layer, first, G, s)
+                       : launch_layer_t<WT, XD, XF, false> (p, lw, layer, first, G, s);
+}
+
+template <int WT>
+int
+launch_layer_wt (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                 hipStream_t s)
+{
+  const int xd = (p.m.dim + 4095) / 4096, xf = (p.m.ffn + 4095) / 4096;
+  if (xd == 1 && xf == 1)
+    return launch_layer_x<WT, 1, 1> (p, lw, layer, first, G, s);
+  if (xd == 1 && xf <= 3)
+    return launch_layer_x<WT, 1, 3> (p, lw, layer, first, G, s);
+  return launch_layer_x<WT, 2, 4> (p, lw, layer, first, G, s);
+}
+} // namespace
+
+bool
+layer_launch_supported (const vkl_decode_model &m, int G)
+{
+  // rows of up to two (dim) and four (ffn) chunks of 4096; every slot needs
+  // workgroups beside the heads; two workgroups per compute unit must fit
+  return m.dim <= 8192 && m.ffn <= 16384 && (m.dim % 8) == 0 && (m.ffn % 8) == 0
+         && G >= m.n_heads + 8 && (G % 8) == 0
+         && 2 * (lds_bytes_needed (m.dim, m.ffn, m.maxlen, m.head_dim) + 32) <= 160 * 1024;
+}
+
+int
+launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+              hipStream_t s)
+{
+  return p.m.wtype == 8 ? launch_layer_wt<8> (p, lw, layer, first, G, s)
+                        : launch_layer_wt<1> (p, lw, layer, first, G, s);
+}
+
+int
+launch_embed_row (const Params &p, hipStream_t s)
+{
+  const int grid = std::max (1, std::min (8, p.m.dim / (kDecThreads * 8)));
+  if (p.m.wtype == 8)
+    embed_row_kernel<8><<<dim3 ((unsigned)grid), dim3 (kDecThreads), 0, s>>> (p);
+  else
+    embed_row_kernel<1><<<dim3 ((unsigned)grid), dim3 (kDecThreads), 0, s>>> (p);
+  return 0;
+}
+} // namespace dec
+} // namespace vkl

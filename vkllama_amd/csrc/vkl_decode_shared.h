@@ -20,8 +20,11 @@ struct Scratch
   float *logits32;    // [vocab]
   float *amax_val;    // [1024]
   uint32_t *amax_idx; // [1024]
-  uint32_t *sync;     // arrival counters and flags, error word, loop state
-  uint8_t *ptab;      // persistent launch: table of the token's phases
+  uint32_t *sync;     // error word, loop state, counter and flags of the fused attention + Wo launch
+  // one launch per layer (vkl_decode_layer.hip)
+  uint16_t *xm;       // [dim] residual stream between the Wo and the down projection
+  uint16_t *sink;     // [max(3*dim, ffn)] where a workgroup whose wait gave up drops its results
+  uint32_t *lsync;    // arrival counters and flags of the stages, launch count
   // long-context attention, split over kAttnChunks chunks of the context
   float *part_max;    // [heads][kAttnChunks]
   float *part_sum;    // [heads][kAttnChunks]
@@ -30,6 +33,7 @@ struct Scratch
   size_t bytes;
 };
 
+constexpr int kLayerSyncBytes = 12288; // see vkl_decode_layer.hip
 constexpr int kAttnChunks = 32;      // upper bound on chunks per head
 constexpr int kAttnSplitMinLen = 1024; // shorter contexts use one workgroup per head (measured at 7B:
                                        // 10.5 against 12.4 us at 768 positions, 12.6 / 12.5 at 1024)
@@ -58,7 +62,9 @@ carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd,
   s.amax_val = (float *)(p + o), o += 4096;
   s.amax_idx = (uint32_t *)(p + o), o += 4096;
   s.sync = (uint32_t *)(p + o), o += 4096;
-  s.ptab = p + o, o += align256 ((size_t)(5 * n_layers + 1) * 128);
+  s.xm = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
+  s.sink = (uint16_t *)(p + o), o += align256 ((size_t)(3 * dim > ffn ? 3 * dim : ffn) * 2);
+  s.lsync = (uint32_t *)(p + o), o += kLayerSyncBytes;
   s.part_max = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_sum = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_out = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * hd * 4);
@@ -450,8 +456,15 @@ final_argmax (const Params &p, int G, uint8_t *lds)
     }
 }
 
-// one token as a single persistent launch (vkl_decode_persist.hip); Q8_0 weights
-int launch_persistent (const Params &p, int n_cu, hipStream_t s);
+// One layer of the step as a single launch (vkl_decode_layer.hip).  first = 0:
+// K/Q/V, attention with one workgroup per head, Wo, up/gate, down; first = 1:
+// from the Wo projection on (the attention output is in memory).  G workgroups
+// that must all be resident at once.
+bool layer_launch_supported (const vkl_decode_model &m, int G);
+int launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                  hipStream_t s);
+// the token's embedding row -> residual stream (one small launch in front of layer 0)
+int launch_embed_row (const Params &p, hipStream_t s);
 } // namespace dec
 } // namespace vkl
 #endif

@@ -227,19 +227,11 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_decode_graph (value != 0);
   else if (n == "phase_timing")
     vkl_decode_phase_timing (value);
-  else if (n == "fuse_attn_wo")
-    vkl_decode_set_fuse_attn_wo (value);
-  else if (n == "fused_wait_test")
+  else if (n == "fuse_attn_wo" || n == "wait_test" || n == "attn_split_min")
     {
-      // value > 0: waits of the fused launch give up after `value` polls and
-      // the heads never signal; 0: back to normal
-      if (vkl_decode_set_wait_limit (value > 0 ? value : 0, value > 0))
-        return fail (m, absl::InvalidArgumentError ("fused_wait_test out of range"));
-    }
-  else if (n == "attn_split_min")
-    {
-      if (vkl_decode_set_attn_split (value))
-        return fail (m, absl::InvalidArgumentError ("attn_split_min must not be negative"));
+      // options of this model's fused decode steps (fields of vkl_decode_model)
+      if (!m->model->set_decode_option (name, value))
+        return fail (m, absl::InvalidArgumentError ("option " + n + ": value out of range"));
     }
   else
     return fail (m, absl::InvalidArgumentError ("unknown option " + n));
@@ -263,13 +255,20 @@ vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value, uint16_t *out,
 }
 
 extern "C" size_t
+vkl_model_decode_recoveries (const vkl_model *m)
+{
+  return m && m->model ? m->model->decode_recoveries () : 0;
+}
+
+extern "C" size_t
 vkl_model_decode_step_bytes (const vkl_model *m, size_t L)
 {
   return m && m->model ? m->model->decode_step_bytes (L) : 0;
 }
 
 extern "C" int
-vkl_model_phase_times (vkl_model *m, double ms_sum[7], uint64_t launches[7])
+vkl_model_phase_times (vkl_model *m, double ms_sum[VKL_DECODE_PHASES],
+                       uint64_t launches[VKL_DECODE_PHASES])
 {
   if (!m || !ms_sum || !launches)
     return (int)absl::StatusCode::kInvalidArgument;

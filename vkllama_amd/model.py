@@ -32,6 +32,7 @@ SIGNATURES = {
     "vkl_model_generate_sampled": (i32, [vp, vp, sz, sz, i32, C.c_float, u64, vp, C.POINTER(C.c_double),
                                          C.POINTER(C.c_double)]),
     "vkl_model_set_option": (i32, [vp, C.c_char_p, i32]),
+    "vkl_model_decode_recoveries": (sz, [vp]),
     "vkl_model_read_kv_cache": (i32, [vp, sz, i32, vp, sz]),
     "vkl_model_decode_step_bytes": (sz, [vp, sz]),
     "vkl_model_phase_times": (i32, [vp, vp, vp]),
@@ -241,16 +242,19 @@ class Llama2:
                     "vkl_model_read_kv_cache")
         return out.view(np.float16)
 
+    def decode_recoveries(self):
+        return int(lib().vkl_model_decode_recoveries(self._h))
+
     def decode_step_bytes(self, L):
         return int(lib().vkl_model_decode_step_bytes(self._h, L))
 
-    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax")
+    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax", "unused", "layer")
 
     def phase_times(self):
         """{phase: (milliseconds summed, launches)} since the last call; filled
         while the option "phase_timing" is on."""
-        ms = np.zeros(7, np.float64)
-        n = np.zeros(7, np.uint64)
+        ms = np.zeros(len(self.PHASES), np.float64)
+        n = np.zeros(len(self.PHASES), np.uint64)
         self._check(lib().vkl_model_phase_times(self._h, ms.ctypes.data, n.ctypes.data), "phase_times")
         return {k: (float(ms[i]), int(n[i])) for i, k in enumerate(self.PHASES)}
 

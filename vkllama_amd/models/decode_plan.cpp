@@ -2,6 +2,7 @@
 #include "models/llama2.h"
 #include "vkl_hip.h"
 #include <string.h>
+#include <string>
 
 namespace vkllama
 {
@@ -170,9 +171,34 @@ DecodePlan::loop (uint32_t *ids, size_t pos0, size_t n_steps)
         "fused decode does not cover this model");
   adopted_valid_ = false;
   return hip_status ("decode loop",
-                     vkl_decode_loop (&desc_, ids, (uint32_t)pos0, (int)n_steps,
+                     vkl_decode_loop (&desc_, ids, (uint32_t)pos0, (int)n_steps, mode_,
                                       (float *)logits32_.data (),
                                       gpu_->stream ()));
+}
+
+bool
+DecodePlan::set_option (const char *name, int value)
+{
+  const std::string n (name);
+  if (n == "attn_split_min")
+    {
+      if (value < 0)
+        return false;
+      desc_.attn_split_min = value;
+    }
+  else if (n == "fuse_attn_wo")
+    desc_.separate_attn_wo = value ? 0 : 1;
+  else if (n == "wait_test")
+    {
+      // value > 0: waits between workgroups give up after `value` polls and
+      // the workgroups waited for never signal; 0: back to normal
+      if (value < 0 || value >= (1 << 24))
+        return false;
+      desc_.wait_polls = value, desc_.wait_test = value > 0 ? 1 : 0;
+    }
+  else
+    return false;
+  return true;
 }
 
 absl::Status
@@ -182,10 +208,16 @@ DecodePlan::check ()
   if (!usable_)
     return absl::OkStatus ();
   if (int e = vkl_decode_status (&desc_, gpu_->stream ()))
-    return absl::InternalError (absl::StrFormat (
-        "decode step: a wait between workgroups gave up (%s); the GPU must not be "
-        "shared while such a launch runs",
-        vkl_error_string (e)));
+    {
+      const bool had_waits = mode_ != 0 || !desc_.separate_attn_wo;
+      mode_ = 0, desc_.separate_attn_wo = 1;
+      return absl::UnavailableError (absl::StrFormat (
+          "decode step: a wait between workgroups gave up (%s): the GPU is shared or "
+          "deals workgroups to its XCDs in another order; %s",
+          vkl_error_string (e),
+          had_waits ? "switched to the launches that wait for nothing, repeat the call"
+                    : "no such launch was in use"));
+    }
   return absl::OkStatus ();
 }
 

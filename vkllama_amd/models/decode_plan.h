@@ -26,6 +26,9 @@ struct DecodePlan
   // true when the fused kernels cover this model (Q8_0, head width 64/128)
   bool usable () const { return usable_; }
   void set_mode (int mode) { mode_ = mode; }
+  // options of this model's decode steps (fields of vkl_decode_model);
+  // false for a name the plan does not know or a value out of range
+  bool set_option (const char *name, int value);
   const vkl_decode_model &desc () const { return desc_; }
   // token id given by the host / read from device-visible memory
   absl::Status step_host_token (uint32_t tok, size_t offset);
@@ -36,8 +39,10 @@ struct DecodePlan
   // ids is device memory, ids[0] the first input token
   absl::Status loop (uint32_t *ids, size_t pos0, size_t n_steps);
   int mode () const { return mode_; }
-  // after the stream has been synchronised: did a persistent launch (mode 1)
-  // give up a wait?  (vkl_decode_status)
+  // After the stream has been synchronised: did a wait between workgroups
+  // inside a launch give up (vkl_decode_status)?  If so the plan switches to
+  // the launches that wait for nothing (mode 0, attention and Wo apart) and
+  // the status is Unavailable: the caller repeats the generation.
   absl::Status check ();
   // copies the fp32 logits of the last step (fused or adopted) to the host
   absl::Status read_logits (float *dst);

@@ -362,6 +362,12 @@ Model::set_decode_mode (int mode)
     plan_->set_mode (mode);
 }
 
+bool
+Model::set_decode_option (const char *name, int value)
+{
+  return plan_ && plan_->set_option (name, value);
+}
+
 void
 Model::set_lastblock_rope_quirk (bool on)
 {
@@ -432,7 +438,16 @@ Model::operator() (std::vector<uint32_t> const &toks, const size_t offset)
       VKLLAMA_STATUS_OK (output_command_->wait ());
       VKLLAMA_STATUS_OK (plan_->step_host_token (toks[0], offset));
       buf_logits.resize (vocab_);
-      VKLLAMA_STATUS_OK (plan_->read_logits (buf_logits.data ()));
+      auto rs = plan_->read_logits (buf_logits.data ());
+      if (absl::IsUnavailable (rs))
+        {
+          // a wait between workgroups gave up; the plan has switched to the
+          // launches that wait for nothing: the same step once more
+          ++decode_recoveries_;
+          VKLLAMA_STATUS_OK (plan_->step_host_token (toks[0], offset));
+          rs = plan_->read_logits (buf_logits.data ());
+        }
+      VKLLAMA_STATUS_OK (rs);
       return buf_logits;
     }
   auto output = forward_ (toks, offset);
@@ -487,6 +502,24 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
                         std::vector<uint32_t> &out, double *prefill_ms,
                         double *decode_ms)
 {
+  auto s = generate_once_ (prompt, n_gen, out, prefill_ms, decode_ms);
+  if (absl::IsUnavailable (s))
+    {
+      // a wait between workgroups gave up somewhere in the loop; the plan has
+      // switched to the launches that wait for nothing.  The generation is
+      // repeated from the prompt: KV rows written so far are rewritten with
+      // the same values.
+      ++decode_recoveries_;
+      s = generate_once_ (prompt, n_gen, out, prefill_ms, decode_ms);
+    }
+  return s;
+}
+
+absl::Status
+Model::generate_once_ (std::vector<uint32_t> const &prompt, size_t n_gen,
+                       std::vector<uint32_t> &out, double *prefill_ms,
+                       double *decode_ms)
+{
   using clock = std::chrono::steady_clock;
   out.clear ();
   if (n_gen == 0)
@@ -528,8 +561,7 @@ Model::generate_greedy (std::vector<uint32_t> const &prompt, size_t n_gen,
   const auto t1 = clock::now ();
   size_t n_toks = prompt.size () + 1;
   size_t i0 = 1;
-  if (fused_decode_ && plan_->usable () && decode_graph_ && plan_->mode () == 0
-      && n_gen > 1 && !samp_on_)
+  if (fused_decode_ && plan_->usable () && decode_graph_ && n_gen > 1 && !samp_on_)
     {
       // ids[0] is at position prompt.size (); each replay appends one id
       VKLLAMA_STATUS_OK (plan_->loop (ids, prompt.size (), n_gen - 1));

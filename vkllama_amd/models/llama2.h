@@ -157,8 +157,11 @@ public:
   // ---- additions -----------------------------------------------------------
   void set_fused_decode (bool on) { fused_decode_ = on; }
   void set_lastblock_rope_quirk (bool on);
-  // 0 = one launch per decode phase, 1 = one persistent launch per token
+  // 0 = one launch per decode phase, 1 = one launch per layer
   void set_decode_mode (int mode);
+  // options of the fused decode steps: "attn_split_min", "fuse_attn_wo",
+  // "wait_test" (DecodePlan::set_option)
+  bool set_decode_option (const char *name, int value);
   // greedy loop replayed from a captured HIP graph (default) or launched
   // step by step
   void set_decode_graph (bool on) { decode_graph_ = on; }
@@ -191,6 +194,9 @@ public:
   size_t decode_phase_bytes (int kind, size_t L) const;
   absl::Status decode_phase_replay (int kind, size_t pos, int rounds,
                                     double *avg_ms, uint64_t *launches);
+  // how often a decode step or generation was repeated because a wait between
+  // workgroups inside a launch had given up (DecodePlan::check)
+  size_t decode_recoveries () const { return decode_recoveries_; }
 
 private:
   absl::StatusOr<Tensor> forward_ (std::vector<uint32_t> const &toks,
@@ -216,7 +222,11 @@ private:
   int samp_k_ = 1;
   float samp_p_ = -1.f;
   uint64_t samp_seed_ = 0;
+  size_t decode_recoveries_ = 0;
   absl::Status pick_token_ (uint32_t *dst, size_t position);
+  absl::Status generate_once_ (std::vector<uint32_t> const &prompt, size_t n_gen,
+                               std::vector<uint32_t> &out, double *prefill_ms,
+                               double *decode_ms);
 };
 
 }
