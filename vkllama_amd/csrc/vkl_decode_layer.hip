@@ -59,6 +59,24 @@ constexpr int kLsTicket = kLsFlag + 4 * 8 * 32; // + slot * 32: workgroups of th
 static_assert ((kLsTicket + 8 * 32) * 4 <= kLayerSyncBytes, "layer-sync area too small");
 constexpr int kSyncErr = 1; // word of Scratch::sync: a wait gave up
 constexpr int kLayerSpinLimit = 1 << 14;
+// The last wave of a workgroup is its courier.  A wave's loads return in
+// order, so a poll or a row read issued behind two weight items would wait
+// for those 16 KiB to arrive from a memory that has 60 MB of requests queued.
+// The courier therefore requests no weights ahead: it counts the workgroup
+// in, polls, brings the row into LDS, and only then streams its own (the
+// workgroup's last) units while the other waves are at their later items.
+constexpr int kCourier = kDecWaves - 1;
+// Weight items a worker requests before the wait for the previous phase.  The
+// memory path of a compute unit serves requests in order, also across waves:
+// the courier's polls and the row queue behind whatever the 14 workers of the
+// compute unit have requested, so the look-ahead is what the wait can hide
+// (one item: 116 KiB per compute unit, some 4 us at the rate a compute unit
+// is served), not everything the registers can hold.
+#ifndef VKL_LAYER_AHEAD
+#define VKL_LAYER_AHEAD 2
+#endif
+constexpr int kAhead = VKL_LAYER_AHEAD;
+#define VKL_LDS __attribute__ ((address_space (3)))
 
 enum Stage
 {
@@ -84,24 +102,86 @@ arrive (uint32_t *cnt, uint32_t n, uint32_t *flag, int nflags, uint32_t mark, bo
 {
   __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
   __syncthreads ();
-  if (threadIdx.x < 64)
+  // (the courier counts in: the other waves go straight on to request the
+  // next phase's weights instead of waiting for the counter's answer)
+  if (__builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier)
     {
+      const int lane = (int)threadIdx.x & 63;
       uint32_t old = 0;
-      if (threadIdx.x == 0)
+      if (lane == 0)
         old = __hip_atomic_fetch_add (cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
       if (old + 1u == n)
         {
-          if (threadIdx.x == 0)
+          if (lane == 0)
             st_coherent_u32 (cnt, 0u);
-          if ((int)threadIdx.x < nflags && !silent)
-            st_coherent_u32 (flag + 32 * (int)threadIdx.x, mark);
+          if (lane < nflags && !silent)
+            st_coherent_u32 (flag + 32 * lane, mark);
         }
     }
 }
 
-// Wave 0 polls `nflags` flags (1 or 8, 32 words apart) until all carry `mark`;
-// ends with a barrier.  False: the wait gave up (the error word is set).
+// The courier polls `nflags` flags (1 or 8, 32 words apart) until all carry
+// `mark` (bounded), then brings the row of K fp16 values straight into LDS
+// (every lane 16 bytes per load, a load fills 1 KiB of consecutive LDS; the
+// tail of the last KiB repeats the row's last 16 bytes and lands in unused
+// LDS behind the row).  Ends with a barrier.  False: the wait gave up (the
+// error word is set, the row is not there).
+template <bool COURIER>
+__device__ __forceinline__ bool
+courier_fetch (bool poll, const uint32_t *flag, int nflags, uint32_t mark, int limit,
+               uint32_t *err, uint32_t *lds_word, uint32_t code, const uint16_t *src, int K,
+               uint8_t *xl, unsigned long long *tr = nullptr)
+{
+  if (COURIER)
+    {
+      const int lane = (int)threadIdx.x & 63;
+      bool ok = !poll;
+      if (poll)
+        {
+          const uint32_t *f = flag + 32 * (lane & (nflags - 1));
+          for (int spin = 0; spin < limit; ++spin)
+            {
+              const bool up = ld_coherent_u32 (f) == mark;
+              if (__builtin_amdgcn_ballot_w64 (!up) == 0)
+                {
+                  ok = true;
+                  break;
+                }
+              __builtin_amdgcn_s_sleep (1);
+            }
+        }
+#ifdef VKL_TRACE
+      if (tr && lane == 0)
+        tr[0] = wall_clock64 ();
+#endif
+      if (ok)
+        {
+          const int bytes = K * 2, n = (bytes + 1023) >> 10;
+          for (int i = 0; i < n; ++i)
+            {
+              const int off = min (i * 1024 + lane * 16, bytes - 16);
+              __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)((const uint8_t *)src + off),
+                                                (VKL_LDS void *)(xl + i * 1024), 16, 0, 0);
+            }
+          __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
+        }
+#ifdef VKL_TRACE
+      if (tr && lane == 0)
+        tr[1] = wall_clock64 ();
+#endif
+      if (lane == 0)
+        {
+          *lds_word = ok ? 1u : 0u;
+          if (!ok)
+            report (err, code);
+        }
+    }
+  __syncthreads ();
+  return *lds_word != 0u;
+}
+
+// the plain wait of the head workgroups (they hold no weights)
 __device__ __forceinline__ bool
 wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t *err,
             uint32_t *lds_word, uint32_t code)
@@ -118,7 +198,7 @@ wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t
               ok = true;
               break;
             }
-          __builtin_amdgcn_s_sleep (2);
+          __builtin_amdgcn_s_sleep (1);
         }
       if (threadIdx.x == 0)
         {
@@ -131,6 +211,158 @@ wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t
   return *lds_word != 0u;
 }
 
+// the row as the courier left it in LDS, into the registers stage_row expects
+template <int XCH>
+__device__ __forceinline__ void
+row_from_lds (const uint16_t *xl, int K, XRegs &x)
+{
+#pragma unroll
+  for (int j = 0; j < XCH; ++j)
+    {
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
+      x.v[j] = ((const uint4 *)xl)[idx];
+    }
+}
+
+struct LayerCtx
+{
+  uint32_t *ls, *err, *word;
+  uint32_t mark;
+  int limit, n_slot, slot, idx, nh, first, wg, G, layer;
+  bool silent;
+};
+
+__device__ __forceinline__ uint32_t *
+cnt_of (const LayerCtx &c, int stage, int k)
+{
+  return c.ls + kLsCnt + (stage * 8 + k) * 32;
+}
+
+__device__ __forceinline__ uint32_t *
+flag_of (const LayerCtx &c, int stage, int k)
+{
+  return c.ls + kLsFlag + (stage * 8 + k) * 32;
+}
+
+#ifdef VKL_TRACE
+#define VKL_TL(slot_)                                                          \
+  if (threadIdx.x == 0 && p.trace)                                             \
+    p.trace[((size_t)layer * 1024 + wg) * 16 + (slot_)] = wall_clock64 ();
+#else
+#define VKL_TL(slot_)
+#endif
+
+// A layer from the attention on, for the workers (COURIER false) or for the
+// courier of the workgroup: the same barriers in the same order in both.
+template <int WT, int XD, int XF, bool NT, bool COURIER>
+__device__ __forceinline__ void
+layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uint8_t *lds)
+{
+  typedef Gemv<WT, NT, 2> GV2;    // up/gate: two-row units
+  typedef Gemv<WT, false, 1> GVO; // Wo: one-row units, plain loads (short phase)
+  typedef Gemv<WT, NT, 1> GVD;    // down
+  const vkl_decode_model &m = p.m;
+  const int dim = m.dim, ffn = m.ffn, wg = c.wg, G = c.G, slot = c.slot, idx = c.idx;
+  const int layer = c.layer;
+  (void)layer;
+  uint16_t *xl = (uint16_t *)lds;
+  bool live = true; // false once a wait of this workgroup gave up
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
+  // heads h = slot, slot + 8, ... run on the first workgroups of XCD `slot`
+  const int n_heads_here = (c.nh - slot + 7) >> 3;
+  if (idx < n_heads_here)
+    {
+      // ---- one head of the attention ---------------------------------------
+      live = wait_flags (flag_of (c, ST_KQV, 0), 8, c.mark, c.limit, c.err, c.word, 0x100u | ST_KQV);
+      VKL_TL (4)
+      if (live)
+        {
+          if (m.head_dim == 128)
+            attention_head<128, true> (p, lw, idx * 8 + slot, lds, nullptr);
+          else
+            attention_head<64, true> (p, lw, idx * 8 + slot, lds, nullptr);
+        }
+      VKL_TL (5)
+      arrive (cnt_of (c, ST_ATT, 0), (uint32_t)c.nh, flag_of (c, ST_ATT, 0), 8, c.mark, c.silent);
+    }
+  else
+    {
+      // ---- Wo + residual -> xm ---------------------------------------------
+      const QMat w = wmat<WT> (lw.wo, dim, dim);
+      float *red = (float *)(lds + (size_t)dim * 2);
+      const Deal dl = Deal{ 1, slot, idx - n_heads_here, c.n_slot - n_heads_here };
+      if (!COURIER)
+        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, kAhead, p.s.x, true, dl);
+      live = courier_fetch<COURIER> (c.first == 0, flag_of (c, ST_ATT, slot), 1, c.mark, c.limit,
+                                     c.err, c.word, 0x100u | ST_ATT, p.s.att, dim, lds);
+      if (COURIER)
+        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true, dl);
+      else if (kAhead < 2)
+        GVO::issue (ps, B, 1), ps.primed = 2;
+      VKL_TL (4)
+      e = Epilogue{};
+      e.y[0] = live ? p.s.xm : p.s.sink, e.residual = p.s.x;
+      e.through = true;
+      GVO::run (ps, A, B, xl, e, red);
+      VKL_TL (5)
+    }
+  arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
+  VKL_TL (6)
+
+  // ---- RMSNorm + up/gate with SiLU -> t -------------------------------------
+  {
+    const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
+    float *red = (float *)(lds + (size_t)dim * 2);
+    load_norm<XD> (lw.ffn_norm, dim, nw);
+    __builtin_amdgcn_sched_barrier (0);
+    const Deal dl = Deal{ 1, slot, idx, c.n_slot };
+    if (!COURIER)
+      GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, kAhead, nullptr, true, dl);
+    live = courier_fetch<COURIER> (true, flag_of (c, ST_WO, 0), 8, c.mark, c.limit, c.err, c.word,
+                                   0x100u | ST_WO, p.s.xm, dim, lds)
+           && live;
+    if (COURIER)
+      GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, dl);
+    else if (kAhead < 2)
+      GV2::issue (ps, B, 1), ps.primed = 2;
+    VKL_TL (7)
+    row_from_lds<XD> (xl, dim, x);
+    stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+    VKL_TL (8)
+    e = Epilogue{};
+    e.y[0] = live ? p.s.t : p.s.sink;
+    e.through = true;
+    GV2::run (ps, A, B, xl, e, red);
+    VKL_TL (9)
+    arrive (cnt_of (c, ST_UP, slot), (uint32_t)c.n_slot, flag_of (c, ST_UP, slot), 1, c.mark, false);
+    VKL_TL (10)
+  }
+
+  // ---- down + residual -> x ---------------------------------------------------
+  {
+    const QMat w = wmat<WT> (lw.w_down, dim, ffn);
+    float *red = (float *)(lds + (size_t)ffn * 2);
+    if (!COURIER)
+      GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, kAhead, p.s.xm, true);
+    live = courier_fetch<COURIER> (true, flag_of (c, ST_UP, 0), 8, c.mark, c.limit, c.err, c.word,
+                                   0x100u | ST_UP, p.s.t, ffn, lds)
+           && live;
+    if (COURIER)
+      GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, p.s.xm, true);
+    else if (kAhead < 2)
+      GVD::issue (ps, B, 1), ps.primed = 2;
+    VKL_TL (11)
+    e = Epilogue{};
+    e.y[0] = live ? p.s.x : p.s.sink, e.residual = p.s.xm;
+    GVD::run (ps, A, B, xl, e, red);
+    VKL_TL (13)
+  }
+}
+
 // XD / XF: 4096-element chunks of a row of dim / ffn values
 template <int WT, int XD, int XF, bool NT>
 __global__ __launch_bounds__ (kDecThreads) __attribute__ ((amdgpu_waves_per_eu (4, 4))) void
@@ -138,11 +370,9 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
                      size_t lds_word_at)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
-  typedef Gemv<WT, NT, 2> GV2;    // K/Q/V, up/gate: two-row units
-  typedef Gemv<WT, false, 1> GVO; // Wo: one-row units, plain loads (short phase)
-  typedef Gemv<WT, NT, 1> GVD;    // down
+  typedef Gemv<WT, NT, 2> GV2; // K/Q/V: two-row units
   const vkl_decode_model &m = p.m;
-  const int dim = m.dim, ffn = m.ffn, nh = first == 0 ? m.n_heads : 0;
+  const int dim = m.dim, nh = first == 0 ? m.n_heads : 0;
   const int wg = (int)blockIdx.x;
   uint32_t *ls = p.s.lsync;
   uint32_t *err = p.s.sync + kSyncErr;
@@ -167,14 +397,14 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       ticket = __hip_atomic_fetch_add (ls + kLsTicket + 32 * xcc, 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
     }
-  auto cnt_of = [&] (int stage, int k) { return ls + kLsCnt + (stage * 8 + k) * 32; };
-  auto flag_of = [&] (int stage, int k) { return ls + kLsFlag + (stage * 8 + k) * 32; };
-  bool live = true; // false once a wait of this workgroup gave up
+  VKL_TL (0)
   Epilogue e = {};
   XRegs x;
   NormRegs nw;
   PipeState ps;
   PipeBuf A, B;
+  // (a scalar: branches on it are wave-uniform)
+  const bool courier = __builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier;
   int slot = 0, idx = 0;
   // (after a barrier that follows the store below)
   auto place = [&] () {
@@ -197,12 +427,16 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       if (threadIdx.x == 0)
         word[1] = xcc, word[2] = ticket;
       stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+      VKL_TL (1)
       place ();
       e = Epilogue{};
       e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
       e.through = true;
       GV2::run (ps, A, B, xl, e, red);
-      arrive (cnt_of (ST_KQV, slot), (uint32_t)n_slot, flag_of (ST_KQV, slot), 1, mark, false);
+      VKL_TL (2)
+      arrive (ls + kLsCnt + (ST_KQV * 8 + slot) * 32, (uint32_t)n_slot,
+              ls + kLsFlag + (ST_KQV * 8 + slot) * 32, 1, mark, false);
+      VKL_TL (3)
     }
   else
     {
@@ -211,70 +445,14 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       __syncthreads ();
       place ();
     }
-  // heads h = slot, slot + 8, ... run on the first workgroups of XCD `slot`
-  const int n_heads_here = (nh - slot + 7) >> 3;
-  const bool is_head = idx < n_heads_here;
-  if (is_head)
-    {
-      // ---- one head of the attention ---------------------------------------
-      live = wait_flags (flag_of (ST_KQV, 0), 8, mark, limit, err, word, 0x100u | ST_KQV);
-      if (live)
-        {
-          if (m.head_dim == 128)
-            attention_head<128, true> (p, lw, idx * 8 + slot, lds, nullptr);
-          else
-            attention_head<64, true> (p, lw, idx * 8 + slot, lds, nullptr);
-        }
-      arrive (cnt_of (ST_ATT, 0), (uint32_t)nh, flag_of (ST_ATT, 0), 8, mark, silent);
-    }
+  const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, first, wg, G, layer, silent };
+  // the courier's path is a copy of the workers' (the branch is wave-uniform):
+  // in one copy, with the courier's weight requests under a condition, the
+  // item buffers of the two roles collide and spill
+  if (courier)
+    layer_tail<WT, XD, XF, NT, true> (p, lw, c, lds);
   else
-    {
-      // ---- Wo + residual -> xm ---------------------------------------------
-      const QMat w = wmat<WT> (lw.wo, dim, dim);
-      float *red = (float *)(lds + (size_t)dim * 2);
-      GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true,
-                  Deal{ 1, slot, idx - n_heads_here, n_slot - n_heads_here });
-      if (first == 0)
-        live = wait_flags (flag_of (ST_ATT, slot), 1, mark, limit, err, word, 0x100u | ST_ATT);
-      load_row<XD> (p.s.att, dim, x);
-      stage_row<false, XD> (x, dim, xl, nw, 0.f, red, nullptr);
-      e = Epilogue{};
-      e.y[0] = live ? p.s.xm : p.s.sink, e.residual = p.s.x;
-      e.through = true;
-      GVO::run (ps, A, B, xl, e, red);
-    }
-  arrive (cnt_of (ST_WO, slot), (uint32_t)n_slot, flag_of (ST_WO, slot), 1, mark, false);
-
-  // ---- RMSNorm + up/gate with SiLU -> t -------------------------------------
-  {
-    const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
-    float *red = (float *)(lds + (size_t)dim * 2);
-    load_norm<XD> (lw.ffn_norm, dim, nw);
-    __builtin_amdgcn_sched_barrier (0);
-    GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true,
-                Deal{ 1, slot, idx, n_slot });
-    live = wait_flags (flag_of (ST_WO, 0), 8, mark, limit, err, word, 0x100u | ST_WO) && live;
-    load_row<XD> (p.s.xm, dim, x);
-    stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
-    e = Epilogue{};
-    e.y[0] = live ? p.s.t : p.s.sink;
-    e.through = true;
-    GV2::run (ps, A, B, xl, e, red);
-    arrive (cnt_of (ST_UP, slot), (uint32_t)n_slot, flag_of (ST_UP, slot), 1, mark, false);
-  }
-
-  // ---- down + residual -> x ---------------------------------------------------
-  {
-    const QMat w = wmat<WT> (lw.w_down, dim, ffn);
-    float *red = (float *)(lds + (size_t)ffn * 2);
-    GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, p.s.xm, true);
-    live = wait_flags (flag_of (ST_UP, 0), 8, mark, limit, err, word, 0x100u | ST_UP) && live;
-    load_row<XF> (p.s.t, ffn, x);
-    stage_row<false, XF> (x, ffn, xl, nw, 0.f, red, nullptr);
-    e = Epilogue{};
-    e.y[0] = live ? p.s.x : p.s.sink, e.residual = p.s.xm;
-    GVD::run (ps, A, B, xl, e, red);
-  }
+    layer_tail<WT, XD, XF, NT, false> (p, lw, c, lds);
   // (every workgroup has read the launch number and taken its ticket before
   // its first arrival, and this one has seen all of them arrive)
   if (wg == 0 && threadIdx.x < 9)
