@@ -58,6 +58,9 @@ int vkl_memcpy_h2d (void *dst, const void *src_h, size_t bytes, void *stream);
 int vkl_memcpy_d2h (void *dst_h, const void *src, size_t bytes, void *stream);
 int vkl_memcpy_d2d (void *dst, const void *src, size_t bytes, void *stream);
 int vkl_memset (void *dst, int value, size_t bytes, void *stream);
+/* free and total device memory in bytes (the budget query of the reference's
+ * allocator, src/core/allocator.cpp, as far as callers need it) */
+int vkl_mem_info (size_t *free_bytes, size_t *total_bytes);
 /* device-to-device copy by a plain streaming kernel (bytes % 16 == 0, both
  * pointers 16-byte aligned): the known-size launch that hardware traffic
  * counters are calibrated against; no counterpart in the reference */
@@ -118,6 +121,29 @@ int vkl_matmul_q8_0_noalloc (const void *x, const void *w_planar, int M,
                              int N, int K, size_t xs, size_t ys, float scale,
                              float bias, int act, const void *residual,
                              void *y, float *y32, void *stream);
+/* A testing aid without counterpart in the reference: the address (on the
+ * current device) and size of the static device array that
+ * vkl_matmul_q8_0_noalloc uses as scratch, so that a test can mark it and see
+ * that a call wrote there and nowhere else. */
+int vkl_debug_static_scratch (void **ptr, size_t *bytes);
+/* Which kernel family a matrix product with M token rows takes, and how (no
+ * counterpart in the reference, whose one shader serves every row count): the
+ * launchers of this header decide it in one host function, and this query
+ * returns that decision without touching the GPU, so that tests can pin the
+ * kernel a workload runs on.  wtype 8 = Q8_0, 1 = FP16 weights; nmat 3 = the
+ * fused K/Q/V product; upgate 1 = the fused up/gate pair; workspace_bytes 0 =
+ * the launcher's own scratch, else a caller's (the no-allocation entry point
+ * passes 8 MiB).  Operands are taken to be dense and 16-byte aligned.
+ * family: 0 none, 1 whole-K workgroups (<= 128 rows), 2 / 3 / 4 K slices + a
+ * reduction launch (<= 32 rows), 5 direct-to-LDS tiles, 6 the general tile
+ * kernel, 7 one weight-streaming pass per token row. */
+typedef struct
+{
+  int family, tile_rows, ksplit, groups, launches;
+  size_t workspace_bytes;
+} vkl_gemm_plan_t;
+int vkl_gemm_plan (int M, int N, int K, int wtype, int nmat, int upgate,
+                   size_t workspace_bytes, vkl_gemm_plan_t *out);
 /* src/ops/multiheadattention_v2.cpp:190-202, src/shaders/kqv_fp16_x_q8_0.comp */
 int vkl_kqv_q8_0 (const void *x, const void *wk, const void *wq,
                   const void *wv, int M, int N, int K, void *k, void *q,

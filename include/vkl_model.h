@@ -88,6 +88,14 @@ size_t vkl_model_decode_recoveries (const vkl_model *m);
 /* one layer's K (value = 0) or V (value = 1) cache, [heads, maxlen, hd] fp16 */
 int vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value,
                              uint16_t *out_h, size_t n);
+/* A testing aid, the mirror of vkl_model_read_kv_cache (no counterpart in the
+ * reference, which fills its caches only through
+ * src/ops/update_kv_cache.cpp): replaces one layer's K (value = 0) or V cache
+ * with n = heads * maxlen * head_dim fp16 values from host memory, so that a
+ * test can put a model at a late position without the prompt pass that leads
+ * there. */
+int vkl_model_write_kv_cache (vkl_model *m, size_t layer, int value,
+                              const uint16_t *rows_h, size_t n);
 /* algorithmic bytes of one decode step at context length L */
 size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
 /* per-phase measurements of the fused decode step: option "phase_timing"

@@ -65,6 +65,7 @@ _decl("vko_q8_0_dequantize_row", None, _u8p, C.c_size_t, _f32p, C.c_int)
 _decl("vko_embedding_q8_0", None, _u8p, C.c_uint32, C.c_uint32, _u32p, C.c_uint32, C.c_uint32, _u16p)
 _decl("vko_embedding_f16", None, _u16p, C.c_uint32, C.c_uint32, _u32p, C.c_uint32, C.c_uint32, _u16p)
 _decl("vko_rmsnorm_f16", None, _u16p, _f32p, C.c_int, C.c_int, C.c_float, _u16p)
+_decl("vko_set_lane_order", None, C.c_int)
 _decl("vko_matmul_q8_0", None, _u16p, _u8p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int, _u16p)
 _decl("vko_kqv_q8_0", None, _u16p, _u8p, _u8p, _u8p, C.c_int, C.c_int, C.c_int, _u16p, _u16p, _u16p)
 _decl("vko_ffn_upgate_q8_0", None, _u16p, _u8p, _u8p, C.c_int, C.c_int, C.c_int, _u16p)
@@ -141,6 +142,14 @@ def rmsnorm(x, w, eps):
     out = np.empty_like(x)
     _lib.vko_rmsnorm_f16(_p(x, _u16p), _p(w, _f32p), rows, W, eps, _p(out, _u16p))
     return out.view(np.float16)
+
+
+def set_lane_order(order):
+    """Order in which the dot-product kernels add the 32 lanes of a subgroup
+    (the reference's subgroupAdd leaves it open): 0 pairwise halving (default),
+    1 sequential, 2 neighbours first, 3 sequential from the last lane, 4 groups
+    of eight then the groups.  Process-wide."""
+    _lib.vko_set_lane_order(int(order))
 
 
 def matmul_q8_0(x, w, K, scale=1.0, bias=0.0, act=0):
@@ -367,6 +376,17 @@ class OracleModel:
         n = c["n_heads"] * c["maxlen"] * hd
         p = fn(self._s, layer)
         return np.ctypeslib.as_array(p, shape=(n,)).reshape(c["n_heads"], c["maxlen"], hd).copy().view(np.float16)
+
+    def set_cache(self, layer, value, rows):
+        """Replaces one layer's K (value False) or V cache with `rows`
+        (float16 [heads, maxlen, head_dim]): puts the model at a late position
+        without the prompt pass that leads there."""
+        c = self.cfg
+        hd = c["dim"] // c["n_heads"]
+        rows = np.ascontiguousarray(rows, np.float16)
+        assert rows.shape == (c["n_heads"], c["maxlen"], hd)
+        p = (_lib.vko_state_vcache if value else _lib.vko_state_kcache)(self._s, layer)
+        C.memmove(p, rows.ctypes.data, rows.nbytes)
 
     def kcache(self, layer):
         return self._cache(_lib.vko_state_kcache, layer)

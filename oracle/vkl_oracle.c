@@ -309,9 +309,58 @@ vko_rmsnorm_f16 (const uint16_t *x, const float *w, int rows, int W,
 /* ------------------------------------------------------------------------ */
 /* dot-product kernels                                                       */
 /* ------------------------------------------------------------------------ */
+/* The shaders combine the 32 lanes of a subgroup with subgroupAdd, whose
+ * order of additions Vulkan leaves to the implementation.  Order 0 (the
+ * default, and the one every fixture is written with) halves the lanes
+ * pairwise; 1 adds them one after the other; 2 pairs neighbours first (the
+ * butterfly a cross-lane reduction in hardware makes); 3 adds them one after
+ * the other from the last lane down; 4 adds four groups of eight lanes
+ * sequentially and then the groups.  The switch exists for
+ * tests that ask how far the reference's own freedom moves a result. */
+static int g_lane_order = 0;
+
+void
+vko_set_lane_order (int order)
+{
+  g_lane_order = order;
+}
+
 static inline float
 lanes32_add (float *l)
 {
+  if (g_lane_order == 1)
+    {
+      float s = l[0];
+      for (int i = 1; i < 32; ++i)
+        s += l[i];
+      return s;
+    }
+  if (g_lane_order == 2)
+    {
+      for (int s = 1; s < 32; s <<= 1)
+        for (int i = 0; i < 32; i += 2 * s)
+          l[i] += l[i + s];
+      return l[0];
+    }
+  if (g_lane_order == 3)
+    {
+      float s = l[31];
+      for (int i = 30; i >= 0; --i)
+        s += l[i];
+      return s;
+    }
+  if (g_lane_order == 4)
+    {
+      /* four quads of eight lanes one after the other, then the quads */
+      float q[4];
+      for (int g = 0; g < 4; ++g)
+        {
+          q[g] = l[8 * g];
+          for (int i = 1; i < 8; ++i)
+            q[g] += l[8 * g + i];
+        }
+      return (q[0] + q[1]) + (q[2] + q[3]);
+    }
   for (int s = 16; s > 0; s >>= 1)
     for (int i = 0; i < s; ++i)
       l[i] += l[i + s];

@@ -54,6 +54,11 @@ void vko_rmsnorm_f16 (const uint16_t *x, const float *w, int rows, int W,
                       float eps, uint16_t *out);
 /* src/shaders/matmul_b0_fp16_x_q8_0.comp:52-139: y[m,n] = act(scale *
  * sum_k x[m,k] deq(W[n,k]) + bias) */
+/* order in which the dot-product kernels add the 32 lanes of a subgroup
+ * (subgroupAdd, implementation-defined in Vulkan): 0 pairwise halving (the
+ * default), 1 sequential, 2 neighbours first, 3 sequential from the last
+ * lane, 4 groups of eight then the groups.  Process-wide; for tests. */
+void vko_set_lane_order (int order);
 void vko_matmul_q8_0 (const uint16_t *x, const uint8_t *w, int M, int N,
                       int K, float scale, float bias, int act, uint16_t *y);
 /* src/shaders/kqv_fp16_x_q8_0.comp:42-139 */

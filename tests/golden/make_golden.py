@@ -103,8 +103,59 @@ def ops():
     print("ops fixture:", sum(v.nbytes for v in d.values()), "bytes raw")
 
 
+ORDERS = (0, 1, 2, 3, 4)
+
+
+def llama2_7b_lane_orders():
+    """How far the reference's own freedom moves the 7B-shape workload: its
+    shaders add the 32 lanes of a subgroup with subgroupAdd, whose order
+    Vulkan leaves open.  The committed sequence (oracle order 0) is fed, token
+    by token, to the oracle in each of its lane orders; per step the
+    fixture keeps the order-0 margin between the first and the second choice,
+    every order's arg-max and its largest logit deviation from order 0.
+    Five passes over 7 GB of weights: some minutes of CPU time."""
+    w = M.synth_weights(LLAMA7B, seed=1234)
+    with open(os.path.join(HERE, "llama2_7b_q8_0_c3_greedy.json")) as f:
+        gold = json.load(f)
+    prompt = np.array(gold["prompt"], np.uint32)
+    ids = gold["oracle_ids"]
+    logits = {}
+    for order in ORDERS:
+        O.set_lane_order(order)
+        om = O.OracleModel(LLAMA7B, w)
+        rows = [om.forward(prompt, 0).copy()]
+        for i in range(31):
+            rows.append(om.forward([ids[i]], 32 + i).copy())
+        om.close()
+        logits[order] = np.stack(rows)
+        print("order", order, "arg-max:", [int(np.argmax(r)) for r in rows])
+    O.set_lane_order(0)
+    ref = logits[0]
+    assert [int(np.argmax(r)) for r in ref] == ids
+    srt = np.sort(ref, axis=1)
+    out = {
+        "config": LLAMA7B, "weight_seed": 1234, "prompt": gold["prompt"], "fed_ids": ids,
+        "lane_orders": {"0": "pairwise halving (the oracle's default)", "1": "sequential", "2": "neighbours first",
+                        "3": "sequential from the last lane", "4": "groups of eight, then the groups"},
+        "max_logit": [float(np.abs(r).max()) for r in ref],
+        "margin_order0": [float(srt[i, -1] - srt[i, -2]) for i in range(32)],
+        "second_choice_order0": [int(np.argsort(-ref[i], kind="stable")[1]) for i in range(32)],
+        "argmax": {str(o): [int(np.argmax(r)) for r in logits[o]] for o in ORDERS},
+        "max_abs_dev_from_order0": {str(o): [float(np.abs(logits[o][i] - ref[i]).max()) for i in range(32)]
+                                    for o in ORDERS[1:]},
+    }
+    with open(os.path.join(HERE, "llama2_7b_q8_0_c3_lane_orders.json"), "w") as f:
+        json.dump(out, f, indent=1)
+    for o in ORDERS[1:]:
+        diff = [i for i in range(32) if out["argmax"][str(o)][i] != ids[i]]
+        print("order %d differs from order 0 at steps %s; margins there %s" % (
+            o, diff, [out["margin_order0"][i] for i in diff]))
+
+
 if __name__ == "__main__":
-    if "--llama2-7b" in sys.argv:
+    if "--llama2-7b-lane-orders" in sys.argv:
+        llama2_7b_lane_orders()
+    elif "--llama2-7b" in sys.argv:
         llama2_7b()
     else:
         ops()

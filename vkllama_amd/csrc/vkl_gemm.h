@@ -46,6 +46,29 @@ constexpr int kGemmMinRowsBatched = 9;
 
 // true if the shapes/alignments are ones the kernel covers
 bool gemm_mfma_supported (const GemmArgs &a);
+// Which kernel family gemm_mfma_launch takes for a problem, and how: decided
+// in ONE place (gemm_plan), which the launcher follows and the workspace
+// query reads, so the two cannot disagree.  Pure host arithmetic: no GPU call.
+enum GemmFamily
+{
+  GEMM_NONE = 0,     // not covered (the caller falls back to one pass per token row)
+  GEMM_ROWSFULL = 1, // <= 128 rows, workgroups over the whole of K (vkl_gemm_rowsfull.hip)
+  GEMM_ROWS128 = 2,  // <= 32 rows, K sliced, four independent waves, whole-line loads
+  GEMM_ROWS64 = 3,   // <= 32 rows, K sliced, 64 weight rows per workgroup
+  GEMM_SLICES = 4,   // <= 32 rows, K sliced, 32 weight rows per workgroup (fp16 weights)
+  GEMM_WIDE = 5,     // many rows, direct-to-LDS tiles (vkl_gemm_wide.hip)
+  GEMM_TILE = 6      // the general tile kernel
+};
+struct GemmPlan
+{
+  int family;
+  int tile_rows; // token rows of a tile / of a launch's row block
+  int ksplit;    // parts of the k range whose fp32 sums go through the workspace (1: none)
+  int groups;    // rowsfull: 16-row groups per workgroup
+  int launches;  // kernel launches, the reduction included
+  size_t workspace_bytes;
+};
+GemmPlan gemm_plan (const GemmArgs &a);
 int gemm_mfma_launch (const GemmArgs &a, hipStream_t s);
 // bytes of fp32 scratch gemm_mfma_launch will use for this problem (0: none)
 size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
@@ -53,11 +76,14 @@ size_t gemm_mfma_workspace_bytes (const GemmArgs &a);
 // direct-to-LDS loads (vkl_gemm_wide.hip).  gemm_mfma_launch takes this form
 // where it applies.
 bool gemm_wide_supported (const GemmArgs &a);
+void gemm_wide_choice (const GemmArgs &a, int *tile_rows, int *ksplit); // tile_rows 0: another form
 int gemm_wide_launch (const GemmArgs &a, hipStream_t s);
 size_t gemm_wide_workspace_bytes (const GemmArgs &a); // fp32 scratch of its k-split (0: none)
 // At most 96 token rows against many rows of Q8_0 weights, each workgroup over
 // the whole of K: no partial sums (vkl_gemm_rowsfull.hip).
 bool gemm_rowsfull_supported (const GemmArgs &a);
+int gemm_rowsfull_groups (const GemmArgs &a);  // 16-row groups per workgroup, 0: another form
+int gemm_rowsfull_launch_rows (const GemmArgs &a); // token rows of one launch
 int gemm_rowsfull_launch (const GemmArgs &a, hipStream_t s);
 // The k-split forms' fp32 scratch of a stream (allocated on first use; null if
 // that fails), its size, and the kernel that adds `parts` partial results of

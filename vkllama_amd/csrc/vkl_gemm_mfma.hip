@@ -17,8 +17,10 @@
 // Tiles are numbered so that workgroups that land on the same XCD (id % 8)
 // walk neighbouring tiles with the token-row tile index fastest: the weight
 // tile they share stays in that XCD's L2.
+#include "../../include/vkl_hip.h"
 #include "vkl_common.h"
 #include "vkl_gemm.h"
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -1182,14 +1184,17 @@ tile_ksplit (const GemmArgs &a)
   // steps are slower, and not for fp16 weights)
   const int want = kGemmSplitTarget / (tiles_m * tiles_n * nz);
   int ksplit = want < (WT == 8 ? 2 : 3) ? 1 : std::max (1, std::min (std::min (want, 8), nk / 8));
-  while (ksplit > 1 && (size_t)nm * ksplit * a.M * a.N * sizeof (float) > kSk2Workspace)
+  // as far as the scratch holds the partial tiles (a caller's may be smaller
+  // than the launcher's own)
+  const size_t have = a.workspace ? std::min (a.workspace_bytes, kSk2Workspace) : kSk2Workspace;
+  while (ksplit > 1 && (size_t)nm * ksplit * a.M * a.N * sizeof (float) > have)
     --ksplit;
   return ksplit;
 }
 
 template <int BM, int WT>
 int
-launch_cfg (const GemmArgs &a, hipStream_t s)
+launch_cfg (const GemmArgs &a, int ksplit, hipStream_t s)
 {
   const int tiles_m = (a.M + BM - 1) / BM;
   const int tiles_n = (a.N + (a.upgate ? 64 : BN) - 1) / (a.upgate ? 64 : BN);
@@ -1198,11 +1203,6 @@ launch_cfg (const GemmArgs &a, hipStream_t s)
   // of at least eight steps, as far as the fp32 workspace holds the partial
   // tiles.  Not for batched products (there are tiles enough).
   const int nz = a.upgate ? 1 : a.nmat;
-  int ksplit = tile_ksplit<BM, WT> (a);
-  // (a caller's workspace may be smaller than the launcher's own)
-  while (a.workspace && ksplit > 1
-         && (size_t)(a.upgate ? 2 : a.nmat) * ksplit * a.M * a.N * sizeof (float) > a.workspace_bytes)
-    --ksplit;
   float *ws = nullptr;
   if (ksplit > 1 && !(ws = a.workspace ? a.workspace : skinny2_workspace (s)))
     ksplit = 1;
@@ -1292,68 +1292,108 @@ half_height_tiles (const GemmArgs &a)
 }
 } // namespace
 
+GemmPlan
+gemm_plan (const GemmArgs &a)
+{
+  GemmPlan p = { GEMM_NONE, 0, 1, 0, 0, 0 };
+  if (!gemm_mfma_supported (a))
+    return p;
+  const size_t nm = a.upgate ? 2 : a.nmat;
+  const size_t have = a.workspace ? std::min (a.workspace_bytes, kSk2Workspace) : kSk2Workspace;
+  // up to 128 token rows against many weight rows: workgroups that run over
+  // the whole of K, no partial sums
+  if (const int g = gemm_rowsfull_groups (a))
+    {
+      const int step = gemm_rowsfull_launch_rows (a);
+      p.family = GEMM_ROWSFULL, p.groups = g;
+      p.tile_rows = a.M <= 32 ? 32 : (a.M <= 64 ? 64 : (a.M <= step ? 96 : step));
+      p.launches = (a.M + step - 1) / step;
+      return p;
+    }
+  if (few_rows_form (a))
+    {
+      // Q8_0: the whole-line forms with slices of 512 if their sums fit the
+      // scratch, else (and for fp16 weights) slices of 1024
+      if (a.wtype == 8)
+        {
+          const int S = (a.Kp + kR64Slice - 1) / kR64Slice;
+          const size_t need = nm * S * 32 * a.N * sizeof (float);
+          if (need <= have)
+            {
+              p.family = (a.Kp % 256) == 0 ? GEMM_ROWS128 : GEMM_ROWS64;
+              p.tile_rows = 32, p.ksplit = S, p.launches = 2, p.workspace_bytes = need;
+              return p;
+            }
+        }
+      const int S = a.wtype == 8 ? skinny2_slices<8> (a) : skinny2_slices<1> (a);
+      const size_t need = nm * S * 32 * a.N * sizeof (float);
+      if (need <= have)
+        {
+          p.family = GEMM_SLICES, p.tile_rows = 32, p.ksplit = S, p.launches = 2;
+          p.workspace_bytes = need;
+          return p;
+        }
+    }
+  int wide_rows = 0, wide_ks = 1;
+  gemm_wide_choice (a, &wide_rows, &wide_ks);
+  if (wide_rows)
+    {
+      p.family = GEMM_WIDE, p.tile_rows = wide_rows, p.ksplit = wide_ks;
+      p.launches = wide_ks > 1 ? 2 : 1;
+      p.workspace_bytes = wide_ks > 1 ? (size_t)wide_ks * a.M * a.N * sizeof (float) : 0;
+      return p;
+    }
+  const bool small = half_height_tiles (a);
+  p.family = GEMM_TILE, p.tile_rows = small ? 64 : 128;
+  if (a.wtype == 8)
+    p.ksplit = small ? tile_ksplit<64, 8> (a) : tile_ksplit<128, 8> (a);
+  else if (a.wtype == 1)
+    p.ksplit = small ? tile_ksplit<64, 1> (a) : tile_ksplit<128, 1> (a);
+  p.launches = p.ksplit > 1 ? 2 : 1;
+  p.workspace_bytes = p.ksplit > 1 ? nm * p.ksplit * a.M * a.N * sizeof (float) : 0;
+  return p;
+}
+
 int
 gemm_mfma_launch (const GemmArgs &a, hipStream_t s)
 {
-  if (!gemm_mfma_supported (a))
-    return (int)hipErrorInvalidValue;
-  // up to 96 token rows against many weight rows: workgroups that run over the
-  // whole of K
-  if (gemm_rowsfull_supported (a))
-    return gemm_rowsfull_launch (a, s);
-  if (few_rows_form (a))
+  const GemmPlan p = gemm_plan (a);
+  int err = 0;
+  switch (p.family)
     {
-      int err = 0;
+    case GEMM_ROWSFULL:
+      return gemm_rowsfull_launch (a, s);
+    case GEMM_ROWS128:
+    case GEMM_ROWS64:
       if (launch_rows64_q8 (a, s, err))
         return err;
-      // (if its workspace holds the partial sums)
+      break;
+    case GEMM_SLICES:
       if (a.wtype == 8 ? launch_skinny2<8> (a, s, err) : launch_skinny2<1> (a, s, err))
         return err;
+      break;
+    case GEMM_WIDE:
+      return gemm_wide_launch (a, s);
+    case GEMM_TILE:
+      {
+        const bool small = p.tile_rows == 64;
+        if (a.wtype == 8)
+          return small ? launch_cfg<64, 8> (a, p.ksplit, s) : launch_cfg<128, 8> (a, p.ksplit, s);
+        if (a.wtype == 2)
+          return small ? launch_cfg<64, 2> (a, p.ksplit, s) : launch_cfg<128, 2> (a, p.ksplit, s);
+        return small ? launch_cfg<64, 1> (a, p.ksplit, s) : launch_cfg<128, 1> (a, p.ksplit, s);
+      }
+    default:
+      return (int)hipErrorInvalidValue;
     }
-  if (gemm_wide_supported (a))
-    return gemm_wide_launch (a, s);
-  const bool small = half_height_tiles (a);
-  if (a.wtype == 8)
-    return small ? launch_cfg<64, 8> (a, s) : launch_cfg<128, 8> (a, s);
-  if (a.wtype == 2)
-    return small ? launch_cfg<64, 2> (a, s) : launch_cfg<128, 2> (a, s);
-  return small ? launch_cfg<64, 1> (a, s) : launch_cfg<128, 1> (a, s);
+  // (a sliced form that could not get its scratch buffer or raise its LDS limit)
+  return err ? err : (int)hipErrorOutOfMemory;
 }
 
 size_t
 gemm_mfma_workspace_bytes (const GemmArgs &a)
 {
-  if (!gemm_mfma_supported (a))
-    return 0;
-  const size_t nm = a.upgate ? 2 : a.nmat;
-  if (gemm_rowsfull_supported (a))
-    return 0;
-  if (few_rows_form (a))
-    {
-      // Q8_0: the whole-line form with slices of 512 if its sums fit, else
-      // the form with slices of 1024
-      if (a.wtype == 8)
-        {
-          const size_t need = nm * ((a.Kp + kR64Slice - 1) / kR64Slice) * 32 * a.N * sizeof (float);
-          if (need <= kSk2Workspace && (!a.workspace || need <= a.workspace_bytes))
-            return need;
-        }
-      const int S = a.wtype == 8 ? skinny2_slices<8> (a) : skinny2_slices<1> (a);
-      const size_t need = nm * S * 32 * a.N * sizeof (float);
-      if (need <= kSk2Workspace)
-        return need;
-    }
-  if (gemm_wide_supported (a))
-    return gemm_wide_workspace_bytes (a);
-  const bool small = half_height_tiles (a);
-  int ksplit;
-  if (a.wtype == 8)
-    ksplit = small ? tile_ksplit<64, 8> (a) : tile_ksplit<128, 8> (a);
-  else if (a.wtype == 2)
-    ksplit = 1;
-  else
-    ksplit = small ? tile_ksplit<64, 1> (a) : tile_ksplit<128, 1> (a);
-  return ksplit > 1 ? nm * ksplit * a.M * a.N * sizeof (float) : 0;
+  return gemm_plan (a).workspace_bytes;
 }
 
 void
@@ -1389,6 +1429,43 @@ gemm_static_scratch (size_t *bytes)
   return g_static_scratch[dev];
 }
 } // namespace vkl
+
+extern "C" int
+vkl_debug_static_scratch (void **ptr, size_t *bytes)
+{
+  VKL_CHECK_ARG (ptr && bytes);
+  *ptr = vkl::gemm_static_scratch (bytes);
+  return *ptr ? 0 : (int)hipErrorInvalidSymbol;
+}
+
+extern "C" int
+vkl_gemm_plan (int M, int N, int K, int wtype, int nmat, int upgate, size_t workspace_bytes,
+               vkl_gemm_plan_t *out)
+{
+  VKL_CHECK_ARG (out && M > 0 && N > 0 && K > 0 && (wtype == 8 || wtype == 1));
+  VKL_CHECK_ARG ((nmat == 1 || nmat == 3) && (upgate == 0 || (upgate == 1 && nmat == 1)));
+  *out = vkl_gemm_plan_t{ 7, 1, 1, 0, M, 0 };
+  if (M < (wtype == 8 ? vkl::kGemmMinRows : vkl::kGemmMinRowsF16))
+    return 0;
+  // dense, aligned stand-ins for the operands: only their alignment is looked at
+  vkl::GemmArgs g = {};
+  uint8_t *const aligned = (uint8_t *)4096;
+  g.x = (const uint16_t *)aligned, g.xs = (size_t)K;
+  g.M = M, g.N = N, g.K = K, g.Kp = (K + 31) / 32 * 32;
+  g.wtype = wtype, g.batch = 1, g.nmat = nmat, g.upgate = upgate;
+  for (int t = 0; t < 3; ++t)
+    {
+      g.wq[t] = aligned, g.wd[t] = (const uint16_t *)aligned, g.wh[t] = (const uint16_t *)aligned;
+      g.y[t] = (uint16_t *)aligned;
+    }
+  g.ws = (size_t)K, g.ys = (size_t)N, g.scale = 1.0f;
+  if (workspace_bytes)
+    g.workspace = (float *)aligned, g.workspace_bytes = workspace_bytes;
+  const vkl::GemmPlan p = vkl::gemm_plan (g);
+  if (p.family != vkl::GEMM_NONE)
+    *out = vkl_gemm_plan_t{ p.family, p.tile_rows, p.ksplit, p.groups, p.launches, p.workspace_bytes };
+  return 0;
+}
 
 #ifdef VKL_TRACE
 extern "C" void

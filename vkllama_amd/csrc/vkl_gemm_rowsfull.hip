@@ -432,6 +432,18 @@ gemm_rowsfull_supported (const GemmArgs &a)
   return rowsfull_plan (a) != 0;
 }
 
+int
+gemm_rowsfull_groups (const GemmArgs &a)
+{
+  return rowsfull_plan (a);
+}
+
+int
+gemm_rowsfull_launch_rows (const GemmArgs &a)
+{
+  return a.upgate ? kRowsFullUpgate : kRowsFullPlain;
+}
+
 namespace
 {
 // one launch: up to 64 token rows for the fused up/gate pair, 96 otherwise

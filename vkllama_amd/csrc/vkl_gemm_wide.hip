@@ -686,6 +686,13 @@ gemm_wide_supported (const GemmArgs &a)
   return wide_plan (a).bm != 0;
 }
 
+void
+gemm_wide_choice (const GemmArgs &a, int *tile_rows, int *ksplit)
+{
+  const WidePlan p = wide_plan (a);
+  *tile_rows = p.bm, *ksplit = p.bm ? p.ksplit : 1;
+}
+
 size_t
 gemm_wide_workspace_bytes (const GemmArgs &a)
 {

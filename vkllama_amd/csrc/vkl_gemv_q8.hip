@@ -280,13 +280,14 @@ matmul_q8_0 (const void *x, const void *w_planar, int M, int N, int K, size_t xs
   size_t have = 0;
   if (no_alloc && M >= vkl::kGemmMinRows)
     {
-      // the scratch the launch would use must fit the static array
+      // The plan the allocating entry point would follow (same kernels, same
+      // split: the results are then the same bit for bit) must fit the static
+      // array; a problem whose partial sums exceed it is refused.
       vkl::GemmArgs g = gemm_args (a, 1, 0);
       workspace = vkl::gemm_static_scratch (&have);
       if (!workspace)
         return (int)hipErrorInvalidSymbol;
-      g.workspace = workspace, g.workspace_bytes = have;
-      if (vkl::gemm_mfma_workspace_bytes (g) > have)
+      if (vkl::gemm_plan (g).workspace_bytes > have)
         return (int)hipErrorInvalidValue;
     }
   int err = 0;

@@ -174,6 +174,14 @@ fill_bytes_kernel (uint8_t *dst, uint8_t v, size_t n)
     dst[i] = v;
 }
 
+int
+vkl_mem_info (size_t *free_bytes, size_t *total_bytes)
+{
+  VKL_CHECK_ARG (free_bytes && total_bytes);
+  VKL_HIP (hipMemGetInfo (free_bytes, total_bytes));
+  return 0;
+}
+
 // A fill kernel rather than hipMemsetAsync, so that the call can be recorded
 // into a HIP graph by a caller.
 int

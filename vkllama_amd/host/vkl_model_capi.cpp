@@ -254,6 +254,16 @@ vkl_model_read_kv_cache (vkl_model *m, size_t layer, int value, uint16_t *out,
   return 0;
 }
 
+extern "C" int
+vkl_model_write_kv_cache (vkl_model *m, size_t layer, int value, const uint16_t *rows,
+                          size_t n)
+{
+  if (!m || !m->model || !rows)
+    return (int)absl::StatusCode::kInvalidArgument;
+  auto s = m->model->write_kv_cache (layer, value != 0, rows, n);
+  return s.ok () ? 0 : fail (m, s);
+}
+
 extern "C" size_t
 vkl_model_decode_recoveries (const vkl_model *m)
 {

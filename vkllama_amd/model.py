@@ -33,6 +33,7 @@ SIGNATURES = {
                                          C.POINTER(C.c_double)]),
     "vkl_model_set_option": (i32, [vp, C.c_char_p, i32]),
     "vkl_model_decode_recoveries": (sz, [vp]),
+    "vkl_model_write_kv_cache": (i32, [vp, sz, i32, vp, sz]),
     "vkl_model_read_kv_cache": (i32, [vp, sz, i32, vp, sz]),
     "vkl_model_decode_step_bytes": (sz, [vp, sz]),
     "vkl_model_phase_times": (i32, [vp, vp, vp]),
@@ -241,6 +242,12 @@ class Llama2:
         self._check(lib().vkl_model_read_kv_cache(self._h, layer, int(value), out.ctypes.data, out.size),
                     "vkl_model_read_kv_cache")
         return out.view(np.float16)
+
+    def write_kv_cache(self, layer, value, rows):
+        """rows: float16 [heads, maxlen, head_dim], the whole cache of the layer"""
+        rows = np.ascontiguousarray(rows, np.float16)
+        self._check(lib().vkl_model_write_kv_cache(self._h, layer, int(value), rows.ctypes.data, rows.size),
+                    "vkl_model_write_kv_cache")
 
     def decode_recoveries(self):
         return int(lib().vkl_model_decode_recoveries(self._h))

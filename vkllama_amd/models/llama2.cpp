@@ -624,6 +624,20 @@ Model::read_kv_cache (size_t layer, bool value, std::vector<uint16_t> &out)
   return output_command_->wait ();
 }
 
+absl::Status
+Model::write_kv_cache (size_t layer, bool value, const uint16_t *rows, size_t n)
+{
+  if (layer >= blocks_.size ())
+    return absl::OutOfRangeError ("no such layer");
+  auto *attn = blocks_[layer]->attention ();
+  Tensor &c = value ? attn->vcache () : attn->kcache ();
+  if (!rows || n != c.size ())
+    return absl::InvalidArgumentError (absl::StrFormat (
+        "a cache holds %zu values, %zu given", c.size (), n));
+  VKLLAMA_STATUS_OK (output_command_->upload (rows, n, c));
+  return output_command_->wait ();
+}
+
 size_t
 Model::decode_step_bytes (size_t L) const
 {

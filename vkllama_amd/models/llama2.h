@@ -184,6 +184,13 @@ public:
   // copies one layer's K or V cache, [heads, maxlen, head_dim] fp16 bits
   absl::Status read_kv_cache (size_t layer, bool value,
                               std::vector<uint16_t> &out);
+  // A testing aid, the mirror of read_kv_cache: replaces one layer's K or V
+  // cache with n = heads * maxlen * head_dim fp16 values, so that a test can
+  // put a model at a late position without running the prompt that leads
+  // there (the reference fills its caches only through
+  // src/ops/update_kv_cache.cpp).
+  absl::Status write_kv_cache (size_t layer, bool value, const uint16_t *rows,
+                               size_t n);
   GPUDevice *device () { return gpu_; }
   size_t vocab_size () const { return vocab_; }
   size_t context_length () const { return maxlen_; }
