@@ -436,9 +436,9 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
     ps.lane = threadIdx.x & 63, ps.wave = threadIdx.x >> 6, ps.wg = wg;
     const int U = mode == 0 ? (N + R - 1) / R : (mode == 1 ? 3 * (N >> 1) : N);
     int lo, hi;
-    // (64 fp16 results per line; owned dealing serves the one-row units of
-    // mode 0 and the pair units of mode 2, whose unit is one result)
-    dealt_units (dl, U, 64, wg, G, lo, hi);
+    // (64 fp16 results per line: 32 two-row units of mode 0, 64 units
+    // otherwise; owned dealing serves mode 0 and the pair units of mode 2)
+    dealt_units (dl, U, mode == 0 && R == 2 ? 32 : 64, wg, G, lo, hi);
     ps.u_lo = lo + ps.wave;
     ps.U = U;
     const int nunits
@@ -624,9 +624,9 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
         h1 = f2h (h2f (h1) + h2f ((uint16_t)(rr >> 16)));
       }
     if (two)
-      stg ((uint32_t *)(e.y[0] + r0), (uint32_t)h0 | ((uint32_t)h1 << 16));
+      st_h2 (e, (uint32_t *)(e.y[0] + r0), (uint32_t)h0 | ((uint32_t)h1 << 16));
     else
-      stg (e.y[0] + r0, h0);
+      st_h (e, e.y[0] + r0, h0);
     if (e.y32)
       {
         stg (e.y32 + r0, h2f (h0));
@@ -639,6 +639,26 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
           ps.best_v = h2f (h0), ps.best_i = (uint32_t)r0;
         if (two && better (h2f (h1), (uint32_t)r0 + 1, ps.best_v, ps.best_i))
           ps.best_v = h2f (h1), ps.best_i = (uint32_t)r0 + 1;
+      }
+  }
+
+  // All items through ONE buffer (the other one may hold an item of the next
+  // phase): the first item is in flight in A (begin with depth 1), later
+  // items are requested when A is free.  For phases whose waves have one
+  // item, seldom two.
+  static __device__ __forceinline__ void
+  run_single (PipeState &ps, PipeBuf &A, const uint16_t *xl, const Epilogue &e)
+  {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      acc[r] = 0.f;
+    const int nit = ps.nit;
+    for (int it = 0; it < nit; ++it)
+      {
+        consume (ps, acc, A, it, xl, e);
+        if (it + 1 < nit)
+          issue (ps, A, it + 1);
       }
   }
 

@@ -76,6 +76,15 @@ constexpr int kCourier = kDecWaves - 1;
 #define VKL_LAYER_AHEAD 2
 #endif
 constexpr int kAhead = VKL_LAYER_AHEAD;
+// The first up/gate item of a wave is requested when the attention output has
+// arrived (0) or already together with the Wo item, while the heads are being
+// computed (1).  The early request fills the memory's idle time, but the
+// heads share compute units with workgroups that request, and a compute
+// unit's memory path is served in order: their polls and cache rows queue
+// behind those items.
+#ifndef VKL_LAYER_UP_EARLY
+#define VKL_LAYER_UP_EARLY 1
+#endif
 #define VKL_LDS __attribute__ ((address_space (3)))
 
 enum Stage
@@ -131,11 +140,20 @@ template <bool COURIER>
 __device__ __forceinline__ bool
 courier_fetch (bool poll, const uint32_t *flag, int nflags, uint32_t mark, int limit,
                uint32_t *err, uint32_t *lds_word, uint32_t code, const uint16_t *src, int K,
-               uint8_t *xl, unsigned long long *tr = nullptr)
+               uint8_t *xl, const float *norm_w = nullptr, int norm_n = 0, uint8_t *norm_lds = nullptr,
+               unsigned long long *tr = nullptr)
 {
   if (COURIER)
     {
       const int lane = (int)threadIdx.x & 63;
+      // (norm weights do not depend on anybody: they travel while this wave polls)
+      if (norm_w)
+        for (int i = 0; i < (norm_n * 4 + 1023) >> 10; ++i)
+          {
+            const int off = min (i * 1024 + lane * 16, norm_n * 4 - 16);
+            __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)((const uint8_t *)norm_w + off),
+                                              (VKL_LDS void *)(norm_lds + i * 1024), 16, 0, 0);
+          }
       bool ok = !poll;
       if (poll)
         {
@@ -164,8 +182,8 @@ courier_fetch (bool poll, const uint32_t *flag, int nflags, uint32_t mark, int l
               __builtin_amdgcn_global_load_lds ((const VKL_GLOBAL void *)((const uint8_t *)src + off),
                                                 (VKL_LDS void *)(xl + i * 1024), 16, 0, 0);
             }
-          __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
         }
+      __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
 #ifdef VKL_TRACE
       if (tr && lane == 0)
         tr[1] = wall_clock64 ();
@@ -211,6 +229,20 @@ wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t
   return *lds_word != 0u;
 }
 
+// norm weights as the courier left them in LDS
+template <int XCH>
+__device__ __forceinline__ void
+norm_from_lds (const uint8_t *nl, int K, NormRegs &n)
+{
+#pragma unroll
+  for (int j = 0; j < XCH; ++j)
+    {
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
+      n.w[j][0] = ((const uint4 *)nl)[2 * idx];
+      n.w[j][1] = ((const uint4 *)nl)[2 * idx + 1];
+    }
+}
+
 // the row as the courier left it in LDS, into the registers stage_row expects
 template <int XCH>
 __device__ __forceinline__ void
@@ -254,12 +286,22 @@ flag_of (const LayerCtx &c, int stage, int k)
 
 // A layer from the attention on, for the workers (COURIER false) or for the
 // courier of the workgroup: the same barriers in the same order in both.
+//
+// The two item buffers are handed from phase to phase so that the memory has
+// work during the attention and no wave waits for a third up/gate item with
+// nothing else to do: the Wo projection takes two-row units (a wave then has
+// one item, rarely two) and runs them through buffer A alone; buffer B
+// receives the wave's FIRST up/gate item together with the Wo item, i.e.
+// while the heads are computed and the memory would otherwise idle; A takes
+// the second up/gate item as soon as the Wo product has left it.  When the
+// residual row arrives both are there, and the third item travels while the
+// second is multiplied.
 template <int WT, int XD, int XF, bool NT, bool COURIER>
 __device__ __forceinline__ void
 layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uint8_t *lds)
 {
   typedef Gemv<WT, NT, 2> GV2;    // up/gate: two-row units
-  typedef Gemv<WT, false, 1> GVO; // Wo: one-row units, plain loads (short phase)
+  typedef Gemv<WT, false, 2> GVO; // Wo: two-row units, plain loads (short phase)
   typedef Gemv<WT, NT, 1> GVD;    // down
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn, wg = c.wg, G = c.G, slot = c.slot, idx = c.idx;
@@ -270,73 +312,89 @@ layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uin
   Epilogue e = {};
   XRegs x;
   NormRegs nw;
-  PipeState ps;
+  PipeState ps, pu; // pu: the up/gate product, begun during the Wo phase
   PipeBuf A, B;
+  const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
+  const Deal deal_up = Deal{ 1, slot, idx, c.n_slot };
+  // where the norm weights of the up/gate phase are parked (behind the staged
+  // row and the reduction words)
+  uint8_t *norm_lds = lds + lds_norm_offset (dim, ffn);
   // heads h = slot, slot + 8, ... run on the first workgroups of XCD `slot`
   const int n_heads_here = (c.nh - slot + 7) >> 3;
   if (idx < n_heads_here)
     {
       // ---- one head of the attention ---------------------------------------
-      live = wait_flags (flag_of (c, ST_KQV, 0), 8, c.mark, c.limit, c.err, c.word, 0x100u | ST_KQV);
-      VKL_TL (4)
-      if (live)
-        {
-          if (m.head_dim == 128)
-            attention_head<128, true> (p, lw, idx * 8 + slot, lds, nullptr);
-          else
-            attention_head<64, true> (p, lw, idx * 8 + slot, lds, nullptr);
-        }
+      // (the cached K and V rows are requested before the wait for this
+      // token's q, k and v: they do not depend on it)
+      auto wait_kqv = [&] () {
+        live = wait_flags (flag_of (c, ST_KQV, 0), 8, c.mark, c.limit, c.err, c.word, 0x100u | ST_KQV);
+        VKL_TL (4)
+        return live;
+      };
+      if (m.head_dim == 128)
+        attention_head<128, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv);
+      else
+        attention_head<64, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv);
       VKL_TL (5)
       arrive (cnt_of (c, ST_ATT, 0), (uint32_t)c.nh, flag_of (c, ST_ATT, 0), 8, c.mark, c.silent);
+      arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
+      VKL_TL (6)
+      if (!COURIER)
+        GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_up);
     }
   else
     {
       // ---- Wo + residual -> xm ---------------------------------------------
       const QMat w = wmat<WT> (lw.wo, dim, dim);
-      float *red = (float *)(lds + (size_t)dim * 2);
       const Deal dl = Deal{ 1, slot, idx - n_heads_here, c.n_slot - n_heads_here };
       if (!COURIER)
-        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, kAhead, p.s.x, true, dl);
+        {
+          GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x, true, dl);
+          if (VKL_LAYER_UP_EARLY)
+            GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_up);
+        }
       live = courier_fetch<COURIER> (c.first == 0, flag_of (c, ST_ATT, slot), 1, c.mark, c.limit,
-                                     c.err, c.word, 0x100u | ST_ATT, p.s.att, dim, lds);
+                                     c.err, c.word, 0x100u | ST_ATT, p.s.att, dim, lds, lw.ffn_norm,
+                                     dim, norm_lds);
       if (COURIER)
-        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 2, p.s.x, true, dl);
-      else if (kAhead < 2)
-        GVO::issue (ps, B, 1), ps.primed = 2;
+        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x, true, dl);
+      else if (!VKL_LAYER_UP_EARLY)
+        GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_up);
       VKL_TL (4)
       e = Epilogue{};
       e.y[0] = live ? p.s.xm : p.s.sink, e.residual = p.s.x;
       e.through = true;
-      GVO::run (ps, A, B, xl, e, red);
+      GVO::run_single (ps, A, xl, e);
       VKL_TL (5)
+      arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
+      VKL_TL (6)
+      // (after the arrival: it waits for everything the wave has in flight)
+      if (!COURIER)
+        GV2::issue (pu, A, 1), pu.primed = 2;
     }
-  arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
-  VKL_TL (6)
 
   // ---- RMSNorm + up/gate with SiLU -> t -------------------------------------
   {
-    const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
     float *red = (float *)(lds + (size_t)dim * 2);
-    load_norm<XD> (lw.ffn_norm, dim, nw);
-    __builtin_amdgcn_sched_barrier (0);
-    const Deal dl = Deal{ 1, slot, idx, c.n_slot };
-    if (!COURIER)
-      GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, kAhead, nullptr, true, dl);
+    // (a head's workgroup had its LDS in use until now: it fetches the norm weights here)
+    const bool head = idx < n_heads_here;
     live = courier_fetch<COURIER> (true, flag_of (c, ST_WO, 0), 8, c.mark, c.limit, c.err, c.word,
-                                   0x100u | ST_WO, p.s.xm, dim, lds)
+                                   0x100u | ST_WO, p.s.xm, dim, lds, head ? lw.ffn_norm : nullptr, dim,
+                                   norm_lds)
            && live;
-    if (COURIER)
-      GV2::begin (ps, A, B, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, dl);
-    else if (kAhead < 2)
-      GV2::issue (ps, B, 1), ps.primed = 2;
     VKL_TL (7)
+    norm_from_lds<XD> (norm_lds, dim, nw);
     row_from_lds<XD> (xl, dim, x);
     stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
     VKL_TL (8)
+    // (the courier's requests come after the barriers of the staging: a wave
+    // that waits for room in the memory path would hold up the other seven)
+    if (COURIER)
+      GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_up);
     e = Epilogue{};
     e.y[0] = live ? p.s.t : p.s.sink;
     e.through = true;
-    GV2::run (ps, A, B, xl, e, red);
+    GV2::run (pu, B, A, xl, e, red);
     VKL_TL (9)
     arrive (cnt_of (c, ST_UP, slot), (uint32_t)c.n_slot, flag_of (c, ST_UP, slot), 1, c.mark, false);
     VKL_TL (10)
@@ -445,6 +503,13 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       __syncthreads ();
       place ();
     }
+#ifdef VKL_TRACE
+  if (threadIdx.x == 0 && p.trace)
+    {
+      p.trace[((size_t)layer * 1024 + wg) * 16 + 12] = __builtin_amdgcn_s_getreg (4 | (0 << 6) | (31 << 11));
+      p.trace[((size_t)layer * 1024 + wg) * 16 + 14] = (unsigned)idx | (unsigned)slot << 16;
+    }
+#endif
   const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, first, wg, G, layer, silent };
   // the courier's path is a copy of the workers' (the branch is wave-uniform):
   // in one copy, with the courier's weight requests under a condition, the

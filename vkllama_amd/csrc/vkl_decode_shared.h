@@ -177,10 +177,18 @@ struct PipeBuf
 // ---------------------------------------------------------------------------
 // LDS use: qk[3*HD] fp16 (rotated q, rotated k, v), sc[maxlen] fp32,
 // part[RPB][HD] fp32, red[2*kDecWaves].
-template <int HD, bool COH>
+struct NoWait
+{
+  __device__ __forceinline__ bool operator() () const { return true; }
+};
+
+// EARLY: the cached rows are requested first, then `wait` is called (it waits
+// for the producers of this token's q, k and v inside the same launch; false:
+// give up, nothing is stored), then q, k and v are read.
+template <int HD, bool COH, bool EARLY = false, typename Wait = NoWait>
 __device__ __forceinline__ void
 attention_head (const Params &p, const vkl_layer_weights &lw, int head,
-                uint8_t *lds, unsigned long long *tr = nullptr)
+                uint8_t *lds, unsigned long long *tr = nullptr, Wait wait = Wait ())
 {
 #ifdef VKL_TRACE
 #define VKL_TRA(slot)                                                         \
@@ -217,12 +225,16 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   const bool is_q = tid < HD / 2, is_k = !is_q && tid < HD;
   const bool is_v = tid >= HD && tid < HD + HD / 2;
   const int pi = is_q ? tid : (is_k ? tid - HD / 2 : (is_v ? tid - HD : 0));
-  const uint32_t inw
-      = ld_u32<COH> ((const uint32_t *)(is_k ? kin : (is_v ? vin : qin)) + pi);
-  const float fc = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
-  const float fs = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
-  // (the scheduler must not move the cache rows ahead of these)
-  __builtin_amdgcn_sched_barrier (0);
+  uint32_t inw = 0;
+  float fc = 0.f, fs = 0.f;
+  if (!EARLY)
+    {
+      inw = ld_u32<COH> ((const uint32_t *)(is_k ? kin : (is_v ? vin : qin)) + pi);
+      fc = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
+      fs = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
+      // (the scheduler must not move the cache rows ahead of these)
+      __builtin_amdgcn_sched_barrier (0);
+    }
   uint4 kpre[PRE], vpre[PRE];
   const int lastrow = max ((int)pos - 1, 0);
 #pragma unroll
@@ -232,6 +244,14 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   for (int j = 0; j < PRE; ++j)
     vpre[j] = ldg4 (vc + (size_t)min (grp + j * RPB, lastrow) * HD + sub * 8);
   __builtin_amdgcn_sched_barrier (0);
+  if (EARLY)
+    {
+      fc = ldg (p.m.freqc + (size_t)pos * (HD / 2) + pi);
+      fs = ldg (p.m.freqs + (size_t)pos * (HD / 2) + pi);
+      if (!wait ())
+        return;
+      inw = ld_u32<COH> ((const uint32_t *)(is_k ? kin : (is_v ? vin : qin)) + pi);
+    }
 
   // RoPE on adjacent pairs at position pos.  The new K and V rows are used
   // from LDS here; they go to the cache at the end of the head (a store
@@ -394,12 +414,20 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
     stg ((uint32_t *)(vc + (size_t)pos * HD) + pi, inw);
 }
 
+// where norm weights are parked in LDS: behind the staged row (whole KiB: a
+// row fetched straight into LDS fills its last KiB) and the reduction words
+__host__ __device__ inline size_t
+lds_norm_offset (int dim, int ffn)
+{
+  const size_t kmax = (size_t)(dim > ffn ? dim : ffn);
+  return ((kmax * 2 + 1023) & ~(size_t)1023) + 256;
+}
+
 __host__ __device__ inline size_t
 lds_bytes_needed (int dim, int ffn, int maxlen, int hd)
 {
-  const size_t kmax = (size_t)(dim > ffn ? dim : ffn);
-  // staged activation row + reduction words + parked norm weights
-  const size_t stage = ((kmax + 31) / 32 * 32) * 2 + 256 + (size_t)dim * 4;
+  // staged activation row + reduction words + parked norm weights (whole KiB)
+  const size_t stage = lds_norm_offset (dim, ffn) + (((size_t)dim * 4 + 1023) & ~(size_t)1023);
   const size_t rpb = kDecThreads / (hd / 8);
   const size_t attn = 1024 + (size_t)((maxlen + 3) & ~3) * 4 + rpb * hd * 4 + 256;
   return stage > attn ? stage : attn;
