@@ -255,7 +255,7 @@ class Llama2:
     def decode_step_bytes(self, L):
         return int(lib().vkl_model_decode_step_bytes(self._h, L))
 
-    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax", "unused", "layer")
+    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax", "unused", "layer", "layers")
 
     def phase_times(self):
         """{phase: (milliseconds summed, launches)} since the last call; filled
