@@ -240,11 +240,9 @@ def main():
     per_phase = {}
     for name, (ms, n) in phases.items():
         if n:
-            # (mode 2: the "layer" timing slot holds ONE launch with all layers)
-            key = "layers" if name == "layer" and n // steps == 1 and cfg["n_layers"] > 1 else name
-            per_phase[key] = {"launches_per_step": n // steps, "avg_us": round(ms * 1e3 / n, 3),
-                              "us_per_step": round(ms * 1e3 / steps, 1),
-                              "bytes_per_launch": m.phase_bytes(key, L_mid)}
+            per_phase[name] = {"launches_per_step": n // steps, "avg_us": round(ms * 1e3 / n, 3),
+                               "us_per_step": round(ms * 1e3 / steps, 1),
+                               "bytes_per_launch": m.phase_bytes(name, L_mid)}
     if "attention" in per_phase and "wo" not in per_phase and phases.get("wo", (0, 0))[1] == 0:
         # short contexts: the attention phase and the Wo projection are one launch
         fused = per_phase.pop("attention")
@@ -266,18 +264,17 @@ def main():
         # the kernel's name as a profiler prints it: phase number, weight type,
         # 4096-value chunks of the staged activation row
         phase_no = {"kqv": 0, "attention": 1, "attention+wo": 1, "wo": 2, "upgate": 3, "down": 4, "lm_head": 5,
-                    "layer": 8, "layers": 9}[dom]
+                    "layer": 8}[dom]
         kstage = cfg["ffn"] if dom == "down" else cfg["dim"]
         per = 34.0 / 32.0 if cfg["wtype"] == 8 else 2.0
         wbytes = (cfg["n_layers"] * (4.0 * cfg["dim"] ** 2 + 3.0 * cfg["dim"] * cfg["ffn"])
                   + cfg["vocab"] * cfg["dim"]) * per
-        if dom in ("layer", "layers"):
+        if dom == "layer":
             # (row chunks of 4096 values as the library picks them: see launch_layer_wt)
             xd, xf = (cfg["dim"] + 4095) // 4096, (cfg["ffn"] + 4095) // 4096
             xd, xf = (1, 1) if (xd, xf) == (1, 1) else ((1, 3) if xd == 1 and xf <= 3 else (2, 4))
-            dom_kernel = "decode_layer_kernel<%d, %d, %d, %s> (%s)" % (
-                8 if cfg["wtype"] == 8 else 1, xd, xf, "true" if wbytes > (288 << 20) else "false",
-                "the five phases of a layer in one launch" if dom == "layer" else "all layers of a token in one launch")
+            dom_kernel = "decode_layer_kernel<%d, %d, %d, %s> (the five phases of a layer in one launch)" % (
+                8 if cfg["wtype"] == 8 else 1, xd, xf, "true" if wbytes > (288 << 20) else "false")
         elif dom == "attention+wo":
             dom_kernel = "decode_attn_wo_kernel<%d, %d> (attention + Wo)" % (8 if cfg["wtype"] == 8 else 1,
                                                                             min(4, (cfg["dim"] + 4095) // 4096))
@@ -321,8 +318,7 @@ def main():
         "data": "synthetic: random-init N(0,0.02) weights" + (" quantised to Q8_0" if cfg["wtype"] == 8 else " in FP16")
                 + ", random prompt ids",
         "config": {"workload": args.workload, "prompt_tokens": n_prompt, "decode_tokens": steps,
-                   "decode_mode": ("one launch per phase", "one launch per layer",
-                                   "one launch for all layers")[args.decode_mode]
+                   "decode_mode": ("one launch per phase", "one launch per layer")[args.decode_mode]
                                   + (", replayed from a HIP graph" if args.decode_graph else ""),
                    "dims": {k: cfg[k] for k in ("dim", "n_layers", "n_heads", "ffn", "vocab", "maxlen")}},
         "decode_tokens_per_second_host_interface": round(host_tok_s, 1),

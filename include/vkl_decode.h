@@ -75,11 +75,10 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
  *           memory with bounded waits for one another, and have the next
  *           phase's weights on the way meanwhile (above the split length:
  *           K/Q/V, split attention, then Wo + up/gate + down in one
- *           launch); 2 = as 1, with ALL layers of a token in one launch
- *           below the split length.  Results are bit for bit those of mode 0.
- *           Models whose rows the one-launch form does not cover run as
- *           mode 0.  The GPU must not be shared while such a launch runs:
- *           see vkl_decode_status
+ *           launch).  Results are bit for bit those of mode 0.  Models whose
+ *           rows the one-launch form does not cover run as mode 0.  The GPU
+ *           must not be shared while such a launch runs: see
+ *           vkl_decode_status
  *  logits32 optional device fp32 [vocab]: widened fp16 logits
  *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
  * Returns 0 or a hipError_t; hipErrorInvalidValue for shapes the kernels do
@@ -127,17 +126,15 @@ int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
  * phase launch with a pair of HIP events on the launch stream and
  * synchronises the stream before it returns.  vkl_decode_phase_times adds up,
  * per phase kind (0 K/Q/V, 1 attention, 2 Wo, 3 up/gate, 4 down, 5 lm_head,
- * 6 arg-max, 8 a whole layer in one launch as mode 1 runs it, or all layers
- * in one as mode 2 does; 7 and 9 are not used), the elapsed milliseconds and
- * the number of launches since the last call, and clears both. */
-#define VKL_DECODE_PHASES 10
-#define VKL_DECODE_PHASE_LAYER 8  /* one layer in one launch */
-#define VKL_DECODE_PHASE_LAYERS 9 /* all layers in one launch (replay and bytes only) */
+ * 6 arg-max, 8 a whole layer in one launch as mode 1 runs it; 7 is not
+ * used), the elapsed milliseconds and the number of launches since the last
+ * call, and clears both. */
+#define VKL_DECODE_PHASES 9
+#define VKL_DECODE_PHASE_LAYER 8
 int vkl_decode_phase_timing (int enable);
 int vkl_decode_phase_times (double ms_sum[VKL_DECODE_PHASES],
                             uint64_t launches[VKL_DECODE_PHASES]);
-/* Launches phase `kind` (0..4 and 8: of every layer in turn; 5: lm_head; 9:
- * all layers as one launch, contexts below the split length only) `rounds`
+/* Launches phase `kind` (0..4 and 8: of every layer in turn; 5: lm_head) `rounds`
  * times back to back on `stream` between ONE pair of events and returns the
  * average milliseconds per launch: the kernel's duration without the cost of
  * an event pair per launch.  The phase's outputs in scratch are overwritten

@@ -72,8 +72,7 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
                                 uint32_t *out_ids_h, double *prefill_ms,
                                 double *decode_ms);
 /* options, all per model: "fused_decode" (fused one-token decode on/off),
- * "decode_mode" (0 = one launch per phase, 1 = one launch per layer, 2 = one
- * launch for all layers),
+ * "decode_mode" (0 = one launch per phase, 1 = one launch per layer),
  * "decode_graph" (replay of the greedy loop from a HIP graph on/off),
  * "attn_split_min" (the context length from which attention is split over
  * several workgroups per head), "fuse_attn_wo" (mode 0: attention and the Wo
@@ -101,7 +100,7 @@ int vkl_model_write_kv_cache (vkl_model *m, size_t layer, int value,
 size_t vkl_model_decode_step_bytes (const vkl_model *m, size_t L);
 /* per-phase measurements of the fused decode step: option "phase_timing"
  * switches them on; see vkl_decode_phase_times / vkl_decode_phase_bytes */
-int vkl_model_phase_times (vkl_model *m, double ms_sum[10], uint64_t launches[10]);
+int vkl_model_phase_times (vkl_model *m, double ms_sum[9], uint64_t launches[9]);
 size_t vkl_model_phase_bytes (const vkl_model *m, int kind, size_t L);
 /* vkl_decode_phase_replay on this model's stream; overwrites decode scratch */
 int vkl_model_phase_replay (vkl_model *m, int kind, size_t pos, int rounds,

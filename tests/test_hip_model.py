@@ -295,8 +295,7 @@ def test_layer_launch_decode_matches_oracle(cfg, seed):
                                  dict(dim=512, n_layers=3, n_heads=8, ffn=1376, vocab=2048, maxlen=128, eps=1e-5,
                                       wtype=1)])
 def test_layer_launch_equals_phase_launches(cfg):
-    """One launch per layer (mode 1) and one launch for all layers (mode 2)
-    against one launch per phase at the row widths of
+    """One launch per layer against one launch per phase at the row widths of
     the 7B and 13B shapes and with fp16 weights: greedy ids and the logits of a
     further step bit for bit, replayed from a graph and launched step by step
     (the launch-per-phase form is what the other tests hold against the
@@ -305,7 +304,7 @@ def test_layer_launch_equals_phase_launches(cfg):
     prompt = np.random.default_rng(3).integers(3, cfg["vocab"], 7).astype(np.uint32)
     m = M.Llama2(cfg, w)
     runs = {}
-    for mode in (0, 1, 2):
+    for mode in (0, 1):
         m.set_option("decode_mode", mode)
         for graph in (1, 0):
             m.set_option("decode_graph", graph)
@@ -330,7 +329,7 @@ def test_layer_launch_long_context_equals_phase_launches():
     m = M.Llama2(cfg, w)
     m.set_option("attn_split_min", 100)
     runs = {}
-    for mode in (0, 1, 2):
+    for mode in (0, 1):
         m.set_option("decode_mode", mode)
         for graph in (1, 0):
             m.set_option("decode_graph", graph)
@@ -423,7 +422,7 @@ def test_attention_and_wo_in_one_launch_equals_two_launches(cfg):
         assert np.array_equal(logits.view(np.uint32), ref_logits.view(np.uint32)), key
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("mode", [0, 1])
 def test_wait_inside_a_launch_is_bounded_and_recovered(mode):
     """Workgroups that wait for others inside a launch (the Wo projection for
     the attention heads, in the attention + Wo launch of mode 0 and in the

@@ -9,7 +9,9 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-HIP_LIB_PATH = os.path.join(_PKG, "lib", "libvkllama_hip.so")
+# VKL_LIB_DIR: another directory holding a build of both libraries (comparing two builds on one GPU)
+LIB_DIR = os.environ.get("VKL_LIB_DIR", os.path.join(_PKG, "lib"))
+HIP_LIB_PATH = os.path.join(LIB_DIR, "libvkllama_hip.so")
 
 vp = C.c_void_p
 sz = C.c_size_t

@@ -36,27 +36,8 @@ typedef _Float16 h16x2 __attribute__ ((ext_vector_type (2)));
 #define VKL_GLOBAL __attribute__ ((address_space (1)))
 typedef uint32_t vkl_u32x4 __attribute__ ((ext_vector_type (4)));
 
-// The thread's index inside its workgroup as the shared device code reads it.
-// A translation unit whose kernel loops over layers defines VKL_TID as
-// vkl::tid_opaque () before it includes these headers: every reader then gets
-// a copy the compiler cannot see through, so that nothing derived from it
-// counts as loop-invariant.  (Loop-invariant code motion would otherwise lift
-// the per-phase state of every phase of the loop body out of the loop, all of
-// it alive at once, and spill hundreds of bytes per lane.)
-#ifndef VKL_TID
-#define VKL_TID ((int)threadIdx.x)
-#endif
-
 namespace vkl
 {
-__device__ __forceinline__ int
-tid_opaque ()
-{
-  int t = (int)threadIdx.x;
-  asm volatile("" : "+v"(t));
-  return t;
-}
-
 // Loads and stores through pointers that were themselves read from memory
 // (e.g. a per-layer table of weight pointers) are FLAT accesses unless the
 // address space is stated: a flat load also counts against the LDS counter,

@@ -71,8 +71,7 @@ enum Phase
   PH_HEAD,
   PH_ARGMAX,
   PH_GEMV, // a stand-alone y = W x (+ residual) on the down projection's path
-  PH_LAYER, // a whole layer in one launch (vkl_decode_layer.hip)
-  PH_LAYERS // all layers in one launch
+  PH_LAYER // a whole layer in one launch (vkl_decode_layer.hip)
 };
 
 // ---------------------------------------------------------------------------
@@ -993,66 +992,34 @@ int
 launch_step (const Params &p, const vkl_decode_model *m, int mode, int n_cu, int G,
              size_t lds, hipStream_t s)
 {
-  const bool fused = mode >= 1 && layer_launch_supported (*m, G);
+  const bool per_layer = mode == 1 && layer_launch_supported (*m, G);
   const bool short_ctx = (int)p.pos + 1 < attn_split_min (*m);
-  if (fused && short_ctx && mode == 1)
+  if (per_layer)
+    if (int e = launch_embed_row (p, s))
+      return e;
+  for (int l = 0; l < m->n_layers; ++l)
     {
-      // one launch per layer, on the rows of the launch-per-phase kernels
-      if (int e = launch_embed_row (p, s))
-        return e;
-      for (int l = 0; l < m->n_layers; ++l)
+      const vkl_layer_weights &lw = m->layers_h[l];
+      if (per_layer && short_ctx)
         {
           if (int e = timer_mark (PH_LAYER, false, s))
             return e;
-          if (int e = launch_layers (p, l, l + 1, 0, 0, G, s))
+          if (int e = launch_layer (p, lw, l, 0, G, s))
             return e;
           if (int e = timer_mark (PH_LAYER, true, s))
             return e;
+          continue;
         }
-    }
-  else if (fused && short_ctx)
-    {
-      // all layers in one launch, on rows of their own: the embedding row is
-      // layer 0's input, the output layer reads what the last layer leaves
-      Params q = p;
-      q.s.x = p.s.lx;
-      if (int e = launch_embed_row (q, s))
-        return e;
-      if (int e = timer_mark (PH_LAYER, false, s))
-        return e;
-      if (int e = launch_layers (p, 0, m->n_layers, 0, 1, G, s))
-        return e;
-      if (int e = timer_mark (PH_LAYER, true, s))
-        return e;
-      q.s.x = p.s.lx + (size_t)m->n_layers * m->dim;
-      const vkl_layer_weights none = {};
-      if (int e = launch_phase<PH_HEAD> (q, none, 0, G, G, lds, s))
-        return e;
-      if (p.next_tok || p.loop)
-        if (int e = launch_phase<PH_ARGMAX> (q, none, 0, 1, G, lds, s))
-          return e;
-      return 0;
-    }
-  else if (fused)
-    {
-      if (int e = launch_embed_row (p, s))
-        return e;
-    }
-  for (int l = 0; l < m->n_layers && !(fused && short_ctx); ++l)
-    {
-      const vkl_layer_weights &lw = m->layers_h[l];
       // (with the embedding row in place, layer 0 is a layer like the others)
-      if (int e = launch_phase<PH_KQV> (p, lw, fused ? std::max (l, 1) : l, G, G, lds, s))
+      if (int e = launch_phase<PH_KQV> (p, lw, per_layer ? std::max (l, 1) : l, G, G, lds, s))
         return e;
-      if (fused)
+      if (per_layer)
         {
-          // long contexts: K/Q/V, the split attention, then the rest of the
-          // layer in one launch
           if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
             return e;
           if (int e = timer_mark (PH_LAYER, false, s))
             return e;
-          if (int e = launch_layers (p, l, l + 1, 1, 0, G, s))
+          if (int e = launch_layer (p, lw, l, 1, G, s))
             return e;
           if (int e = timer_mark (PH_LAYER, true, s))
             return e;
@@ -1138,7 +1105,7 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (int e = check_model (m))
     return e;
   VKL_CHECK_ARG (tok != nullptr && pos < (uint32_t)m->maxlen);
-  VKL_CHECK_ARG (mode >= 0 && mode <= 2);
+  VKL_CHECK_ARG (mode >= 0 && mode <= 1);
   static int n_cu = 0;
   if (n_cu == 0)
     {
@@ -1254,7 +1221,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
 {
   if (int e = check_model (m))
     return e;
-  VKL_CHECK_ARG (mode >= 0 && mode <= 2);
+  VKL_CHECK_ARG (mode >= 0 && mode <= 1);
   VKL_CHECK_ARG (ids != nullptr && n_steps >= 0);
   VKL_CHECK_ARG ((uint64_t)pos0 + (uint64_t)n_steps <= (uint64_t)m->maxlen);
   if (n_steps == 0)
@@ -1372,9 +1339,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
 {
   if (int e = check_model (m))
     return e;
-  VKL_CHECK_ARG (((kind >= PH_KQV && kind <= PH_HEAD) || kind == PH_LAYER || kind == PH_LAYERS) && rounds > 0
-                 && avg_ms);
-  VKL_CHECK_ARG (kind != PH_LAYERS || (int)pos + 1 < attn_split_min (*m));
+  VKL_CHECK_ARG (((kind >= PH_KQV && kind <= PH_HEAD) || kind == PH_LAYER) && rounds > 0 && avg_ms);
   VKL_CHECK_ARG (pos < (uint32_t)m->maxlen);
   int dev = 0, n_cu = 0;
   VKL_HIP (hipGetDevice (&dev));
@@ -1394,7 +1359,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;
-  VKL_CHECK_ARG ((kind != PH_LAYER && kind != PH_LAYERS) || layer_launch_supported (*m, G));
+  VKL_CHECK_ARG (kind != PH_LAYER || layer_launch_supported (*m, G));
   const bool was_on = g_timer.on;
   g_timer.on = false;
   hipEvent_t e0, e1;
@@ -1409,11 +1374,6 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
         {
           const vkl_layer_weights none = {};
           err = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s), ++n;
-          continue;
-        }
-      if (kind == PH_LAYERS)
-        {
-          err = launch_layers (p, 0, m->n_layers, 0, 1, G, s), ++n;
           continue;
         }
       for (int l = 0; l < m->n_layers && !err; ++l, ++n)
@@ -1437,7 +1397,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
               err = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s);
               break;
             case PH_LAYER:
-              err = launch_layers (p, l, l + 1, (int)pos + 1 < attn_split_min (*m) ? 0 : 1, 0, G, s);
+              err = launch_layer (p, lw, l, (int)pos + 1 < attn_split_min (*m) ? 0 : 1, G, s);
               break;
             default:
               err = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s);
@@ -1488,18 +1448,10 @@ vkl_decode_phase_bytes (const vkl_decode_model *m, int kind, size_t L)
       return mat (dim, ffn) + ffn * 2 + 2 * dim * 2;
     case PH_HEAD:
       return mat (V, dim) + dim * 2 + dim * 4 + V * 2 + V * 4;
-    case PH_LAYER:
-    case PH_LAYERS:
-      {
-        // the five phases of a layer, each handed-over row written and read
-        // once; above the split length the launch holds Wo, up/gate and down
-        const size_t tail = vkl_decode_phase_bytes (m, PH_WO, L) + vkl_decode_phase_bytes (m, PH_UPGATE, L)
-                            + vkl_decode_phase_bytes (m, PH_DOWN, L);
-        if ((int)L >= attn_split_min (*m))
-          return tail;
-        return (size_t)(kind == PH_LAYERS ? m->n_layers : 1)
-               * (vkl_decode_phase_bytes (m, PH_KQV, L) + vkl_decode_phase_bytes (m, PH_ATTN, L) + tail);
-      }
+    case PH_LAYER: // the five phases; each handed-over row is written and read once
+      return vkl_decode_phase_bytes (m, PH_KQV, L) + vkl_decode_phase_bytes (m, PH_ATTN, L)
+             + vkl_decode_phase_bytes (m, PH_WO, L) + vkl_decode_phase_bytes (m, PH_UPGATE, L)
+             + vkl_decode_phase_bytes (m, PH_DOWN, L);
     default:
       return (size_t)1024 * 8;
     }

@@ -33,7 +33,7 @@ issue_x (const uint16_t *src, int K, XRegs &x)
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     {
-      const int idx = VKL_TID + j * kDecThreads;
+      const int idx = threadIdx.x + j * kDecThreads;
       x.v[j] = make_uint4 (0, 0, 0, 0);
       if (idx * 8 < K)
         x.v[j] = ldg4 (src + idx * 8);
@@ -48,7 +48,7 @@ issue_embed_q8 (const QMat tab, size_t row, int K, XRegs &x)
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     {
-      const int idx = VKL_TID + j * kDecThreads;
+      const int idx = threadIdx.x + j * kDecThreads;
       x.v[j] = make_uint4 (0, 0, 0, 0);
       if (idx * 8 < K)
         {
@@ -88,7 +88,7 @@ issue_norm (const float *w, int K, NormRegs &n)
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     {
-      const int idx = VKL_TID + j * kDecThreads;
+      const int idx = threadIdx.x + j * kDecThreads;
       n.w[j][0] = n.w[j][1] = make_uint4 (0, 0, 0, 0);
       if (idx * 8 < K)
         {
@@ -107,7 +107,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 {
   float alpha = 0.f;
 #ifdef VKL_TRACE
-  if (tr && VKL_TID == 0)
+  if (tr && threadIdx.x == 0)
     {
       // x has arrived once its first word can be read
       asm volatile("" ::"v"(x.v[0].x), "v"(x.v[3].w));
@@ -120,7 +120,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         {
-          const bool in = (int)(VKL_TID + j * kDecThreads) * 8 < K;
+          const bool in = (int)(threadIdx.x + j * kDecThreads) * 8 < K;
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -133,7 +133,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
         }
       const float total = block_sum (s, red);
 #ifdef VKL_TRACE
-      if (tr && VKL_TID == 0)
+      if (tr && threadIdx.x == 0)
         tr[3] = wall_clock64 ();
 #endif
       alpha = 1.0f / sqrtf (total / (float)K + eps);
@@ -141,7 +141,7 @@ finish_x (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     {
-      const int idx = VKL_TID + j * kDecThreads;
+      const int idx = threadIdx.x + j * kDecThreads;
       if (idx * 8 >= K)
         continue;
       uint4 o = x.v[j];
@@ -182,7 +182,7 @@ load_row (const uint16_t *src, int K, XRegs &x)
 #pragma unroll
   for (int j = 0; j < XCH; ++j)
     {
-      const int idx = min (VKL_TID + j * kDecThreads, (K >> 3) - 1);
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
       x.v[j] = ldg4 (src + idx * 8);
     }
 }
@@ -194,7 +194,7 @@ load_norm (const float *w, int K, NormRegs &n)
 #pragma unroll
   for (int j = 0; j < XCH; ++j)
     {
-      const int idx = min (VKL_TID + j * kDecThreads, (K >> 3) - 1);
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
       n.w[j][0] = ldg4 (w + idx * 8);
       n.w[j][1] = ldg4 (w + idx * 8 + 4);
     }
@@ -207,7 +207,7 @@ stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 {
   float alpha = 0.f;
 #ifdef VKL_TRACE
-  if (tr && VKL_TID == 0)
+  if (tr && threadIdx.x == 0)
     {
       asm volatile("" ::"v"(x.v[0].x), "v"(x.v[XCH - 1].w));
       tr[1] = wall_clock64 ();
@@ -219,7 +219,7 @@ stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
       for (int j = 0; j < XCH; ++j)
         {
-          const bool in = (int)(VKL_TID + j * kDecThreads) * 8 < K;
+          const bool in = (int)(threadIdx.x + j * kDecThreads) * 8 < K;
           const uint32_t w[4] = { x.v[j].x, x.v[j].y, x.v[j].z, x.v[j].w };
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -232,7 +232,7 @@ stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
         }
       const float total = block_sum (s, red);
 #ifdef VKL_TRACE
-      if (tr && VKL_TID == 0)
+      if (tr && threadIdx.x == 0)
         tr[3] = wall_clock64 ();
 #endif
       alpha = 1.0f / sqrtf (total / (float)K + eps);
@@ -240,7 +240,7 @@ stage_row (const XRegs &x, int K, uint16_t *xl, const NormRegs &n, float eps,
 #pragma unroll
   for (int j = 0; j < XCH; ++j)
     {
-      const int idx = min (VKL_TID + j * kDecThreads, (K >> 3) - 1);
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
       uint4 o = x.v[j];
       if (NORM)
         {
@@ -419,13 +419,8 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
   begin (PipeState &ps, PipeBuf &A, PipeBuf &B, int mode, const QMat a,
          const QMat b, const QMat c, int N, int K, int wg, int G, int depth,
          const uint16_t *residual = nullptr, bool always = false,
-         const Deal dl = Deal{ 0, 0, 0, 0 }, int tid = -1)
+         const Deal dl = Deal{ 0, 0, 0, 0 })
   {
-    // (tid: the caller's copy of VKL_TID; a loop over layers passes one
-    // the compiler cannot see through, or it would hoist the state of every
-    // phase out of the loop and run out of registers)
-    if (tid < 0)
-      tid = VKL_TID;
     ps.mode = mode;
     ps.residual = residual;
     ps.m0 = a;
@@ -438,7 +433,7 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
     else
       ps.Kp = K * 2, ps.nb = 0; // row bytes
     ps.nch = (ps.Kp + CHUNK - 1) / CHUNK;
-    ps.lane = tid & 63, ps.wave = tid >> 6, ps.wg = wg;
+    ps.lane = threadIdx.x & 63, ps.wave = threadIdx.x >> 6, ps.wg = wg;
     const int U = mode == 0 ? (N + R - 1) / R : (mode == 1 ? 3 * (N >> 1) : N);
     int lo, hi;
     // (64 fp16 results per line: 32 two-row units of mode 0, 64 units
@@ -702,7 +697,7 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
             bi[ps.wave] = ps.best_i;
           }
         __syncthreads ();
-        if (VKL_TID == 0)
+        if (threadIdx.x == 0)
           {
             float v = bv[0];
             uint32_t i = bi[0];

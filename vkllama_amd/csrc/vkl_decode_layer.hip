@@ -40,8 +40,6 @@
 // it in vain) and drops its results into a sink instead of storing them.  The
 // error word names the first cause: 0x100 | stage for a wait that gave
 // up, 0x200 | xcd for an XCD that was dealt more than its share of workgroups.
-// (see vkl_common.h: this kernel loops over layers)
-#define VKL_TID vkl::tid_opaque ()
 #include "vkl_decode_gemv.h"
 #include "vkl_decode_shared.h"
 #include <algorithm>
@@ -56,8 +54,8 @@ namespace
 // 128-byte line of its own
 constexpr int kLsLaunch = 0;              // launches completed so far
 constexpr int kLsCnt = 32;                // + (stage * 8 + slot) * 32
-constexpr int kLsFlag = 32 + 5 * 8 * 32;  // + (stage * 8 + slot) * 32
-constexpr int kLsTicket = kLsFlag + 5 * 8 * 32; // + slot * 32: workgroups of the XCD that have started
+constexpr int kLsFlag = 32 + 4 * 8 * 32;  // + (stage * 8 + slot) * 32
+constexpr int kLsTicket = kLsFlag + 4 * 8 * 32; // + slot * 32: workgroups of the XCD that have started
 static_assert ((kLsTicket + 8 * 32) * 4 <= kLayerSyncBytes, "layer-sync area too small");
 constexpr int kSyncErr = 1; // word of Scratch::sync: a wait gave up
 constexpr int kLayerSpinLimit = 1 << 14;
@@ -68,6 +66,16 @@ constexpr int kLayerSpinLimit = 1 << 14;
 // in, polls, brings the row into LDS, and only then streams its own (the
 // workgroup's last) units while the other waves are at their later items.
 constexpr int kCourier = kDecWaves - 1;
+// Weight items a worker requests before the wait for the previous phase.  The
+// memory path of a compute unit serves requests in order, also across waves:
+// the courier's polls and the row queue behind whatever the 14 workers of the
+// compute unit have requested, so the look-ahead is what the wait can hide
+// (one item: 116 KiB per compute unit, some 4 us at the rate a compute unit
+// is served), not everything the registers can hold.
+#ifndef VKL_LAYER_AHEAD
+#define VKL_LAYER_AHEAD 2
+#endif
+constexpr int kAhead = VKL_LAYER_AHEAD;
 // The first up/gate item of a wave is requested when the attention output has
 // arrived (0) or already together with the Wo item, while the heads are being
 // computed (1).  The early request fills the memory's idle time, but the
@@ -84,8 +92,7 @@ enum Stage
   ST_KQV = 0,
   ST_ATT,
   ST_WO,
-  ST_UP,
-  ST_DOWN
+  ST_UP
 };
 
 // the error word keeps the FIRST cause reported since the host last looked
@@ -106,9 +113,9 @@ arrive (uint32_t *cnt, uint32_t n, uint32_t *flag, int nflags, uint32_t mark, bo
   __syncthreads ();
   // (the courier counts in: the other waves go straight on to request the
   // next phase's weights instead of waiting for the counter's answer)
-  if (__builtin_amdgcn_readfirstlane ((int)(VKL_TID >> 6)) == kCourier)
+  if (__builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier)
     {
-      const int lane = VKL_TID & 63;
+      const int lane = (int)threadIdx.x & 63;
       uint32_t old = 0;
       if (lane == 0)
         old = __hip_atomic_fetch_add (cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -138,7 +145,7 @@ courier_fetch (bool poll, const uint32_t *flag, int nflags, uint32_t mark, int l
 {
   if (COURIER)
     {
-      const int lane = VKL_TID & 63;
+      const int lane = (int)threadIdx.x & 63;
       // (norm weights do not depend on anybody: they travel while this wave polls)
       if (norm_w)
         for (int i = 0; i < (norm_n * 4 + 1023) >> 10; ++i)
@@ -197,9 +204,9 @@ __device__ __forceinline__ bool
 wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t *err,
             uint32_t *lds_word, uint32_t code)
 {
-  if (VKL_TID < 64)
+  if (threadIdx.x < 64)
     {
-      const uint32_t *f = flag + 32 * (VKL_TID & (nflags - 1));
+      const uint32_t *f = flag + 32 * ((int)threadIdx.x & (nflags - 1));
       bool ok = false;
       for (int spin = 0; spin < limit; ++spin)
         {
@@ -211,7 +218,7 @@ wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t
             }
           __builtin_amdgcn_s_sleep (1);
         }
-      if (VKL_TID == 0)
+      if (threadIdx.x == 0)
         {
           *lds_word = ok ? 1u : 0u;
           if (!ok)
@@ -230,7 +237,7 @@ norm_from_lds (const uint8_t *nl, int K, NormRegs &n)
 #pragma unroll
   for (int j = 0; j < XCH; ++j)
     {
-      const int idx = min (VKL_TID + j * kDecThreads, (K >> 3) - 1);
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
       n.w[j][0] = ((const uint4 *)nl)[2 * idx];
       n.w[j][1] = ((const uint4 *)nl)[2 * idx + 1];
     }
@@ -244,7 +251,7 @@ row_from_lds (const uint16_t *xl, int K, XRegs &x)
 #pragma unroll
   for (int j = 0; j < XCH; ++j)
     {
-      const int idx = min (VKL_TID + j * kDecThreads, (K >> 3) - 1);
+      const int idx = min ((int)threadIdx.x + j * kDecThreads, (K >> 3) - 1);
       x.v[j] = ((const uint4 *)xl)[idx];
     }
 }
@@ -252,9 +259,9 @@ row_from_lds (const uint16_t *xl, int K, XRegs &x)
 struct LayerCtx
 {
   uint32_t *ls, *err, *word;
-  uint32_t mark0; // flags raised in layer l of this launch carry mark0 + l - l0
-  int limit, n_slot, slot, idx, nh, first, wg, G, l0, l1;
-  bool silent, own_rows;
+  uint32_t mark;
+  int limit, n_slot, slot, idx, nh, first, wg, G, layer;
+  bool silent;
 };
 
 __device__ __forceinline__ uint32_t *
@@ -269,52 +276,16 @@ flag_of (const LayerCtx &c, int stage, int k)
   return c.ls + kLsFlag + (stage * 8 + k) * 32;
 }
 
-// a record of the layer table in device memory, through scalar loads (a
-// vector load would queue behind the weight items in flight)
-__device__ __forceinline__ vkl_layer_weights
-layer_record (const vkl_layer_weights *tab, int l)
-{
-  typedef const __attribute__ ((address_space (4))) unsigned long long *cptr;
-  static_assert (sizeof (vkl_layer_weights) == 11 * 8, "eleven pointers");
-  cptr t = (cptr) (tab + l);
-  vkl_layer_weights w;
-  w.wk = (const void *)t[0], w.wq = (const void *)t[1], w.wv = (const void *)t[2];
-  w.wo = (const void *)t[3], w.w_gate = (const void *)t[4], w.w_up = (const void *)t[5];
-  w.w_down = (const void *)t[6];
-  w.attn_norm = (const float *)t[7], w.ffn_norm = (const float *)t[8];
-  w.kcache = (void *)t[9], w.vcache = (void *)t[10];
-  return w;
-}
-
-// The activation rows of one layer.  Several layers in one launch: every
-// layer has rows of its own (no row is written twice inside a launch, so no
-// cache can hold an older copy of a line); one layer per launch: the rows of
-// the launch-per-phase kernels.
-struct LayerRows
-{
-  uint16_t *x, *kqv, *att, *xm, *t, *xout;
-};
-
-__device__ __forceinline__ LayerRows
-rows_of_layer (const Params &p, int l, bool own_rows)
-{
-  if (!own_rows)
-    return LayerRows{ p.s.x, p.s.kqv, p.s.att, p.s.xm, p.s.t, p.s.x };
-  const size_t dim = (size_t)p.m.dim, ffn = layer_row_stride (p.m.ffn);
-  return LayerRows{ p.s.lx + (size_t)l * dim,  p.s.lkqv + (size_t)l * 3 * dim, p.s.latt + (size_t)l * dim,
-                    p.s.lxm + (size_t)l * dim, p.s.lt + (size_t)l * ffn,      p.s.lx + (size_t)(l + 1) * dim };
-}
-
 #ifdef VKL_TRACE
 #define VKL_TL(slot_)                                                          \
-  if (VKL_TID == 0 && p.trace)                                             \
+  if (threadIdx.x == 0 && p.trace)                                             \
     p.trace[((size_t)layer * 1024 + wg) * 16 + (slot_)] = wall_clock64 ();
 #else
 #define VKL_TL(slot_)
 #endif
 
-// Layers [l0, l1) for the workers (COURIER false) or for the courier of the
-// workgroup: the same barriers in the same order in both.
+// A layer from the attention on, for the workers (COURIER false) or for the
+// courier of the workgroup: the same barriers in the same order in both.
 //
 // The two item buffers are handed from phase to phase so that the memory has
 // work during the attention and no wave waits for a third up/gate item with
@@ -327,181 +298,147 @@ rows_of_layer (const Params &p, int l, bool own_rows)
 // second is multiplied.
 template <int WT, int XD, int XF, bool NT, bool COURIER>
 __device__ __forceinline__ void
-layers_body (const Params &p, const LayerCtx &c, uint8_t *lds)
+layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uint8_t *lds)
 {
-  typedef Gemv<WT, NT, 2> GV2;    // K/Q/V, up/gate: two-row units
+  typedef Gemv<WT, NT, 2> GV2;    // up/gate: two-row units
   typedef Gemv<WT, false, 2> GVO; // Wo: two-row units, plain loads (short phase)
   typedef Gemv<WT, NT, 1> GVD;    // down
   const vkl_decode_model &m = p.m;
   const int dim = m.dim, ffn = m.ffn, wg = c.wg, G = c.G, slot = c.slot, idx = c.idx;
+  const int layer = c.layer;
+  (void)layer;
   uint16_t *xl = (uint16_t *)lds;
   bool live = true; // false once a wait of this workgroup gave up
-  // where norm weights are parked (behind the staged row and the reduction words)
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps, pu; // pu: the up/gate product, begun during the Wo phase
+  PipeBuf A, B;
+  const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
+  const Deal deal_up = Deal{ 1, slot, idx, c.n_slot };
+  // where the norm weights of the up/gate phase are parked (behind the staged
+  // row and the reduction words)
   uint8_t *norm_lds = lds + lds_norm_offset (dim, ffn);
-  const Deal deal_all = Deal{ 1, slot, idx, c.n_slot };
   // heads h = slot, slot + 8, ... run on the first workgroups of XCD `slot`
   const int n_heads_here = (c.nh - slot + 7) >> 3;
-  const bool own_rows = c.own_rows;
-  for (int layer = c.l0; layer < c.l1; ++layer)
+  if (idx < n_heads_here)
     {
-      const int tid = VKL_TID;
-      const vkl_layer_weights lw = layer_record (p.m.layers, layer);
-      const LayerRows r = rows_of_layer (p, layer, own_rows);
-      const uint32_t mark = c.mark0 + (uint32_t)(layer - c.l0);
-      Epilogue e = {};
-      XRegs x;
-      NormRegs nw;
-      PipeState ps, pu; // pu: the up/gate product, begun during the Wo phase
-      PipeBuf A, B;
-      const QMat up = wmat<WT> (lw.w_up, ffn, dim), gate = wmat<WT> (lw.w_gate, ffn, dim);
-      if (c.first == 0)
-        {
-          // ---- RMSNorm + K/Q/V ---------------------------------------------
-          const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
-                     wv = wmat<WT> (lw.wv, dim, dim);
-          float *red = (float *)(lds + (size_t)dim * 2);
-          VKL_TL (0)
-          if (!COURIER)
-            GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 2, nullptr, true, Deal{ 0, 0, 0, 0 }, tid);
-          // (the first layer of a launch reads what an earlier launch wrote)
-          live = courier_fetch<COURIER> (layer > c.l0, flag_of (c, ST_DOWN, 0), 8, mark - 1u, c.limit,
-                                         c.err, c.word, 0x100u | ST_DOWN, r.x, dim, lds, lw.attn_norm, dim,
-                                         norm_lds)
-                 && live;
-          norm_from_lds<XD> (norm_lds, dim, nw);
-          row_from_lds<XD> (xl, dim, x);
-          stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
-          VKL_TL (1)
-          if (COURIER)
-            GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 2, nullptr, true, Deal{ 0, 0, 0, 0 }, tid);
-          e = Epilogue{};
-          uint16_t *y = live ? r.kqv : p.s.sink;
-          e.y[0] = y, e.y[1] = y + dim, e.y[2] = y + 2 * dim;
-          e.through = true;
-          GV2::run (ps, A, B, xl, e, red);
-          VKL_TL (2)
-          arrive (cnt_of (c, ST_KQV, slot), (uint32_t)c.n_slot, flag_of (c, ST_KQV, slot), 1, mark, false);
-          VKL_TL (3)
-        }
-      if (idx < n_heads_here)
-        {
-          // ---- one head of the attention -----------------------------------
-          // (the cached K and V rows are requested before the wait for this
-          // token's q, k and v: they do not depend on it)
-          auto wait_kqv = [&] () {
-            live = wait_flags (flag_of (c, ST_KQV, 0), 8, mark, c.limit, c.err, c.word, 0x100u | ST_KQV)
-                   && live;
-            VKL_TL (4)
-            return live;
-          };
-          if (m.head_dim == 128)
-            attention_head<128, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv, r.kqv, r.att);
-          else
-            attention_head<64, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv, r.kqv, r.att);
-          VKL_TL (5)
-          arrive (cnt_of (c, ST_ATT, 0), (uint32_t)c.nh, flag_of (c, ST_ATT, 0), 8, mark, c.silent);
-          arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, mark, false);
-          VKL_TL (6)
-          if (!COURIER)
-            GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_all, tid);
-        }
+      // ---- one head of the attention ---------------------------------------
+      // (the cached K and V rows are requested before the wait for this
+      // token's q, k and v: they do not depend on it)
+      auto wait_kqv = [&] () {
+        live = wait_flags (flag_of (c, ST_KQV, 0), 8, c.mark, c.limit, c.err, c.word, 0x100u | ST_KQV);
+        VKL_TL (4)
+        return live;
+      };
+      if (m.head_dim == 128)
+        attention_head<128, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv);
       else
-        {
-          // ---- Wo + residual -> xm -----------------------------------------
-          const QMat w = wmat<WT> (lw.wo, dim, dim);
-          const Deal dl = Deal{ 1, slot, idx - n_heads_here, c.n_slot - n_heads_here };
-          if (!COURIER)
-            {
-              GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, r.x, true, dl, tid);
-              if (VKL_LAYER_UP_EARLY)
-                GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_all, tid);
-            }
-          live = courier_fetch<COURIER> (c.first == 0, flag_of (c, ST_ATT, slot), 1, mark, c.limit, c.err,
-                                         c.word, 0x100u | ST_ATT, r.att, dim, lds, lw.ffn_norm, dim, norm_lds)
-                 && live;
-          if (COURIER)
-            GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, r.x, true, dl, tid);
-          else if (!VKL_LAYER_UP_EARLY)
-            GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_all, tid);
-          VKL_TL (4)
-          e = Epilogue{};
-          e.y[0] = live ? r.xm : p.s.sink, e.residual = r.x;
-          e.through = true;
-          GVO::run_single (ps, A, xl, e);
-          VKL_TL (5)
-          arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, mark, false);
-          VKL_TL (6)
-          // (after the arrival: it waits for everything the wave has in flight)
-          if (!COURIER)
-            GV2::issue (pu, A, 1), pu.primed = 2;
-        }
-
-      // ---- RMSNorm + up/gate with SiLU -> t ---------------------------------
-      {
-        float *red = (float *)(lds + (size_t)dim * 2);
-        // (a head's workgroup had its LDS in use until now: it fetches the norm weights here)
-        const bool head = idx < n_heads_here;
-        live = courier_fetch<COURIER> (true, flag_of (c, ST_WO, 0), 8, mark, c.limit, c.err, c.word,
-                                       0x100u | ST_WO, r.xm, dim, lds, head ? lw.ffn_norm : nullptr, dim,
-                                       norm_lds)
-               && live;
-        VKL_TL (7)
-        norm_from_lds<XD> (norm_lds, dim, nw);
-        row_from_lds<XD> (xl, dim, x);
-        stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
-        VKL_TL (8)
-        // (the courier's requests come after the barriers of the staging: a wave
-        // that waits for room in the memory path would hold up the other seven)
-        if (COURIER)
-          GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_all, tid);
-        e = Epilogue{};
-        e.y[0] = live ? r.t : p.s.sink;
-        e.through = true;
-        GV2::run (pu, B, A, xl, e, red);
-        VKL_TL (9)
-        arrive (cnt_of (c, ST_UP, slot), (uint32_t)c.n_slot, flag_of (c, ST_UP, slot), 1, mark, false);
-        VKL_TL (10)
-      }
-
-      // ---- down + residual -> x of the next layer -----------------------------
-      {
-        const QMat w = wmat<WT> (lw.w_down, dim, ffn);
-        float *red = (float *)(lds + (size_t)ffn * 2);
-        if (!COURIER)
-          GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, r.xm, true, deal_all, tid);
-        live = courier_fetch<COURIER> (true, flag_of (c, ST_UP, 0), 8, mark, c.limit, c.err, c.word,
-                                       0x100u | ST_UP, r.t, ffn, lds)
-               && live;
-        if (COURIER)
-          GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, r.xm, true, deal_all, tid);
-        VKL_TL (11)
-        e = Epilogue{};
-        e.y[0] = live ? r.xout : p.s.sink, e.residual = r.xm;
-        e.through = true;
-        GVD::run (ps, A, B, xl, e, red);
-        VKL_TL (13)
-        if (layer + 1 < c.l1)
-          arrive (cnt_of (c, ST_DOWN, slot), (uint32_t)c.n_slot, flag_of (c, ST_DOWN, slot), 1, mark, false);
-      }
+        attention_head<64, true, true> (p, lw, idx * 8 + slot, lds, nullptr, wait_kqv);
+      VKL_TL (5)
+      arrive (cnt_of (c, ST_ATT, 0), (uint32_t)c.nh, flag_of (c, ST_ATT, 0), 8, c.mark, c.silent);
+      arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
+      VKL_TL (6)
+      if (!COURIER)
+        GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_up);
     }
+  else
+    {
+      // ---- Wo + residual -> xm ---------------------------------------------
+      const QMat w = wmat<WT> (lw.wo, dim, dim);
+      const Deal dl = Deal{ 1, slot, idx - n_heads_here, c.n_slot - n_heads_here };
+      if (!COURIER)
+        {
+          GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x, true, dl);
+          if (VKL_LAYER_UP_EARLY)
+            GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_up);
+        }
+      live = courier_fetch<COURIER> (c.first == 0, flag_of (c, ST_ATT, slot), 1, c.mark, c.limit,
+                                     c.err, c.word, 0x100u | ST_ATT, p.s.att, dim, lds, lw.ffn_norm,
+                                     dim, norm_lds);
+      if (COURIER)
+        GVO::begin (ps, A, B, 0, w, w, w, dim, dim, wg, G, 1, p.s.x, true, dl);
+      else if (!VKL_LAYER_UP_EARLY)
+        GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_up);
+      VKL_TL (4)
+      e = Epilogue{};
+      e.y[0] = live ? p.s.xm : p.s.sink, e.residual = p.s.x;
+      e.through = true;
+      GVO::run_single (ps, A, xl, e);
+      VKL_TL (5)
+      arrive (cnt_of (c, ST_WO, slot), (uint32_t)c.n_slot, flag_of (c, ST_WO, slot), 1, c.mark, false);
+      VKL_TL (6)
+      // (after the arrival: it waits for everything the wave has in flight)
+      if (!COURIER)
+        GV2::issue (pu, A, 1), pu.primed = 2;
+    }
+
+  // ---- RMSNorm + up/gate with SiLU -> t -------------------------------------
+  {
+    float *red = (float *)(lds + (size_t)dim * 2);
+    // (a head's workgroup had its LDS in use until now: it fetches the norm weights here)
+    const bool head = idx < n_heads_here;
+    live = courier_fetch<COURIER> (true, flag_of (c, ST_WO, 0), 8, c.mark, c.limit, c.err, c.word,
+                                   0x100u | ST_WO, p.s.xm, dim, lds, head ? lw.ffn_norm : nullptr, dim,
+                                   norm_lds)
+           && live;
+    VKL_TL (7)
+    norm_from_lds<XD> (norm_lds, dim, nw);
+    row_from_lds<XD> (xl, dim, x);
+    stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+    VKL_TL (8)
+    // (the courier's requests come after the barriers of the staging: a wave
+    // that waits for room in the memory path would hold up the other seven)
+    if (COURIER)
+      GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 2, nullptr, true, deal_up);
+    e = Epilogue{};
+    e.y[0] = live ? p.s.t : p.s.sink;
+    e.through = true;
+    GV2::run (pu, B, A, xl, e, red);
+    VKL_TL (9)
+    arrive (cnt_of (c, ST_UP, slot), (uint32_t)c.n_slot, flag_of (c, ST_UP, slot), 1, c.mark, false);
+    VKL_TL (10)
+  }
+
+  // ---- down + residual -> x ---------------------------------------------------
+  {
+    const QMat w = wmat<WT> (lw.w_down, dim, ffn);
+    float *red = (float *)(lds + (size_t)ffn * 2);
+    if (!COURIER)
+      GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, kAhead, p.s.xm, true);
+    live = courier_fetch<COURIER> (true, flag_of (c, ST_UP, 0), 8, c.mark, c.limit, c.err, c.word,
+                                   0x100u | ST_UP, p.s.t, ffn, lds)
+           && live;
+    if (COURIER)
+      GVD::begin (ps, A, B, 0, w, w, w, dim, ffn, wg, G, 2, p.s.xm, true);
+    else if (kAhead < 2)
+      GVD::issue (ps, B, 1), ps.primed = 2;
+    VKL_TL (11)
+    e = Epilogue{};
+    e.y[0] = live ? p.s.x : p.s.sink, e.residual = p.s.xm;
+    GVD::run (ps, A, B, xl, e, red);
+    VKL_TL (13)
+  }
 }
 
 // XD / XF: 4096-element chunks of a row of dim / ffn values
 template <int WT, int XD, int XF, bool NT>
 __global__ __launch_bounds__ (kDecThreads) __attribute__ ((amdgpu_waves_per_eu (4, 4))) void
-decode_layer_kernel (const Params p, int l0, int l1, int first, int own_rows, int G,
+decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int first, int G,
                      size_t lds_word_at)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
+  typedef Gemv<WT, NT, 2> GV2; // K/Q/V: two-row units
   const vkl_decode_model &m = p.m;
-  const int nh = first == 0 ? m.n_heads : 0;
+  const int dim = m.dim, nh = first == 0 ? m.n_heads : 0;
   const int wg = (int)blockIdx.x;
   uint32_t *ls = p.s.lsync;
   uint32_t *err = p.s.sync + kSyncErr;
   uint32_t *word = (uint32_t *)(lds + lds_word_at); // [0] wait result, [1] XCD, [2] ticket
+  uint16_t *xl = (uint16_t *)lds;
   const bool silent = m.wait_test != 0;
-  // the number of this launch's first layer; flags raised in a layer carry its number
-  const uint32_t mark0 = ld_coherent_u32 (ls + kLsLaunch) + 1u;
+  // the number of this launch; flags raised in it carry it
+  const uint32_t mark = ld_coherent_u32 (ls + kLsLaunch) + 1u;
   // once a wait has given up the step is lost anyway: the launches that
   // follow until the host has looked do not wait at all
   const int limit
@@ -511,41 +448,81 @@ decode_layer_kernel (const Params p, int l0, int l1, int first, int own_rows, in
   // deals workgroups to XCDs except that each gets G / 8 of them (if not, a
   // counter below never fills up and the bounded waits report it).
   const int n_slot = G >> 3;
+  uint32_t xcc = 0, ticket = 0;
   if (threadIdx.x == 0)
     {
-      const uint32_t xcc = __builtin_amdgcn_s_getreg (20 | (0 << 6) | (3 << 11)) & 7u;
-      word[1] = xcc;
-      word[2] = __hip_atomic_fetch_add (ls + kLsTicket + 32 * xcc, 1u, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT);
+      xcc = __builtin_amdgcn_s_getreg (20 | (0 << 6) | (3 << 11)) & 7u;
+      ticket = __hip_atomic_fetch_add (ls + kLsTicket + 32 * xcc, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
     }
-  __syncthreads ();
-  const int slot = __builtin_amdgcn_readfirstlane ((int)word[1]);
-  const int idx = __builtin_amdgcn_readfirstlane ((int)word[2]);
-  if (idx >= n_slot && threadIdx.x == 0)
-    report (err, 0x200u | (uint32_t)slot);
+  VKL_TL (0)
+  Epilogue e = {};
+  XRegs x;
+  NormRegs nw;
+  PipeState ps;
+  PipeBuf A, B;
   // (a scalar: branches on it are wave-uniform)
   const bool courier = __builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier;
+  int slot = 0, idx = 0;
+  // (after a barrier that follows the store below)
+  auto place = [&] () {
+    slot = __builtin_amdgcn_readfirstlane ((int)word[1]);
+    idx = __builtin_amdgcn_readfirstlane ((int)word[2]);
+    if (idx >= n_slot && threadIdx.x == 0)
+      report (err, 0x200u | (uint32_t)slot);
+  };
+
+  if (first == 0)
+    {
+      // ---- RMSNorm + K/Q/V -------------------------------------------------
+      const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
+                 wv = wmat<WT> (lw.wv, dim, dim);
+      float *red = (float *)(lds + (size_t)dim * 2);
+      load_row<XD> (p.s.x, dim, x);
+      load_norm<XD> (lw.attn_norm, dim, nw);
+      __builtin_amdgcn_sched_barrier (0);
+      GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1, nullptr, true);
+      if (threadIdx.x == 0)
+        word[1] = xcc, word[2] = ticket;
+      stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+      VKL_TL (1)
+      place ();
+      e = Epilogue{};
+      e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
+      e.through = true;
+      GV2::run (ps, A, B, xl, e, red);
+      VKL_TL (2)
+      arrive (ls + kLsCnt + (ST_KQV * 8 + slot) * 32, (uint32_t)n_slot,
+              ls + kLsFlag + (ST_KQV * 8 + slot) * 32, 1, mark, false);
+      VKL_TL (3)
+    }
+  else
+    {
+      if (threadIdx.x == 0)
+        word[1] = xcc, word[2] = ticket;
+      __syncthreads ();
+      place ();
+    }
 #ifdef VKL_TRACE
   if (threadIdx.x == 0 && p.trace)
     {
-      p.trace[((size_t)l0 * 1024 + wg) * 16 + 12] = __builtin_amdgcn_s_getreg (4 | (0 << 6) | (31 << 11));
-      p.trace[((size_t)l0 * 1024 + wg) * 16 + 14] = (unsigned)idx | (unsigned)slot << 16;
+      p.trace[((size_t)layer * 1024 + wg) * 16 + 12] = __builtin_amdgcn_s_getreg (4 | (0 << 6) | (31 << 11));
+      p.trace[((size_t)layer * 1024 + wg) * 16 + 14] = (unsigned)idx | (unsigned)slot << 16;
     }
 #endif
-  const LayerCtx c = { ls,  err,   word, mark0, limit, n_slot, slot,  idx,
-                       nh,  first, wg,   G,     l0,    l1,     silent, own_rows != 0 };
+  const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, first, wg, G, layer, silent };
   // the courier's path is a copy of the workers' (the branch is wave-uniform):
   // in one copy, with the courier's weight requests under a condition, the
   // item buffers of the two roles collide and spill
   if (courier)
-    layers_body<WT, XD, XF, NT, true> (p, c, lds);
+    layer_tail<WT, XD, XF, NT, true> (p, lw, c, lds);
   else
-    layers_body<WT, XD, XF, NT, false> (p, c, lds);
+    layer_tail<WT, XD, XF, NT, false> (p, lw, c, lds);
   // (every workgroup has read the launch number and taken its ticket before
   // its first arrival, and this one has seen all of them arrive)
   if (wg == 0 && threadIdx.x < 9)
     st_coherent_u32 (threadIdx.x == 8 ? ls + kLsLaunch : ls + kLsTicket + 32 * (int)threadIdx.x,
-                     threadIdx.x == 8 ? mark0 + (uint32_t)(l1 - l0 - 1) : 0u);
+                     threadIdx.x == 8 ? mark : 0u);
 }
 
 // the token's embedding row as the start of the residual stream
@@ -587,7 +564,8 @@ embed_row_kernel (const Params p)
 
 template <int WT, int XD, int XF, bool NT>
 int
-launch_layer_t (const Params &p, int l0, int l1, int first, int own_rows, int G, hipStream_t s)
+launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                hipStream_t s)
 {
   const size_t at = (lds_bytes_needed (p.m.dim, p.m.ffn, p.m.maxlen, p.m.head_dim) + 15) & ~(size_t)15;
   const size_t lds = at + 16;
@@ -599,28 +577,30 @@ launch_layer_t (const Params &p, int l0, int l1, int first, int own_rows, int G,
       lds_set = lds;
     }
   decode_layer_kernel<WT, XD, XF, NT>
-      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, l0, l1, first, own_rows, G, at);
+      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, first, G, at);
   return 0;
 }
 
 template <int WT, int XD, int XF>
 int
-launch_layer_x (const Params &p, int l0, int l1, int first, int own_rows, int G, hipStream_t s)
+launch_layer_x (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                hipStream_t s)
 {
-  return p.stream_once ? launch_layer_t<WT, XD, XF, true> (p, l0, l1, first, own_rows, G, s)
-                       : launch_layer_t<WT, XD, XF, false> (p, l0, l1, first, own_rows, G, s);
+  return p.stream_once ? launch_layer_t<WT, XD, XF, true> (p, lw, layer, first, G, s)
+                       : launch_layer_t<WT, XD, XF, false> (p, lw, layer, first, G, s);
 }
 
 template <int WT>
 int
-launch_layer_wt (const Params &p, int l0, int l1, int first, int own_rows, int G, hipStream_t s)
+launch_layer_wt (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                 hipStream_t s)
 {
   const int xd = (p.m.dim + 4095) / 4096, xf = (p.m.ffn + 4095) / 4096;
   if (xd == 1 && xf == 1)
-    return launch_layer_x<WT, 1, 1> (p, l0, l1, first, own_rows, G, s);
+    return launch_layer_x<WT, 1, 1> (p, lw, layer, first, G, s);
   if (xd == 1 && xf <= 3)
-    return launch_layer_x<WT, 1, 3> (p, l0, l1, first, own_rows, G, s);
-  return launch_layer_x<WT, 2, 4> (p, l0, l1, first, own_rows, G, s);
+    return launch_layer_x<WT, 1, 3> (p, lw, layer, first, G, s);
+  return launch_layer_x<WT, 2, 4> (p, lw, layer, first, G, s);
 }
 } // namespace
 
@@ -630,19 +610,16 @@ layer_launch_supported (const vkl_decode_model &m, int G)
   // rows of up to two (dim) and four (ffn) chunks of 4096; every slot needs
   // workgroups beside the heads; two workgroups per compute unit must fit
   return m.dim <= 8192 && m.ffn <= 16384 && (m.dim % 8) == 0 && (m.ffn % 8) == 0
-         && (m.dim % 64) == 0 && G >= m.n_heads + 8 && (G % 8) == 0
+         && G >= m.n_heads + 8 && (G % 8) == 0
          && 2 * (lds_bytes_needed (m.dim, m.ffn, m.maxlen, m.head_dim) + 32) <= 160 * 1024;
 }
 
 int
-launch_layers (const Params &p, int l0, int l1, int first, int own_rows, int G, hipStream_t s)
+launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+              hipStream_t s)
 {
-  // (rows shared by all layers serve one layer per launch only)
-  if (l0 < 0 || l1 <= l0 || l1 > p.m.n_layers || (first != 0 && l1 - l0 != 1)
-      || (!own_rows && l1 - l0 != 1) || (own_rows && first != 0))
-    return (int)hipErrorInvalidValue;
-  return p.m.wtype == 8 ? launch_layer_wt<8> (p, l0, l1, first, own_rows, G, s)
-                        : launch_layer_wt<1> (p, l0, l1, first, own_rows, G, s);
+  return p.m.wtype == 8 ? launch_layer_wt<8> (p, lw, layer, first, G, s)
+                        : launch_layer_wt<1> (p, lw, layer, first, G, s);
 }
 
 int

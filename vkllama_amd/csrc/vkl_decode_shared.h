@@ -25,12 +25,6 @@ struct Scratch
   uint16_t *xm;       // [dim] residual stream between the Wo and the down projection
   uint16_t *sink;     // [max(3*dim, ffn)] where a workgroup whose wait gave up drops its results
   uint32_t *lsync;    // arrival counters and flags of the stages, launch count
-  // rows of their own for every layer (several layers in one launch)
-  uint16_t *lx;       // [n_layers + 1][dim]: the residual stream entering layer l
-  uint16_t *lkqv;     // [n_layers][3 * dim]
-  uint16_t *latt;     // [n_layers][dim]
-  uint16_t *lxm;      // [n_layers][dim]
-  uint16_t *lt;       // [n_layers][layer_row_stride (ffn)]
   // long-context attention, split over kAttnChunks chunks of the context
   float *part_max;    // [heads][kAttnChunks]
   float *part_sum;    // [heads][kAttnChunks]
@@ -52,13 +46,6 @@ align256 (size_t v)
   return (v + 255) & ~(size_t)255;
 }
 
-// rows that workgroups of different XCDs share start on cache lines
-__host__ __device__ inline size_t
-layer_row_stride (int n)
-{
-  return ((size_t)n + 63) & ~(size_t)63;
-}
-
 __host__ __device__ inline Scratch
 carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd,
        int n_layers)
@@ -78,11 +65,6 @@ carve (void *base, int dim, int ffn, int vocab, int heads, int maxlen, int hd,
   s.xm = (uint16_t *)(p + o), o += align256 ((size_t)dim * 2);
   s.sink = (uint16_t *)(p + o), o += align256 ((size_t)(3 * dim > ffn ? 3 * dim : ffn) * 2);
   s.lsync = (uint32_t *)(p + o), o += kLayerSyncBytes;
-  s.lx = (uint16_t *)(p + o), o += align256 ((size_t)(n_layers + 1) * layer_row_stride (dim) * 2);
-  s.lkqv = (uint16_t *)(p + o), o += align256 ((size_t)n_layers * 3 * layer_row_stride (dim) * 2);
-  s.latt = (uint16_t *)(p + o), o += align256 ((size_t)n_layers * layer_row_stride (dim) * 2);
-  s.lxm = (uint16_t *)(p + o), o += align256 ((size_t)n_layers * layer_row_stride (dim) * 2);
-  s.lt = (uint16_t *)(p + o), o += align256 ((size_t)n_layers * layer_row_stride (ffn) * 2);
   s.part_max = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_sum = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * 4);
   s.part_out = (float *)(p + o), o += align256 ((size_t)heads * kAttnChunks * hd * 4);
@@ -112,7 +94,7 @@ struct Params
 
 #ifdef VKL_TRACE
 #define VKL_TR(slot)                                                          \
-  if (VKL_TID == 0 && p.trace)                                            \
+  if (threadIdx.x == 0 && p.trace)                                            \
     p.trace[((size_t)(layer * 8 + phase) * 1024 + wg) * 8 + (slot)]           \
         = wall_clock64 ();
 #define VKL_TRP                                                               \
@@ -164,8 +146,8 @@ block_sum (float v, float *red)
 {
   v = wave_sum (v);
   __syncthreads ();
-  if ((VKL_TID & 63) == 0)
-    red[VKL_TID >> 6] = v;
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = v;
   __syncthreads ();
   float t = 0.f;
 #pragma unroll
@@ -206,15 +188,11 @@ struct NoWait
 template <int HD, bool COH, bool EARLY = false, typename Wait = NoWait>
 __device__ __forceinline__ void
 attention_head (const Params &p, const vkl_layer_weights &lw, int head,
-                uint8_t *lds, unsigned long long *tr = nullptr, Wait wait = Wait (),
-                const uint16_t *kqv_row = nullptr, uint16_t *att_row = nullptr)
+                uint8_t *lds, unsigned long long *tr = nullptr, Wait wait = Wait ())
 {
-  // (rows other than the scratch's shared ones: a launch over several layers)
-  const uint16_t *kqv = kqv_row ? kqv_row : p.s.kqv;
-  uint16_t *att = att_row ? att_row : p.s.att;
 #ifdef VKL_TRACE
 #define VKL_TRA(slot)                                                         \
-  if (tr && VKL_TID == 0)                                                 \
+  if (tr && threadIdx.x == 0)                                                 \
     tr[slot] = wall_clock64 ();
 #else
 #define VKL_TRA(slot)
@@ -231,10 +209,10 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
   float *red = part + RPB * HD;           // [2*kDecWaves]
   uint16_t *kc = (uint16_t *)lw.kcache + (size_t)head * maxlen * HD;
   uint16_t *vc = (uint16_t *)lw.vcache + (size_t)head * maxlen * HD;
-  const uint16_t *kin = kqv + head * HD;
-  const uint16_t *qin = kqv + dim + head * HD;
-  const uint16_t *vin = kqv + 2 * dim + head * HD;
-  const int tid = VKL_TID;
+  const uint16_t *kin = p.s.kqv + head * HD;
+  const uint16_t *qin = p.s.kqv + dim + head * HD;
+  const uint16_t *vin = p.s.kqv + 2 * dim + head * HD;
+  const int tid = threadIdx.x;
   const int sub = tid % LPR, grp = tid / LPR;
 
   // This token's q, k, v and its rotation factors are requested first and
@@ -426,7 +404,7 @@ attention_head (const Params &p, const vkl_layer_weights &lw, int head,
     o = row_sum<4> (o);
     const float onext = dpp_get<0x104> (o); // row_shl:4: the lane four up
     if (c < HD && (tid & 7) == 0)
-      st_u32<COH> ((uint32_t *)(att + head * HD) + (c >> 1),
+      st_u32<COH> ((uint32_t *)(p.s.att + head * HD) + (c >> 1),
                    (uint32_t)f2h (o) | ((uint32_t)f2h (onext) << 16));
   }
   __syncthreads ();
@@ -463,7 +441,7 @@ final_argmax (const Params &p, int G, uint8_t *lds)
   // G per-workgroup partials -> first maximum
   float v = -INFINITY;
   uint32_t idx = 0xffffffffu;
-  for (int i = VKL_TID; i < G; i += kDecThreads)
+  for (int i = threadIdx.x; i < G; i += kDecThreads)
     {
       const float pv = __uint_as_float (
           ld_u32<COH> ((const uint32_t *)(p.s.amax_val + i)));
@@ -481,13 +459,13 @@ final_argmax (const Params &p, int G, uint8_t *lds)
     }
   float *bv = (float *)lds;
   uint32_t *bi = (uint32_t *)(lds + 64);
-  if ((VKL_TID & 63) == 0)
+  if ((threadIdx.x & 63) == 0)
     {
-      bv[VKL_TID >> 6] = v;
-      bi[VKL_TID >> 6] = idx;
+      bv[threadIdx.x >> 6] = v;
+      bi[threadIdx.x >> 6] = idx;
     }
   __syncthreads ();
-  if (VKL_TID == 0)
+  if (threadIdx.x == 0)
     {
       for (int w = 1; w < kDecWaves; ++w)
         if (better (bv[w], bi[w], v, idx))
@@ -506,15 +484,13 @@ final_argmax (const Params &p, int G, uint8_t *lds)
     }
 }
 
-// Layers [l0, l1) of the step as a single launch (vkl_decode_layer.hip).
-// first = 0: per layer K/Q/V, attention with one workgroup per head, Wo,
-// up/gate, down.  own_rows = 1: every layer works on rows of its own
-// (Scratch::lx ...: layer l reads lx[l] and leaves lx[l + 1]); own_rows = 0
-// (one layer only): on the rows of the launch-per-phase kernels.  first = 1 (one layer): from the
-// Wo projection on (the attention output is in memory).  G workgroups that
-// must all be resident at once.
+// One layer of the step as a single launch (vkl_decode_layer.hip).  first = 0:
+// K/Q/V, attention with one workgroup per head, Wo, up/gate, down; first = 1:
+// from the Wo projection on (the attention output is in memory).  G workgroups
+// that must all be resident at once.
 bool layer_launch_supported (const vkl_decode_model &m, int G);
-int launch_layers (const Params &p, int l0, int l1, int first, int own_rows, int G, hipStream_t s);
+int launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+                  hipStream_t s);
 // the token's embedding row -> residual stream (one small launch in front of layer 0)
 int launch_embed_row (const Params &p, hipStream_t s);
 } // namespace dec

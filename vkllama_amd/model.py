@@ -8,7 +8,7 @@ import numpy as np
 
 from . import capi
 
-HOST_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libvkllama_host.so")
+HOST_LIB_PATH = os.path.join(capi.LIB_DIR, "libvkllama_host.so")
 
 vp, sz, u32, u64, i32 = C.c_void_p, C.c_size_t, C.c_uint32, C.c_uint64, C.c_int
 
@@ -255,7 +255,7 @@ class Llama2:
     def decode_step_bytes(self, L):
         return int(lib().vkl_model_decode_step_bytes(self._h, L))
 
-    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax", "unused", "layer", "layers")
+    PHASES = ("kqv", "attention", "wo", "upgate", "down", "lm_head", "argmax", "unused", "layer")
 
     def phase_times(self):
         """{phase: (milliseconds summed, launches)} since the last call; filled

@@ -157,8 +157,7 @@ public:
   // ---- additions -----------------------------------------------------------
   void set_fused_decode (bool on) { fused_decode_ = on; }
   void set_lastblock_rope_quirk (bool on);
-  // 0 = one launch per decode phase, 1 = one launch per layer, 2 = one launch
-  // for all layers
+  // 0 = one launch per decode phase, 1 = one launch per layer
   void set_decode_mode (int mode);
   // options of the fused decode steps: "attn_split_min", "fuse_attn_wo",
   // "wait_test" (DecodePlan::set_option)
