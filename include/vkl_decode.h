@@ -73,12 +73,12 @@ size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
  *           split length); 1 = one launch per layer: all workgroups stay
  *           resident through the five phases, hand activations over through
  *           memory with bounded waits for one another, and have the next
- *           phase's weights on the way meanwhile (above the split length:
- *           K/Q/V, split attention, then Wo + up/gate + down in one
- *           launch).  Results are bit for bit those of mode 0.  Models whose
- *           rows the one-launch form does not cover run as mode 0.  The GPU
- *           must not be shared while such a launch runs: see
- *           vkl_decode_status
+ *           phase's weights on the way meanwhile.  Results are bit for bit
+ *           those of mode 0.  Positions at or above the split length (the
+ *           attention then takes more than one workgroup per head) and
+ *           models whose rows the one-launch form does not cover run as
+ *           mode 0.  The GPU must not be shared while such a launch runs:
+ *           see vkl_decode_status
  *  logits32 optional device fp32 [vocab]: widened fp16 logits
  *  next_tok optional device-visible uint32: arg-max id, lowest index on ties
  * Returns 0 or a hipError_t; hipErrorInvalidValue for shapes the kernels do
@@ -89,9 +89,10 @@ int vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok,
 
 /* Launches in which workgroups wait for one another (mode 1; the attention +
  * Wo launch of mode 0) need every workgroup resident at once and the
- * workgroups dealt round-robin over the XCDs; where that does not hold (a GPU
- * shared with other work, another dispatch order) a bounded wait inside the
- * kernel gives up or the kernel notices the placement, the launch still ends,
+ * same number of them on each XCD; where that does not hold (a GPU shared
+ * with other work, another way of dealing workgroups to XCDs) a bounded wait
+ * inside the kernel gives up or the kernel notices the placement, the launch
+ * still ends,
  * the workgroup concerned drops its results instead of storing them, and the
  * step's results are invalid.  This call synchronises the stream and returns
  * 0 if nothing of the kind happened since the last call,

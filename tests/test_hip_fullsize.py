@@ -116,16 +116,17 @@ def test_c3_llama2_7b_q8_0_against_oracle():
     assert ids == gold["oracle_ids"]
     assert same >= 31
     # the greedy loop: replayed from a graph (bench.py's form), launched step
-    # by step, and with one launch per layer give one sequence, which
+    # by step, and with one launch per phase give one sequence, which
     # follows the oracle's up to the first near-tie (where margin_ok above has
     # already accepted the GPU's choice) and takes the GPU's choice there
     ids1, _, _ = m.generate_greedy(prompt, 32)
     m.set_option("decode_graph", 0)
     ids2, _, _ = m.generate_greedy(prompt, 32)
     assert list(ids2) == list(ids1)
-    m.set_option("decode_mode", 1)
+    m.set_option("decode_mode", 0)  # (the runs above: the default, one launch per layer)
     ids3, _, _ = m.generate_greedy(prompt, 32)
     assert list(ids3) == list(ids1)
+    assert m.decode_recoveries() == 0
     n = next((i for i in range(32) if int(ids1[i]) != ids[i]), 32)
     assert [int(t) for t in ids1[:n + 1]] == gpu_ids[:n + 1]
     m.close()
@@ -253,6 +254,7 @@ def test_c5_full_depth_decode_against_oracle_from_filled_caches():
     m = M.Llama2(cfg, w)
     om = O.OracleModel(cfg, w)
     fill_caches(m, om, cfg, 3968, seed=5)
+    m.set_option("decode_mode", 0)
     assert decode_steps_against_oracle(m, om, 1234, 3968, 4) >= 3
     m.set_option("decode_mode", 1)
     got, want = m.forward([77], 3972), om.forward([77], 3972)
@@ -271,6 +273,7 @@ def test_c4_full_depth_decode_against_oracle_from_filled_caches():
     m = M.Llama2(cfg, w)
     om = O.OracleModel(cfg, w)
     fill_caches(m, om, cfg, 2048, seed=6)
+    m.set_option("decode_mode", 0)
     assert decode_steps_against_oracle(m, om, 4321, 2048, 4) >= 3
     m.set_option("decode_mode", 1)
     got, want = m.forward([77], 2052), om.forward([77], 2052)

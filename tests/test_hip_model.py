@@ -28,18 +28,26 @@ def logit_err(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-6))
 
 
+def set_path(m, fused):
+    """0: operator chain for single tokens too; 1: fused decode step, one launch
+    per phase; 2: fused decode step, one launch per layer (the default)."""
+    m.set_option("fused_decode", int(fused > 0))
+    if fused:
+        m.set_option("decode_mode", fused - 1)
+
+
 @pytest.fixture(scope="module")
 def small():
     w = M.synth_weights(SMALL, seed=11)
     return SMALL, w
 
 
-@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("fused", [0, 1, 2])
 def test_prefill_then_decode_logits_and_caches(small, fused):
     cfg, w = small
     prompt = np.array([5, 17, 99, 3, 64, 8, 1000], np.uint32)
     m = M.Llama2(cfg, w)
-    m.set_option("fused_decode", fused)
+    set_path(m, fused)
     om = O.OracleModel(cfg, w)
     got = m.forward(prompt, 0)
     want = om.forward(prompt, 0)
@@ -96,12 +104,12 @@ def test_fused_decode_equals_operator_chain(small):
 
 
 @pytest.mark.parametrize("cfg,seed", [(SMALL, 11), (SMALL128, 5)])
-@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("fused", [0, 1, 2])
 def test_greedy_ids_identical_to_oracle_small(cfg, seed, fused):
     w = M.synth_weights(cfg, seed=seed)
     prompt = np.array([5, 17, 99, 3], np.uint32)
     m = M.Llama2(cfg, w)
-    m.set_option("fused_decode", fused)
+    set_path(m, fused)
     ids, _, _ = m.generate_greedy(prompt, 24)
     want, _ = O.OracleModel(cfg, w).generate_greedy(prompt, 24)
     assert list(ids) == list(want)
@@ -192,7 +200,7 @@ def test_lastblock_rope_quirk_switch(small):
         m.close()
 
 
-@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("fused", [0, 1, 2])
 def test_fp16_weights_model(fused):
     """FP16 matrices: operator chain, and the fused decode step on its fp16
     weight path."""
@@ -200,7 +208,7 @@ def test_fp16_weights_model(fused):
     w = M.synth_weights(cfg, seed=3)
     prompt = np.array([5, 17, 99], np.uint32)
     m = M.Llama2(cfg, w)
-    m.set_option("fused_decode", fused)
+    set_path(m, fused)
     om = O.OracleModel(cfg, w)
     assert logit_err(m.forward(prompt, 0), om.forward(prompt, 0)) < 1e-2
     assert logit_err(m.forward([4], 3), om.forward([4], 3)) < 1e-2
@@ -465,7 +473,7 @@ def test_wait_inside_a_launch_is_bounded_and_recovered(mode):
     m.close()
 
 
-@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("fused", [0, 1, 2])
 def test_sampled_generation_on_the_device(small, fused):
     """generate_sampled: k = 1 is the greedy sequence; a seed reproduces a top-k
     sequence; every drawn token is one of the k most likely tokens of the
@@ -474,7 +482,7 @@ def test_sampled_generation_on_the_device(small, fused):
     cfg, w = small
     prompt = np.array([5, 17, 99, 3], np.uint32)
     m = M.Llama2(cfg, w)
-    m.set_option("fused_decode", fused)
+    set_path(m, fused)
     greedy, _, _ = m.generate_greedy(prompt, 12)
     top1, _, _ = m.generate_sampled(prompt, 12, topk=1, seed=3)
     assert list(top1) == list(greedy)

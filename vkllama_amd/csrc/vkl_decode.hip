@@ -992,39 +992,28 @@ int
 launch_step (const Params &p, const vkl_decode_model *m, int mode, int n_cu, int G,
              size_t lds, hipStream_t s)
 {
-  const bool per_layer = mode == 1 && layer_launch_supported (*m, G);
-  const bool short_ctx = (int)p.pos + 1 < attn_split_min (*m);
+  // (one head per workgroup inside the layer launch: contexts long enough for
+  // the split attention take the launches per phase)
+  const bool per_layer = mode == 1 && layer_launch_supported (*m, G)
+                         && (int)p.pos + 1 < attn_split_min (*m);
   if (per_layer)
     if (int e = launch_embed_row (p, s))
       return e;
   for (int l = 0; l < m->n_layers; ++l)
     {
       const vkl_layer_weights &lw = m->layers_h[l];
-      if (per_layer && short_ctx)
-        {
-          if (int e = timer_mark (PH_LAYER, false, s))
-            return e;
-          if (int e = launch_layer (p, lw, l, 0, G, s))
-            return e;
-          if (int e = timer_mark (PH_LAYER, true, s))
-            return e;
-          continue;
-        }
-      // (with the embedding row in place, layer 0 is a layer like the others)
-      if (int e = launch_phase<PH_KQV> (p, lw, per_layer ? std::max (l, 1) : l, G, G, lds, s))
-        return e;
       if (per_layer)
         {
-          if (int e = launch_attention (p, m, lw, l, n_cu, lds, s))
-            return e;
           if (int e = timer_mark (PH_LAYER, false, s))
             return e;
-          if (int e = launch_layer (p, lw, l, 1, G, s))
+          if (int e = launch_layer (p, lw, l, G, s))
             return e;
           if (int e = timer_mark (PH_LAYER, true, s))
             return e;
           continue;
         }
+      if (int e = launch_phase<PH_KQV> (p, lw, l, G, G, lds, s))
+        return e;
       if (attn_wo_fused (p, m, G))
         {
           if (int e = launch_attn_wo (p, lw, l, G, lds, s))
@@ -1359,7 +1348,8 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
   p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
   hipStream_t s = (hipStream_t)stream;
   const int G = n_cu * 2;
-  VKL_CHECK_ARG (kind != PH_LAYER || layer_launch_supported (*m, G));
+  VKL_CHECK_ARG (kind != PH_LAYER
+                 || (layer_launch_supported (*m, G) && (int)pos + 1 < attn_split_min (*m)));
   const bool was_on = g_timer.on;
   g_timer.on = false;
   hipEvent_t e0, e1;
@@ -1397,7 +1387,7 @@ vkl_decode_phase_replay (const vkl_decode_model *m, int kind, uint32_t pos,
               err = launch_phase<PH_UPGATE> (p, lw, l, G, G, lds, s);
               break;
             case PH_LAYER:
-              err = launch_layer (p, lw, l, (int)pos + 1 < attn_split_min (*m) ? 0 : 1, G, s);
+              err = launch_layer (p, lw, l, G, s);
               break;
             default:
               err = launch_phase<PH_DOWN> (p, lw, l, G, G, lds, s);

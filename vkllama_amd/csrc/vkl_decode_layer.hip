@@ -111,14 +111,18 @@ arrive (uint32_t *cnt, uint32_t n, uint32_t *flag, int nflags, uint32_t mark, bo
 {
   __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
   __syncthreads ();
-  // (the courier counts in: the other waves go straight on to request the
-  // next phase's weights instead of waiting for the counter's answer)
-  if (__builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier)
+  // (the courier counts in: the other waves go on to request the next phase's
+  // weights instead of waiting for the counter's answer; they wait for the
+  // second barrier so that the atomic enters the compute unit's memory path,
+  // which is served in order, ahead of those requests)
+  uint32_t old = 0;
+  const bool courier = __builtin_amdgcn_readfirstlane ((int)(threadIdx.x >> 6)) == kCourier;
+  const int lane = (int)threadIdx.x & 63;
+  if (courier && lane == 0)
+    old = __hip_atomic_fetch_add (cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_barrier ();
+  if (courier)
     {
-      const int lane = (int)threadIdx.x & 63;
-      uint32_t old = 0;
-      if (lane == 0)
-        old = __hip_atomic_fetch_add (cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
       if (old + 1u == n)
         {
@@ -260,7 +264,7 @@ struct LayerCtx
 {
   uint32_t *ls, *err, *word;
   uint32_t mark;
-  int limit, n_slot, slot, idx, nh, first, wg, G, layer;
+  int limit, n_slot, slot, idx, nh, wg, G, layer;
   bool silent;
 };
 
@@ -353,7 +357,7 @@ layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uin
           if (VKL_LAYER_UP_EARLY)
             GV2::begin (pu, B, A, 2, up, gate, up, ffn, dim, wg, G, 1, nullptr, true, deal_up);
         }
-      live = courier_fetch<COURIER> (c.first == 0, flag_of (c, ST_ATT, slot), 1, c.mark, c.limit,
+      live = courier_fetch<COURIER> (true, flag_of (c, ST_ATT, slot), 1, c.mark, c.limit,
                                      c.err, c.word, 0x100u | ST_ATT, p.s.att, dim, lds, lw.ffn_norm,
                                      dim, norm_lds);
       if (COURIER)
@@ -424,13 +428,13 @@ layer_tail (const Params &p, const vkl_layer_weights &lw, const LayerCtx &c, uin
 // XD / XF: 4096-element chunks of a row of dim / ffn values
 template <int WT, int XD, int XF, bool NT>
 __global__ __launch_bounds__ (kDecThreads) __attribute__ ((amdgpu_waves_per_eu (4, 4))) void
-decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int first, int G,
+decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int G,
                      size_t lds_word_at)
 {
   extern __shared__ __align__ (16) uint8_t lds[];
   typedef Gemv<WT, NT, 2> GV2; // K/Q/V: two-row units
   const vkl_decode_model &m = p.m;
-  const int dim = m.dim, nh = first == 0 ? m.n_heads : 0;
+  const int dim = m.dim, nh = m.n_heads;
   const int wg = (int)blockIdx.x;
   uint32_t *ls = p.s.lsync;
   uint32_t *err = p.s.sync + kSyncErr;
@@ -472,37 +476,29 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       report (err, 0x200u | (uint32_t)slot);
   };
 
-  if (first == 0)
-    {
-      // ---- RMSNorm + K/Q/V -------------------------------------------------
-      const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
-                 wv = wmat<WT> (lw.wv, dim, dim);
-      float *red = (float *)(lds + (size_t)dim * 2);
-      load_row<XD> (p.s.x, dim, x);
-      load_norm<XD> (lw.attn_norm, dim, nw);
-      __builtin_amdgcn_sched_barrier (0);
-      GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1, nullptr, true);
-      if (threadIdx.x == 0)
-        word[1] = xcc, word[2] = ticket;
-      stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
-      VKL_TL (1)
-      place ();
-      e = Epilogue{};
-      e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
-      e.through = true;
-      GV2::run (ps, A, B, xl, e, red);
-      VKL_TL (2)
-      arrive (ls + kLsCnt + (ST_KQV * 8 + slot) * 32, (uint32_t)n_slot,
-              ls + kLsFlag + (ST_KQV * 8 + slot) * 32, 1, mark, false);
-      VKL_TL (3)
-    }
-  else
-    {
-      if (threadIdx.x == 0)
-        word[1] = xcc, word[2] = ticket;
-      __syncthreads ();
-      place ();
-    }
+  {
+    // ---- RMSNorm + K/Q/V -------------------------------------------------
+    const QMat wk = wmat<WT> (lw.wk, dim, dim), wq = wmat<WT> (lw.wq, dim, dim),
+               wv = wmat<WT> (lw.wv, dim, dim);
+    float *red = (float *)(lds + (size_t)dim * 2);
+    load_row<XD> (p.s.x, dim, x);
+    load_norm<XD> (lw.attn_norm, dim, nw);
+    __builtin_amdgcn_sched_barrier (0);
+    GV2::begin (ps, A, B, 1, wk, wq, wv, dim, dim, wg, G, 1, nullptr, true);
+    if (threadIdx.x == 0)
+      word[1] = xcc, word[2] = ticket;
+    stage_row<true, XD> (x, dim, xl, nw, m.eps, red, nullptr);
+    VKL_TL (1)
+    place ();
+    e = Epilogue{};
+    e.y[0] = p.s.kqv, e.y[1] = p.s.kqv + dim, e.y[2] = p.s.kqv + 2 * dim;
+    e.through = true;
+    GV2::run (ps, A, B, xl, e, red);
+    VKL_TL (2)
+    arrive (ls + kLsCnt + (ST_KQV * 8 + slot) * 32, (uint32_t)n_slot,
+            ls + kLsFlag + (ST_KQV * 8 + slot) * 32, 1, mark, false);
+    VKL_TL (3)
+  }
 #ifdef VKL_TRACE
   if (threadIdx.x == 0 && p.trace)
     {
@@ -510,7 +506,7 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       p.trace[((size_t)layer * 1024 + wg) * 16 + 14] = (unsigned)idx | (unsigned)slot << 16;
     }
 #endif
-  const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, first, wg, G, layer, silent };
+  const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, wg, G, layer, silent };
   // the courier's path is a copy of the workers' (the branch is wave-uniform):
   // in one copy, with the courier's weight requests under a condition, the
   // item buffers of the two roles collide and spill
@@ -564,7 +560,7 @@ embed_row_kernel (const Params p)
 
 template <int WT, int XD, int XF, bool NT>
 int
-launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int G,
                 hipStream_t s)
 {
   const size_t at = (lds_bytes_needed (p.m.dim, p.m.ffn, p.m.maxlen, p.m.head_dim) + 15) & ~(size_t)15;
@@ -577,30 +573,30 @@ launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int fir
       lds_set = lds;
     }
   decode_layer_kernel<WT, XD, XF, NT>
-      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, first, G, at);
+      <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G, at);
   return 0;
 }
 
 template <int WT, int XD, int XF>
 int
-launch_layer_x (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+launch_layer_x (const Params &p, const vkl_layer_weights &lw, int layer, int G,
                 hipStream_t s)
 {
-  return p.stream_once ? launch_layer_t<WT, XD, XF, true> (p, lw, layer, first, G, s)
-                       : launch_layer_t<WT, XD, XF, false> (p, lw, layer, first, G, s);
+  return p.stream_once ? launch_layer_t<WT, XD, XF, true> (p, lw, layer, G, s)
+                       : launch_layer_t<WT, XD, XF, false> (p, lw, layer, G, s);
 }
 
 template <int WT>
 int
-launch_layer_wt (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+launch_layer_wt (const Params &p, const vkl_layer_weights &lw, int layer, int G,
                  hipStream_t s)
 {
   const int xd = (p.m.dim + 4095) / 4096, xf = (p.m.ffn + 4095) / 4096;
   if (xd == 1 && xf == 1)
-    return launch_layer_x<WT, 1, 1> (p, lw, layer, first, G, s);
+    return launch_layer_x<WT, 1, 1> (p, lw, layer, G, s);
   if (xd == 1 && xf <= 3)
-    return launch_layer_x<WT, 1, 3> (p, lw, layer, first, G, s);
-  return launch_layer_x<WT, 2, 4> (p, lw, layer, first, G, s);
+    return launch_layer_x<WT, 1, 3> (p, lw, layer, G, s);
+  return launch_layer_x<WT, 2, 4> (p, lw, layer, G, s);
 }
 } // namespace
 
@@ -615,11 +611,11 @@ layer_launch_supported (const vkl_decode_model &m, int G)
 }
 
 int
-launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
+launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int G,
               hipStream_t s)
 {
-  return p.m.wtype == 8 ? launch_layer_wt<8> (p, lw, layer, first, G, s)
-                        : launch_layer_wt<1> (p, lw, layer, first, G, s);
+  return p.m.wtype == 8 ? launch_layer_wt<8> (p, lw, layer, G, s)
+                        : launch_layer_wt<1> (p, lw, layer, G, s);
 }
 
 int

@@ -484,13 +484,11 @@ final_argmax (const Params &p, int G, uint8_t *lds)
     }
 }
 
-// One layer of the step as a single launch (vkl_decode_layer.hip).  first = 0:
-// K/Q/V, attention with one workgroup per head, Wo, up/gate, down; first = 1:
-// from the Wo projection on (the attention output is in memory).  G workgroups
-// that must all be resident at once.
+// One layer of the step as a single launch (vkl_decode_layer.hip): K/Q/V,
+// attention with one workgroup per head, Wo, up/gate, down.  G workgroups that
+// must all be resident at once.
 bool layer_launch_supported (const vkl_decode_model &m, int G);
-int launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int first, int G,
-                  hipStream_t s);
+int launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int G, hipStream_t s);
 // the token's embedding row -> residual stream (one small launch in front of layer 0)
 int launch_embed_row (const Params &p, hipStream_t s);
 } // namespace dec

@@ -19,7 +19,7 @@ hip_status (const char *what, int e)
 }
 
 DecodePlan::DecodePlan ()
-    : gpu_ (nullptr), usable_ (false), mode_ (0), adopted_valid_ (false),
+    : gpu_ (nullptr), usable_ (false), mode_ (1), adopted_valid_ (false),
       vocab_ (0)
 {
   memset (&desc_, 0, sizeof (desc_));
