@@ -111,6 +111,18 @@ int vkl_decode_status (const vkl_decode_model *m, void *stream);
 int vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
                      int n_steps, int mode, float *logits32, void *stream);
 
+/* The same loop with the sampler of models/samplers.cpp:37-101 instead of the
+ * arg-max as the last launch of every captured step (vkl_sample_f32's kernel:
+ * topp < 0 keeps the topk largest logits, else the top-p set): the token of
+ * position pos0 + i + 1 is drawn with the uniform number of (seed, that
+ * position).  topk, topp and seed live in device memory, so one captured
+ * graph serves every request; results are those of n_steps calls of
+ * vkl_decode_step, each followed by vkl_sample_f32 with counter = position. */
+int vkl_decode_loop_sampled (const vkl_decode_model *m, uint32_t *ids,
+                             uint32_t pos0, int n_steps, int mode,
+                             float *logits32, int topk, float topp,
+                             uint64_t seed, void *stream);
+
 /* device pointer to the fp16 logits [vocab] of the last step inside scratch */
 const void *vkl_decode_logits_f16 (const vkl_decode_model *m);
 /* arg-max over fp32 values (first maximum); out is device-visible */

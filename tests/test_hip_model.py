@@ -490,6 +490,18 @@ def test_sampled_generation_on_the_device(small, fused):
     b, _, _ = m.generate_sampled(prompt, 16, topk=8, seed=7)
     c, _, _ = m.generate_sampled(prompt, 16, topk=8, seed=8)
     assert list(a) == list(b) and list(a) != list(c) and list(a) != list(greedy[:1]) * 16
+    # the loop replayed from a captured graph (the draw is the last launch of
+    # every step, k / p / seed in device memory) and launched step by step
+    # with the sampler called from the host draw the same tokens
+    m.set_option("decode_graph", 0)
+    for kw in (dict(topk=8, seed=7), dict(topk=3, seed=11), dict(topp=0.6, seed=5)):
+        m.set_option("decode_graph", 1)
+        replayed, _, _ = m.generate_sampled(prompt, 16, **kw)
+        m.set_option("decode_graph", 0)
+        stepwise, _, _ = m.generate_sampled(prompt, 16, **kw)
+        assert list(replayed) == list(stepwise), kw
+    m.set_option("decode_graph", 1)
+    assert list(m.generate_sampled(prompt, 16, topk=8, seed=7)[0]) == list(a)
     om = O.OracleModel(cfg, w)
     logits = om.forward(prompt, 0)
     pos = len(prompt)

@@ -1034,6 +1034,8 @@ launch_step (const Params &p, const vkl_decode_model *m, int mode, int n_cu, int
   const vkl_layer_weights none = {};
   if (int e = launch_phase<PH_HEAD> (p, none, 0, G, G, lds, s))
     return e;
+  if (p.loop && p.sample)
+    return sample_loop_launch (p.logits32, m->vocab, p.sample, (uint32_t *)p.loop, p.ids, s);
   if (p.next_tok || p.loop)
     if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
       return e;
@@ -1159,6 +1161,12 @@ set_loop_state_kernel (uint32_t *state, uint32_t index, uint32_t pos)
   state[1] = pos;
 }
 
+__global__ void
+set_sample_params_kernel (uint32_t *dst, uint32_t k, uint32_t p_bits, uint32_t seed_lo, uint32_t seed_hi)
+{
+  dst[0] = k, dst[1] = p_bits, dst[2] = seed_lo, dst[3] = seed_hi;
+}
+
 // One captured step per (model, id buffer, logits buffer, attention form).
 struct StepGraph
 {
@@ -1166,6 +1174,7 @@ struct StepGraph
   uint64_t model_hash = 0; // over every pointer, dimension and option the launches hold
   int long_ctx = 0;
   int mode = 0;
+  int sampled = 0;
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   uint64_t used = 0;
@@ -1204,9 +1213,11 @@ drop_graph (StepGraph &g)
 // kAttnSplitMinLen positions, split above); token index and position live in
 // device memory and are advanced by the step's last kernel, so every replay
 // is the identical sequence of launches with identical arguments.
-extern "C" int
-vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
-                 int n_steps, int mode, float *logits32, void *stream)
+namespace
+{
+int
+decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0, int n_steps, int mode,
+             float *logits32, bool sampled, int topk, float topp, uint64_t seed, void *stream)
 {
   if (int e = check_model (m))
     return e;
@@ -1230,6 +1241,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
   p.next_tok = nullptr;
   p.loop = p.s.sync + 16;
   p.ids = ids;
+  p.sample = sampled ? p.s.sync + 20 : nullptr;
   p.gemv_res = nullptr;
   p.stream_once = step_weight_bytes (*m) > kCacheResidentBytes;
 #ifdef VKL_TRACE
@@ -1240,6 +1252,10 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
   g_timer.on = false;
   const uint64_t mh = hash_model (m);
   set_loop_state_kernel<<<dim3 (1), dim3 (1), 0, s>>> ((uint32_t *)p.loop, 0u, pos0);
+  if (sampled)
+    set_sample_params_kernel<<<dim3 (1), dim3 (1), 0, s>>> (p.s.sync + 20, (uint32_t)topk,
+                                                            __builtin_bit_cast (uint32_t, topp),
+                                                            (uint32_t)seed, (uint32_t)(seed >> 32));
   int err = 0;
   int done = 0;
   while (done < n_steps && !err)
@@ -1255,7 +1271,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
         {
           if (c.exec && c.scratch == m->scratch && c.ids == ids
               && c.logits == p.logits32 && c.model_hash == mh
-              && c.long_ctx == long_ctx && c.mode == mode)
+              && c.long_ctx == long_ctx && c.mode == mode && c.sampled == (int)sampled)
             g = &c;
           if (c.used < lru->used)
             lru = &c;
@@ -1290,7 +1306,7 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
               break;
             }
           g->scratch = m->scratch, g->ids = ids, g->logits = p.logits32;
-          g->model_hash = mh, g->long_ctx = long_ctx, g->mode = mode;
+          g->model_hash = mh, g->long_ctx = long_ctx, g->mode = mode, g->sampled = (int)sampled;
         }
       g->used = ++g_graph_clock;
       for (; done < upto && !err; ++done)
@@ -1298,6 +1314,24 @@ vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
     }
   g_timer.on = timing;
   return err ? err : vkl_launch_status ();
+}
+}
+
+extern "C" int
+vkl_decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0,
+                 int n_steps, int mode, float *logits32, void *stream)
+{
+  return decode_loop (m, ids, pos0, n_steps, mode, logits32, false, 1, -1.f, 0, stream);
+}
+
+extern "C" int
+vkl_decode_loop_sampled (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0, int n_steps,
+                         int mode, float *logits32, int topk, float topp, uint64_t seed,
+                         void *stream)
+{
+  VKL_CHECK_ARG (topp >= 0.f || topk >= 1);
+  VKL_CHECK_ARG (topp < 0.f || topp <= 1.0f);
+  return decode_loop (m, ids, pos0, n_steps, mode, logits32, true, topk, topp, seed, stream);
 }
 
 extern "C" int

@@ -85,6 +85,9 @@ struct Params
   // memory so that every step is the same sequence of launches
   const uint32_t *loop; // {index into ids, position}, or null
   uint32_t *ids;        // loop: input token ids[index], result to ids[index + 1]
+  // loop only: if set, the step ends with a draw from the logits instead of
+  // the arg-max ({k, bits of p, seed low, seed high} in device memory)
+  const uint32_t *sample;
   const uint16_t *gemv_res; // stand-alone product (PH_GEMV): residual operand or null
   int stream_once; // the weights of a step exceed the caches: request them non-temporally
 #ifdef VKL_TRACE
@@ -492,5 +495,10 @@ int launch_layer (const Params &p, const vkl_layer_weights &lw, int layer, int G
 // the token's embedding row -> residual stream (one small launch in front of layer 0)
 int launch_embed_row (const Params &p, hipStream_t s);
 } // namespace dec
+// vkl_sample.hip: the draw that ends a step of a replayed loop; dev_params =
+// {k, bits of p, seed low, seed high} in device memory, loop = {index,
+// position}: writes ids[index + 1] and advances both loop words
+int sample_loop_launch (const float *logits, int V, const uint32_t *dev_params, uint32_t *loop,
+                        uint32_t *ids, hipStream_t s);
 } // namespace vkl
 #endif

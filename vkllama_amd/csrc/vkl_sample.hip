@@ -61,11 +61,27 @@ struct SampleArgs
   uint32_t *cand_ids; // optional: candidates of this draw, most likely first
   float *cand_probs;
   uint32_t *cand_n;
+  // a step of a replayed decode loop (all three set): k, p and the seed come
+  // from `dev` = {k, bits of p, seed low, seed high} in device memory, so that
+  // one captured launch serves every request; loop = {index into ids,
+  // position}; the token of position + 1 goes to ids[index + 1], drawn with
+  // that position as the counter, and both loop words advance
+  const uint32_t *dev;
+  uint32_t *loop;
+  uint32_t *ids;
 };
 
 __global__ __launch_bounds__ (kSampThreads) void
-sample_kernel (const SampleArgs a)
+sample_kernel (const SampleArgs args)
 {
+  SampleArgs a = args;
+  if (a.dev)
+    {
+      a.p = __uint_as_float (vkl::ldg (a.dev + 1));
+      const int k = (int)vkl::ldg (a.dev);
+      a.k = a.p >= 0.f ? kMaxCand : (k > kMaxCand ? kMaxCand : max (k, 1));
+      a.seed = (uint64_t)vkl::ldg (a.dev + 2) | ((uint64_t)vkl::ldg (a.dev + 3) << 32);
+    }
   __shared__ uint32_t hist[256];
   __shared__ uint64_t cand[kMaxCand];
   __shared__ uint64_t prefix_s;
@@ -184,7 +200,13 @@ sample_kernel (const SampleArgs a)
   float sum = 0.f;
   for (int i = 0; i < n; ++i)
     sum += ex[i];
-  const uint32_t ctr = a.counter + (a.counter_dev ? vkl::ldg (a.counter_dev) : 0u);
+  uint32_t ctr = a.counter + (a.counter_dev ? vkl::ldg (a.counter_dev) : 0u);
+  uint32_t index = 0, position = 0;
+  if (a.loop)
+    {
+      index = vkl::ldg (a.loop), position = vkl::ldg (a.loop + 1);
+      ctr = a.counter + position + 1u;
+    }
   const float target = uniform01 (a.seed, ctr);
   float cum = 0.f;
   int pick = -1;
@@ -203,9 +225,32 @@ sample_kernel (const SampleArgs a)
     pick = n - 1;
   if (a.cand_n)
     *a.cand_n = (uint32_t)n;
-  *a.tok = 0xffffffffu - (uint32_t)cand[pick];
+  const uint32_t drawn = 0xffffffffu - (uint32_t)cand[pick];
+  if (a.loop)
+    {
+      a.ids[index + 1] = drawn;
+      a.loop[0] = index + 1u, a.loop[1] = position + 1u;
+    }
+  else
+    *a.tok = drawn;
 }
 } // namespace
+
+namespace vkl
+{
+// the draw of a replayed decode step (see SampleArgs::dev)
+int
+sample_loop_launch (const float *logits, int V, const uint32_t *dev_params, uint32_t *loop,
+                    uint32_t *ids, hipStream_t s)
+{
+  SampleArgs a = {};
+  a.logits = logits, a.V = V;
+  a.k = 1, a.p = -1.f;
+  a.dev = dev_params, a.loop = loop, a.ids = ids;
+  sample_kernel<<<dim3 (1), dim3 (kSampThreads), 0, s>>> (a);
+  return 0;
+}
+}
 
 extern "C" int
 vkl_sample_f32 (const float *logits, int V, int k, float p, uint64_t seed,
@@ -216,7 +261,7 @@ vkl_sample_f32 (const float *logits, int V, int k, float p, uint64_t seed,
   VKL_CHECK_ARG (logits && tok && V > 0);
   VKL_CHECK_ARG (p >= 0.f || k >= 1);
   VKL_CHECK_ARG (p < 0.f || p <= 1.0f);
-  SampleArgs a;
+  SampleArgs a = {};
   a.logits = logits, a.V = V;
   a.k = p >= 0.f ? kMaxCand : (k > kMaxCand ? kMaxCand : k);
   a.p = p, a.seed = seed, a.counter = counter, a.counter_dev = counter_dev;

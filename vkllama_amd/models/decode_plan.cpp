@@ -176,6 +176,20 @@ DecodePlan::loop (uint32_t *ids, size_t pos0, size_t n_steps)
                                       gpu_->stream ()));
 }
 
+absl::Status
+DecodePlan::loop_sampled (uint32_t *ids, size_t pos0, size_t n_steps, int topk, float topp,
+                          uint64_t seed)
+{
+  if (!usable_)
+    return absl::FailedPreconditionError (
+        "fused decode does not cover this model");
+  adopted_valid_ = false;
+  return hip_status ("sampled decode loop",
+                     vkl_decode_loop_sampled (&desc_, ids, (uint32_t)pos0, (int)n_steps, mode_,
+                                              (float *)logits32_.data (), topk, topp, seed,
+                                              gpu_->stream ()));
+}
+
 bool
 DecodePlan::set_option (const char *name, int value)
 {

@@ -38,6 +38,10 @@ struct DecodePlan
   // n_steps greedy tokens replayed from a captured graph (vkl_decode_loop);
   // ids is device memory, ids[0] the first input token
   absl::Status loop (uint32_t *ids, size_t pos0, size_t n_steps);
+  // the same with a draw from the top-k / top-p candidates instead of the
+  // arg-max at the end of every replayed step (vkl_decode_loop_sampled)
+  absl::Status loop_sampled (uint32_t *ids, size_t pos0, size_t n_steps, int topk,
+                             float topp, uint64_t seed);
   int mode () const { return mode_; }
   // After the stream has been synchronised: did a wait between workgroups
   // inside a launch give up (vkl_decode_status)?  If so the plan switches to

@@ -561,10 +561,18 @@ Model::generate_once_ (std::vector<uint32_t> const &prompt, size_t n_gen,
   const auto t1 = clock::now ();
   size_t n_toks = prompt.size () + 1;
   size_t i0 = 1;
-  if (fused_decode_ && plan_->usable () && decode_graph_ && n_gen > 1 && !samp_on_)
+  if (fused_decode_ && plan_->usable () && decode_graph_ && n_gen > 1)
     {
       // ids[0] is at position prompt.size (); each replay appends one id
-      VKLLAMA_STATUS_OK (plan_->loop (ids, prompt.size (), n_gen - 1));
+      if (samp_on_)
+        {
+          VKLLAMA_STATUS_OK (plan_->loop_sampled (ids, prompt.size (), n_gen - 1, samp_k_,
+                                                  samp_p_, samp_seed_));
+        }
+      else
+        {
+          VKLLAMA_STATUS_OK (plan_->loop (ids, prompt.size (), n_gen - 1));
+        }
       i0 = n_gen;
     }
   for (size_t i = i0; i < n_gen; ++i, ++n_toks)
