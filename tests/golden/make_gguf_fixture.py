@@ -43,24 +43,28 @@ def build():
         kv("x.i32s", ARRAY, struct.pack("<IQ", I32, 2) + struct.pack("<ii", -7, 9)),
     ]
     # tensor infos: name, uint32 n_dims, uint64 dims (innermost first), uint32 ggml type, uint64 offset into the data
-    # section.  An F32 vector of 4 weights, and a Q8_0 matrix of 2 rows x 32 columns (one 34-byte block per row).
+    # section.  An F32 vector of 4 weights, a Q8_0 matrix of 2 rows x 32 columns (one 34-byte block per row), and an
+    # F16 matrix of 2 rows x 3 columns.
     norm = struct.pack("<4f", 1.0, -2.0, 0.5, 3.25)
     blocks = b""
     for row in range(2):
         scale = struct.pack("<e", 0.25 * (row + 1))                 # fp16 d
         quants = bytes((i * (row + 1) - 16) & 0xff for i in range(32))   # int8 q[32]
         blocks += scale + quants
+    halves = struct.pack("<6e", 1.0, -0.5, 65504.0, 6.1035e-05, 0.0, -2.75)   # row 0, then row 1
     infos = (gstr("output_norm.weight") + struct.pack("<I", 1) + struct.pack("<Q", 4) + struct.pack("<IQ", 0, 0)
              + gstr("blk.0.attn_q.weight") + struct.pack("<I", 2) + struct.pack("<QQ", 32, 2)
-             + struct.pack("<IQ", 8, 32))                            # second tensor at the next multiple of 32
-    head = b"GGUF" + struct.pack("<I", 3) + struct.pack("<Q", 2) + struct.pack("<Q", len(kvs)) + b"".join(kvs) + infos
+             + struct.pack("<IQ", 8, 32)                             # second tensor at the next multiple of 32
+             + gstr("blk.0.attn_k.weight") + struct.pack("<I", 2) + struct.pack("<QQ", 3, 2)
+             + struct.pack("<IQ", 1, 128))                           # 32 + 68 bytes of blocks, padded to 128
+    head = b"GGUF" + struct.pack("<I", 3) + struct.pack("<Q", 3) + struct.pack("<Q", len(kvs)) + b"".join(kvs) + infos
     head += b"\0" * ((-len(head)) % 32)
-    data = norm + b"\0" * 16 + blocks
-    return head + data, norm, blocks
+    data = norm + b"\0" * 16 + blocks + b"\0" * 28 + halves
+    return head + data, norm, blocks, halves
 
 
 if __name__ == "__main__":
-    raw, _, _ = build()
+    raw, _, _, _ = build()
     with open(os.path.join(HERE, "handmade_v3.gguf"), "wb") as f:
         f.write(raw)
     print("handmade_v3.gguf:", len(raw), "bytes")

@@ -69,7 +69,7 @@ def test_reader_on_a_file_this_repository_did_not_write():
     assert k["tokenizer.ggml.tokens"][0] == 9 and k["x.i32s"][0] == 9
     assert len(k) == 13
     t = g["tensors"]
-    assert list(t) == ["output_norm.weight", "blk.0.attn_q.weight"]
+    assert list(t) == ["output_norm.weight", "blk.0.attn_q.weight", "blk.0.attn_k.weight"]
     n = t["output_norm.weight"]
     assert n["type"] == 0 and n["dims"] == [4] and n["bsize"] == 16
     assert list(n["data"].view(np.float32)) == [1.0, -2.0, 0.5, 3.25]
@@ -79,6 +79,11 @@ def test_reader_on_a_file_this_repository_did_not_write():
         blk = q["data"][34 * row:34 * row + 34]
         assert blk[:2].view(np.float16)[0] == np.float16(0.25 * (row + 1))
         assert list(blk[2:].view(np.int8)) == [((i * (row + 1) - 16 + 128) % 256) - 128 for i in range(32)]
+    # an F16 matrix of 2 rows x 3 columns behind the padding: 1, -0.5, the largest
+    # and the smallest normal value, zero, -2.75, as their bit patterns
+    h = t["blk.0.attn_k.weight"]
+    assert h["type"] == 1 and h["dims"] == [3, 2] and h["bsize"] == 12
+    assert h["data"].view(np.uint16).tolist() == [0x3C00, 0xB800, 0x7BFF, 0x0400, 0x0000, 0xC180]
 
 
 def test_malformed_files_are_refused(model_file, tmp_path):
