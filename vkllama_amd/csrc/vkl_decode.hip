@@ -47,8 +47,16 @@ attn_split_min (const vkl_decode_model &m)
 // workgroup held up the heads' atomics); all zeroed by the layer's K/Q/V phase
 // (each on a cache line of its own, clear of the words the persistent mode uses)
 constexpr int kSyncAttnDone = 32;
+constexpr int kSyncHeadDone = 64; // workgroups of the lm_head launch whose arg-max partials are in memory
 constexpr int kSyncAttnFlag = 768; // + 32 * slot
 constexpr int kFuseSpinLimit = 1 << 13; // some 10 ms; a head takes microseconds
+
+// the lm_head launch ends with the arg-max (not when a sampler follows it)
+__host__ __device__ __forceinline__ bool
+head_picks_token (const Params &p)
+{
+  return (p.next_tok || p.loop) && !p.sample;
+}
 
 __device__ __forceinline__ void
 reset_attn_done (const Params &p, int wg)
@@ -219,9 +227,7 @@ run_phase (const Params &p, const vkl_layer_weights &lw, int layer, int phase,
         GV::run (ps, A, B, xl, e, red);
         break;
       }
-    case PH_ARGMAX:
-      if (wg == 0 && (p.next_tok || p.loop))
-        final_argmax<false> (p, G, lds);
+    default: // (PH_ARGMAX: the lm_head launch picks the token itself)
       break;
     }
   VKL_TR (4);
@@ -339,6 +345,32 @@ run_phase_direct (const Params &p, const vkl_layer_weights &lw, int layer,
     }
   GV::run (ps, A, B, xl, e, red);
   VKL_TR (4);
+  if (PHASE == PH_HEAD && head_picks_token (p))
+    {
+      // The launch's last workgroup picks the token (no wait: every workgroup
+      // counts in once its partials are in memory and only the last one goes
+      // on), hands it to the next step and, in a replayed loop, starts the
+      // next step's residual stream with the token's embedding row.
+      __builtin_amdgcn_s_waitcnt (0x0f70); // vmcnt(0)
+      __syncthreads ();
+      uint32_t *last = (uint32_t *)red;
+      if (threadIdx.x == 0)
+        {
+          uint32_t *done = p.s.sync + kSyncHeadDone;
+          const uint32_t old
+              = __hip_atomic_fetch_add (done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          *last = old + 1u == (uint32_t)G ? 1u : 0u;
+          if (old + 1u == (uint32_t)G)
+            st_coherent_u32 (done, 0u);
+        }
+      __syncthreads ();
+      if (*last == 0u)
+        return;
+      __syncthreads ();
+      const uint32_t id = final_argmax<true> (p, G, lds);
+      if (p.loop)
+        embed_row<WT> (p, id, 0, 1);
+    }
 }
 
 template <int PHASE, int WT, int XCH, bool NT>
@@ -996,7 +1028,9 @@ launch_step (const Params &p, const vkl_decode_model *m, int mode, int n_cu, int
   // the split attention take the launches per phase)
   const bool per_layer = mode == 1 && layer_launch_supported (*m, G)
                          && (int)p.pos + 1 < attn_split_min (*m);
-  if (per_layer)
+  // (in a replayed greedy loop the previous step's lm_head launch has left the
+  // row; the loop launches this once in front of its first step)
+  if (per_layer && !(p.loop && !p.sample))
     if (int e = launch_embed_row (p, s))
       return e;
   for (int l = 0; l < m->n_layers; ++l)
@@ -1036,9 +1070,7 @@ launch_step (const Params &p, const vkl_decode_model *m, int mode, int n_cu, int
     return e;
   if (p.loop && p.sample)
     return sample_loop_launch (p.logits32, m->vocab, p.sample, (uint32_t *)p.loop, p.ids, s);
-  if (p.next_tok || p.loop)
-    if (int e = launch_phase<PH_ARGMAX> (p, none, 0, 1, G, lds, s))
-      return e;
+  // (otherwise the lm_head launch has picked the token: head_picks_token)
   return 0;
 }
 
@@ -1256,6 +1288,8 @@ decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0, int n_step
     set_sample_params_kernel<<<dim3 (1), dim3 (1), 0, s>>> (p.s.sync + 20, (uint32_t)topk,
                                                             __builtin_bit_cast (uint32_t, topp),
                                                             (uint32_t)seed, (uint32_t)(seed >> 32));
+  else if (mode == 1 && layer_launch_supported (*m, G))
+    launch_embed_row (p, s); // the first step's row; every step leaves the next one's
   int err = 0;
   int done = 0;
   while (done < n_steps && !err)

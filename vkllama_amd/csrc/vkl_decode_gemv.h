@@ -704,8 +704,9 @@ template <int WT = 8, bool NT = false, int RU = 2> struct Gemv
             for (int w = 1; w < kDecWaves; ++w)
               if (better (bv[w], bi[w], v, i))
                 v = bv[w], i = bi[w];
-            stg ((uint32_t *)(e.amax_val + ps.wg), __float_as_uint (v));
-            stg (e.amax_idx + ps.wg, i);
+            // (written through: the launch's last workgroup may read them)
+            st_coherent_u32 ((uint32_t *)(e.amax_val + ps.wg), __float_as_uint (v));
+            st_coherent_u32 (e.amax_idx + ps.wg, i);
           }
       }
   }

@@ -526,36 +526,7 @@ template <int WT>
 __global__ __launch_bounds__ (kDecThreads) void
 embed_row_kernel (const Params p)
 {
-  const int dim = p.m.dim;
-  uint32_t tok = ldg (step_tok (p));
-  if (tok >= (uint32_t)p.m.vocab)
-    tok = 0;
-  for (int i = (int)(blockIdx.x * kDecThreads + threadIdx.x) * 8; i < dim;
-       i += (int)(gridDim.x * kDecThreads) * 8)
-    {
-      uint32_t o[4];
-      if (WT == 8)
-        {
-          const QMat tab = qmat (p.m.tok_embd, p.m.vocab, dim);
-          const unsigned long long q
-              = ldg ((const unsigned long long *)(tab.q + (size_t)tok * dim + i));
-          const float sc = h2f (ldg (tab.d + (size_t)tok * (dim >> 5) + (i >> 5)));
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            {
-              const int8_t b0 = (int8_t)((q >> (16 * j)) & 0xff);
-              const int8_t b1 = (int8_t)((q >> (16 * j + 8)) & 0xff);
-              o[j] = (uint32_t)f2h ((float)b0 * sc) | ((uint32_t)f2h ((float)b1 * sc) << 16);
-            }
-        }
-      else
-        {
-          const uint4 v = ldg4 ((const uint16_t *)p.m.tok_embd + (size_t)tok * dim + i);
-          o[0] = v.x, o[1] = v.y, o[2] = v.z, o[3] = v.w;
-        }
-      uint32_t *dst = (uint32_t *)(p.s.x + i);
-      stg (dst, o[0]), stg (dst + 1, o[1]), stg (dst + 2, o[2]), stg (dst + 3, o[3]);
-    }
+  embed_row<WT> (p, ldg (step_tok (p)), (int)blockIdx.x, (int)gridDim.x);
 }
 
 template <int WT, int XD, int XF, bool NT>

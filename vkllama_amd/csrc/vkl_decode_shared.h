@@ -437,8 +437,45 @@ lds_bytes_needed (int dim, int ffn, int maxlen, int hd)
 }
 
 
-template <bool COH>
+// the token's embedding row -> x (residual stream) by all threads of a
+// workgroup: nblk workgroups share the row
+template <int WT>
 __device__ __forceinline__ void
+embed_row (const Params &p, uint32_t tok, int blk, int nblk)
+{
+  const int dim = p.m.dim;
+  if (tok >= (uint32_t)p.m.vocab)
+    tok = 0;
+  for (int i = (int)(blk * kDecThreads + threadIdx.x) * 8; i < dim; i += nblk * kDecThreads * 8)
+    {
+      uint32_t o[4];
+      if (WT == 8)
+        {
+          const QMat tab = qmat (p.m.tok_embd, p.m.vocab, dim);
+          const unsigned long long q
+              = ldg ((const unsigned long long *)(tab.q + (size_t)tok * dim + i));
+          const float sc = h2f (ldg (tab.d + (size_t)tok * (dim >> 5) + (i >> 5)));
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            {
+              const int8_t b0 = (int8_t)((q >> (16 * j)) & 0xff);
+              const int8_t b1 = (int8_t)((q >> (16 * j + 8)) & 0xff);
+              o[j] = (uint32_t)f2h ((float)b0 * sc) | ((uint32_t)f2h ((float)b1 * sc) << 16);
+            }
+        }
+      else
+        {
+          const uint4 v = ldg4 ((const uint16_t *)p.m.tok_embd + (size_t)tok * dim + i);
+          o[0] = v.x, o[1] = v.y, o[2] = v.z, o[3] = v.w;
+        }
+      uint32_t *dst = (uint32_t *)(p.s.x + i);
+      stg (dst, o[0]), stg (dst + 1, o[1]), stg (dst + 2, o[2]), stg (dst + 3, o[3]);
+    }
+}
+
+// Returns the id to every thread (through LDS).
+template <bool COH>
+__device__ __forceinline__ uint32_t
 final_argmax (const Params &p, int G, uint8_t *lds)
 {
   // G per-workgroup partials -> first maximum
@@ -484,7 +521,10 @@ final_argmax (const Params &p, int G, uint8_t *lds)
         }
       else
         stg (p.next_tok, id);
+      bi[kDecWaves] = id;
     }
+  __syncthreads ();
+  return bi[kDecWaves];
 }
 
 // One layer of the step as a single launch (vkl_decode_layer.hip): K/Q/V,
