@@ -138,10 +138,12 @@ int vkl_argmax_f32 (const float *x, int n, uint32_t *out, void *stream);
  * src/core/gpu_device.cpp).  While enabled, vkl_decode_step brackets every
  * phase launch with a pair of HIP events on the launch stream and
  * synchronises the stream before it returns.  vkl_decode_phase_times adds up,
- * per phase kind (0 K/Q/V, 1 attention, 2 Wo, 3 up/gate, 4 down, 5 lm_head,
- * 6 arg-max, 8 a whole layer in one launch as mode 1 runs it; 7 is not
- * used), the elapsed milliseconds and the number of launches since the last
- * call, and clears both. */
+ * per phase kind (0 K/Q/V, 1 attention, 2 Wo, 3 up/gate, 4 down, 5 lm_head
+ * with the arg-max its last workgroup forms, 8 a whole layer in one launch as
+ * mode 1 runs it; 6 and 7 are not used), the elapsed milliseconds and the
+ * number of launches since the last call, and clears both.  The timer is one
+ * per process: use it from one host thread, with no other decode call in
+ * flight. */
 #define VKL_DECODE_PHASES 9
 #define VKL_DECODE_PHASE_LAYER 8
 int vkl_decode_phase_timing (int enable);

@@ -30,6 +30,36 @@ vkl_launch_status ()
   return (int)hipGetLastError ();
 }
 
+#include <mutex>
+namespace vkl
+{
+// The dynamic-LDS limit of one kernel, raised when a launch needs more than
+// any launch before it on that device (a function attribute is kept per
+// device); safe to call from several host threads.
+struct LdsLimit
+{
+  std::mutex mu;
+  size_t set[16] = {};
+  int
+  raise (const void *kernel, size_t bytes)
+  {
+    int dev = 0;
+    if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
+      return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock (mu);
+    if (bytes > set[dev])
+      {
+        const hipError_t e
+            = hipFuncSetAttribute (kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess)
+          return (int)e;
+        set[dev] = bytes;
+      }
+    return 0;
+  }
+};
+}
+
 typedef _Float16 h16;
 typedef _Float16 h16x2 __attribute__ ((ext_vector_type (2)));
 

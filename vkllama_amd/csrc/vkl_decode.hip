@@ -815,14 +815,9 @@ launch_phase_wt (const Params &p, const vkl_layer_weights &lw, int layer,
   if (PHASE == PH_WO || PHASE == PH_UPGATE || PHASE == PH_DOWN || PHASE == PH_HEAD
       || PHASE == PH_GEMV || (PHASE == PH_KQV && layer > 0))
     return launch_direct<PHASE, WT> (p, lw, layer, grid, G, lds, s);
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_kernel<PHASE, WT>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
+  static LdsLimit limit;
+  if (int e = limit.raise ((const void *)decode_phase_kernel<PHASE, WT>, lds))
+    return e;
   decode_phase_kernel<PHASE, WT>
       <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer,
                                                                  G);
@@ -836,14 +831,9 @@ int
 launch_direct_nt (const Params &p, const vkl_layer_weights &lw, int layer,
                   int grid, int G, size_t lds, hipStream_t s)
 {
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute (
-          (const void *)decode_phase_direct_kernel<PHASE, WT, XCH, NT>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
+  static LdsLimit limit;
+  if (int e = limit.raise ((const void *)decode_phase_direct_kernel<PHASE, WT, XCH, NT>, lds))
+    return e;
   decode_phase_direct_kernel<PHASE, WT, XCH, NT>
       <<<dim3 ((unsigned)grid), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G);
   return 0;
@@ -911,13 +901,9 @@ int
 launch_attn_wo_xch (const Params &p, const vkl_layer_weights &lw, int layer, int G, size_t lds,
                     hipStream_t s)
 {
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute ((const void *)decode_attn_wo_kernel<WT, XCH>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
+  static LdsLimit limit;
+  if (int e = limit.raise ((const void *)decode_attn_wo_kernel<WT, XCH>, lds))
+    return e;
   decode_attn_wo_kernel<WT, XCH>
       <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G - p.m.n_heads);
   return 0;
@@ -1214,6 +1200,7 @@ struct StepGraph
 constexpr int kStepGraphs = 8;
 StepGraph g_graphs[kStepGraphs];
 uint64_t g_graph_clock = 0;
+std::mutex g_graph_mu; // the cache above: loops of several host threads take turns
 
 uint64_t
 hash_model (const vkl_decode_model *m)
@@ -1280,6 +1267,7 @@ decode_loop (const vkl_decode_model *m, uint32_t *ids, uint32_t pos0, int n_step
   p.trace = nullptr;
 #endif
   const int G = n_cu * 2;
+  std::lock_guard<std::mutex> lock (g_graph_mu);
   const bool timing = g_timer.on;
   g_timer.on = false;
   const uint64_t mh = hash_model (m);

@@ -536,13 +536,9 @@ launch_layer_t (const Params &p, const vkl_layer_weights &lw, int layer, int G,
 {
   const size_t at = (lds_bytes_needed (p.m.dim, p.m.ffn, p.m.maxlen, p.m.head_dim) + 15) & ~(size_t)15;
   const size_t lds = at + 16;
-  static size_t lds_set = 0;
-  if (lds > lds_set)
-    {
-      VKL_HIP (hipFuncSetAttribute ((const void *)decode_layer_kernel<WT, XD, XF, NT>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set = lds;
-    }
+  static LdsLimit limit;
+  if (int e = limit.raise ((const void *)decode_layer_kernel<WT, XD, XF, NT>, lds))
+    return e;
   decode_layer_kernel<WT, XD, XF, NT>
       <<<dim3 ((unsigned)G), dim3 (kDecThreads), lds, s>>> (p, lw, layer, G, at);
   return 0;

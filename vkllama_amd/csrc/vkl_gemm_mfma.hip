@@ -1086,19 +1086,8 @@ template <int WT>
 bool
 skinny2_prepare (size_t lds)
 {
-  static bool lds_set[16] = {};
-  int dev = 0;
-  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
-    return false;
-  if (!lds_set[dev])
-    {
-      if (hipFuncSetAttribute ((const void *)gemm_skinny2_kernel<WT>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-          != hipSuccess)
-        return false;
-      lds_set[dev] = true;
-    }
-  return true;
+  static LdsLimit limit;
+  return limit.raise ((const void *)gemm_skinny2_kernel<WT>, lds) == 0;
 }
 
 // the whole-line form for Q8_0 weights
@@ -1112,21 +1101,10 @@ launch_rows64_q8 (const GemmArgs &a, hipStream_t s, int &err)
   const size_t need = (size_t)nm * S * 32 * a.N * sizeof (float);
   if (need > kSk2Workspace || (a.workspace && need > a.workspace_bytes))
     return false;
-  static bool lds_set[16] = {};
-  int dev = 0;
-  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
+  static LdsLimit limit64, limit128;
+  if (limit64.raise ((const void *)gemm_rows64_q8_kernel, kR64Lds) != 0
+      || limit128.raise ((const void *)gemm_rows128_q8_kernel, kR128Lds) != 0)
     return false;
-  if (!lds_set[dev])
-    {
-      if (hipFuncSetAttribute ((const void *)gemm_rows64_q8_kernel,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kR64Lds)
-              != hipSuccess
-          || hipFuncSetAttribute ((const void *)gemm_rows128_q8_kernel,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kR128Lds)
-                 != hipSuccess)
-        return false;
-      lds_set[dev] = true;
-    }
   float *ws = a.workspace ? a.workspace : skinny2_workspace (s);
   if (!ws)
     return false;
@@ -1418,6 +1396,7 @@ gemm_static_scratch (size_t *bytes)
   int dev = 0;
   if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
     return nullptr;
+  std::lock_guard<std::mutex> lock (g_ws_mu);
   if (!g_static_scratch[dev])
     {
       // with this device current: the address of ITS copy of the array

@@ -407,18 +407,11 @@ template <int G, int KS, int NL, int DX, int DW, int TB, bool UPGATE>
 int
 rowsfull_run (const GemmArgs &a, int groups, int gpm, int vec, hipStream_t s)
 {
-  static bool lds_set[16] = {};
-  int dev = 0;
-  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
-    return (int)hipErrorInvalidDevice;
   constexpr size_t lds = rowsfull_lds<G, KS, DX, DW, TB> ();
   static_assert (lds <= 160 * 1024, "a workgroup's LDS");
-  if (!lds_set[dev])
-    {
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_rowsfull_q8_kernel<G, KS, NL, DX, DW, TB, UPGATE>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      lds_set[dev] = true;
-    }
+  static LdsLimit limit;
+  if (int e = limit.raise ((const void *)gemm_rowsfull_q8_kernel<G, KS, NL, DX, DW, TB, UPGATE>, lds))
+    return e;
   constexpr int per = UPGATE ? G / 2 : G;
   const dim3 grid ((unsigned)((groups + per - 1) / per));
   gemm_rowsfull_q8_kernel<G, KS, NL, DX, DW, TB, UPGATE><<<grid, dim3 ((KS + NL) * 64), lds, s>>> (a, groups, gpm, vec);

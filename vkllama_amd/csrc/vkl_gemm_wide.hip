@@ -703,32 +703,18 @@ gemm_wide_workspace_bytes (const GemmArgs &a)
 int
 gemm_wide_launch (const GemmArgs &a, hipStream_t s)
 {
-  static bool lds_set[16] = {};
-  int dev = 0;
-  if (hipGetDevice (&dev) != hipSuccess || dev < 0 || dev >= 16)
-    return (int)hipErrorInvalidDevice;
   constexpr size_t lds256 = wide_lds_f16<256> (), lds128 = wide_lds_f16<128> ();
   constexpr size_t q256 = wide_lds_q8<256> (), q128 = wide_lds_q8<128> ();
-  if (!lds_set[dev])
-    {
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<256, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<256, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_f16_kernel<128, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, QGRID, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<256, QGRID, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q256));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, QGRID, false>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
-      VKL_HIP (hipFuncSetAttribute ((const void *)gemm_wide_q8_kernel<128, QGRID, true>,
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)q128));
-      lds_set[dev] = true;
-    }
+  static LdsLimit limits[8];
+  const void *const kernels[8]
+      = { (const void *)gemm_wide_f16_kernel<256, false>,       (const void *)gemm_wide_f16_kernel<256, true>,
+          (const void *)gemm_wide_f16_kernel<128, false>,       (const void *)gemm_wide_f16_kernel<128, true>,
+          (const void *)gemm_wide_q8_kernel<256, QGRID, false>, (const void *)gemm_wide_q8_kernel<256, QGRID, true>,
+          (const void *)gemm_wide_q8_kernel<128, QGRID, false>, (const void *)gemm_wide_q8_kernel<128, QGRID, true> };
+  const size_t need[8] = { lds256, lds256, lds128, lds128, q256, q256, q128, q128 };
+  for (int i = 0; i < 8; ++i)
+    if (int e = limits[i].raise (kernels[i], need[i]))
+      return e;
   const WidePlan plan = wide_plan (a);
   const int bm = plan.bm;
   int ksplit = plan.ksplit;
