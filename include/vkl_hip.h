@@ -200,7 +200,8 @@ int vkl_rope_kvwrite_f16 (void *q, const void *k, const void *v, int S, int H,
  * probabilities stored.  Scores and output are rounded to fp16 where the
  * shaders round them; the softmax runs with a running maximum and the
  * division by the sum of exponentials last, so the fp16 weights of the second
- * product are exp(score - max) instead of the normalised probabilities
+ * product are exp(score - max) instead of the normalised probabilities and
+ * the sum adds them as rounded
  * (outputs within 5e-3 of the three shaders' relative to the size of the terms
  * summed; the operators' bar is 1e-2).  q [H,S,hd] with strides (qcs,
  * qhs); k, v [H,L,hd] views with strides (kcs, khs), (vcs, vhs), e.g. the

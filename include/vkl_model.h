@@ -77,7 +77,9 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
  * "attn_split_min" (the context length from which attention is split over
  * several workgroups per head), "fuse_attn_wo" (mode 0: attention and the Wo
  * projection in one launch on/off), "lastblock_rope_quirk" (the reference's
- * last-block RoPE position), "wait_test" (a testing aid: waits between
+ * last-block RoPE position), "operator_attention" (prompt pass: scores,
+ * softmax and P V as the reference's three operators with probabilities
+ * rounded to fp16 one by one, instead of the one-launch attention), "wait_test" (a testing aid: waits between
  * workgroups inside a launch give up after that many polls and are never
  * answered; 0 = normal), "phase_timing" (process-wide measuring aid) */
 int vkl_model_set_option (vkl_model *m, const char *name, int value);

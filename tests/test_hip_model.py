@@ -218,6 +218,31 @@ def test_fp16_weights_model(fused):
     m.close()
 
 
+def test_operator_attention_option(small):
+    """Option "operator_attention": the attention of a prompt pass as the
+    reference's three operators (scores, masked softmax with probabilities
+    rounded to fp16 one by one, P V; multiheadattention_v2.cpp:272-317)
+    instead of the one-launch attention with its running maximum.  RoPE and
+    cache rows do not depend on the form (bit-identical caches), both forms
+    meet the oracle's logits, and the greedy ids are the oracle's either way."""
+    cfg, w = small
+    prompt = np.random.default_rng(3).integers(3, cfg["vocab"], 37).astype(np.uint32)
+    om = O.OracleModel(cfg, w)
+    want = om.forward(prompt, 0)
+    a, b = M.Llama2(cfg, w), M.Llama2(cfg, w)
+    b.set_option("operator_attention", 1)
+    la, lb = a.forward(prompt, 0), b.forward(prompt, 0)
+    assert logit_err(la, want) < 1e-2 and logit_err(lb, want) < 1e-2
+    assert not np.array_equal(la, lb)                       # two forms, two roundings
+    assert np.array_equal(a.read_kv_cache(0, 0), b.read_kv_cache(0, 0))
+    assert np.array_equal(a.read_kv_cache(0, 1), b.read_kv_cache(0, 1))
+    ids, _ = om.generate_greedy(prompt, 8)
+    assert list(b.generate_greedy(prompt, 8)[0]) == list(ids)
+    b.set_option("operator_attention", 0)
+    assert np.array_equal(b.forward(prompt, 0), la)
+    a.close(), b.close(), om.close()
+
+
 def test_errors(small):
     cfg, w = small
     m = M.Llama2(cfg, w)

@@ -292,9 +292,12 @@ attn_prefill_kernel (const AttnArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           {
-            const float e = fast_exp (sv[blk][r] - m); // exp (kNeg - m) = 0
-            sum += e;
-            pf[blk][r >> 3][r & 7] = (_Float16)e;
+            // exp (kNeg - m) = 0.  The sum takes the weight as the product
+            // below consumes it, rounded to fp16: the weights then add up to
+            // one exactly.
+            const _Float16 e = (_Float16)fast_exp (sv[blk][r] - m);
+            sum += (float)e;
+            pf[blk][r >> 3][r & 7] = e;
           }
 #pragma unroll
       for (int db = 0; db < DB; ++db)

@@ -221,6 +221,8 @@ vkl_model_set_option (vkl_model *m, const char *name, int value)
     m->model->set_fused_decode (value != 0);
   else if (n == "lastblock_rope_quirk")
     m->model->set_lastblock_rope_quirk (value != 0);
+  else if (n == "operator_attention")
+    m->model->set_operator_attention (value != 0);
   else if (n == "decode_mode")
     m->model->set_decode_mode (value);
   else if (n == "decode_graph")

@@ -369,6 +369,13 @@ Model::set_decode_option (const char *name, int value)
 }
 
 void
+Model::set_operator_attention (bool on)
+{
+  for (auto *b : blocks_)
+    b->attention ()->set_operator_attention (on);
+}
+
+void
 Model::set_lastblock_rope_quirk (bool on)
 {
   for (auto *b : blocks_)

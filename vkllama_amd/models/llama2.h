@@ -12,7 +12,9 @@
 //    the logits, lowest index on ties) so that a decode loop needs no
 //    128 KB logits download per token;
 //  - set_lastblock_rope_quirk(false) rotates the last block's clipped query
-//    at its true position instead of the reference's `offset`.
+//    at its true position instead of the reference's `offset`;
+//  - set_operator_attention(true) runs the attention of a prompt pass as the
+//    reference's three operators with their rounding points.
 #ifndef __VKLLAMA_MODELS_LLAMA2_H__
 #define __VKLLAMA_MODELS_LLAMA2_H__
 // clang-format off
@@ -157,6 +159,9 @@ public:
   // ---- additions -----------------------------------------------------------
   void set_fused_decode (bool on) { fused_decode_ = on; }
   void set_lastblock_rope_quirk (bool on);
+  // prompt pass: attention as the reference's three operators (see
+  // MultiHeadAttentionV2::set_operator_attention)
+  void set_operator_attention (bool on);
   // 0 = one launch per decode phase, 1 = one launch per layer
   void set_decode_mode (int mode);
   // options of the fused decode steps: "attn_split_min", "fuse_attn_wo",

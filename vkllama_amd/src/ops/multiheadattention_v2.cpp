@@ -189,7 +189,7 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
   // scores and outputs where the operators do but forms its softmax with a
   // running maximum (see vkl_attn_prefill_causal_f16).
   attn_fused_last_ = false;
-  if (use_kvcache_ && dtype_ == FP16 && (dim_ == 64 || dim_ == 128)
+  if (!operator_attention_ && use_kvcache_ && dtype_ == FP16 && (dim_ == 64 || dim_ == 128)
       && k.dtype () == FP16 && q.dtype () == FP16 && v.dtype () == FP16)
     {
       const int q_row0 = clip_output_ ? (int)S - 1 : 0;
@@ -274,8 +274,8 @@ MultiHeadAttentionV2::operator() (Tensor X, const size_t offset) noexcept
   // heads*dim]: the three operators below without the [heads, seqlen,
   // read_len] tensors in memory (online softmax: outputs within 5e-3 of
   // theirs relative to the size of the terms summed)
-  if (dtype_ == FP16 && (dim_ == 64 || dim_ == 128) && roped_q->dtype () == FP16
-      && roped_k->dtype () == FP16 && transposed_v->dtype () == FP16)
+  if (!operator_attention_ && dtype_ == FP16 && (dim_ == 64 || dim_ == 128)
+      && roped_q->dtype () == FP16 && roped_k->dtype () == FP16 && transposed_v->dtype () == FP16)
     {
       const size_t Sq = roped_q->height (), Lk = roped_k->height ();
       if (!(attn_out_.channels () == 1 && attn_out_.height () == Sq

@@ -36,6 +36,10 @@ public:
   // `offset` instead of offset + rows - 1 (multiheadattention_v2.cpp:222-233,
   // 251 with rope_fp16.comp:34).  true (default) reproduces that.
   void set_lastblock_rope_quirk (bool on) { rope_quirk_ = on; }
+  // true: scores, softmax and P V run as the three operators of the reference
+  // (probabilities rounded to fp16 one by one, multiheadattention_v2.cpp:272-317)
+  // instead of the one-launch attention with its running maximum
+  void set_operator_attention (bool on) { operator_attention_ = on; }
 
   // the next call only: the residual is added in the output projection's launch
   void set_residual (const Tensor *r) noexcept { residual_ = r; }
@@ -78,6 +82,7 @@ private:
   Tensor attn_out_;     // [1, S, heads*dim] of the one-launch attention
   OpTimer attn_timer_;
   bool attn_fused_last_ = false;
+  bool operator_attention_ = false;
 };
 }
 #endif
