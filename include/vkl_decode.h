@@ -62,7 +62,23 @@ typedef struct
   int wait_test;       /* testing aid: the workgroups that others wait for
                           never raise their flags, so every such wait gives
                           up */
+  void *flags;         /* from vkl_decode_flags_acquire: the flags that
+                          workgroups poll inside a launch.  Null: no launch
+                          waits (mode 1 and the attention + Wo launch run as
+                          the launches per phase) */
 } vkl_decode_model;
+
+/* The flags that the workgroups of a launch raise for one another live in
+ * device memory that no cache holds: they are polled through the scalar memory
+ * path, which the weight requests of a compute unit do not queue in, and a
+ * cached copy in the poller's L2 would hide the store of another XCD.  Such
+ * memory must never be freed once a kernel has read it (allocations made after
+ * the free have held wrong values on this GPU), so the library keeps a pool:
+ * acquire hands out a zeroed area of the current device (a new one only if
+ * none is free), release returns it to the pool.  One area per model.
+ * No counterpart in the reference. */
+int vkl_decode_flags_acquire (void **flags);
+void vkl_decode_flags_release (void *flags);
 
 /* bytes of device scratch a model of these dimensions needs */
 size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);

@@ -48,7 +48,7 @@ attn_split_min (const vkl_decode_model &m)
 // (each on a cache line of its own, clear of the words the persistent mode uses)
 constexpr int kSyncAttnDone = 32;
 constexpr int kSyncHeadDone = 64; // workgroups of the lm_head launch whose arg-max partials are in memory
-constexpr int kSyncAttnFlag = 768; // + 32 * slot
+constexpr int kAttnFlagGroup = 4;  // group of vkl_decode_model::flags, + 32 * slot
 constexpr int kFuseSpinLimit = 1 << 13; // some 10 ms; a head takes microseconds
 
 // the lm_head launch ends with the arg-max (not when a sampler follows it)
@@ -62,7 +62,12 @@ __device__ __forceinline__ void
 reset_attn_done (const Params &p, int wg)
 {
   if (wg == 0 && threadIdx.x < 9)
-    st_coherent_u32 (p.s.sync + (threadIdx.x == 8 ? kSyncAttnDone : kSyncAttnFlag + 32 * (int)threadIdx.x), 0u);
+    {
+      if (threadIdx.x == 8)
+        st_coherent_u32 (p.s.sync + kSyncAttnDone, 0u);
+      else if (p.m.flags)
+        st_coherent_u32 ((uint32_t *)p.m.flags + kAttnFlagGroup * kFlagGroupWords + 32 * (int)threadIdx.x, 0u);
+    }
 }
 
 
@@ -423,7 +428,7 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
           old = (uint32_t)__builtin_amdgcn_readfirstlane ((int)old);
           // (wait_test: a test of the bounded wait; the flags then stay unset)
           if (old + 1u == (uint32_t)nh && threadIdx.x < 8 && !m.wait_test)
-            st_coherent_u32 (p.s.sync + kSyncAttnFlag + 32 * (int)threadIdx.x, 1u);
+            st_coherent_u32 ((uint32_t *)m.flags + kAttnFlagGroup * kFlagGroupWords + 32 * (int)threadIdx.x, 1u);
         }
       return;
     }
@@ -442,12 +447,15 @@ decode_attn_wo_kernel (const Params p, const vkl_layer_weights lw, int layer, in
   uint32_t *seen = (uint32_t *)red + 2 * kDecWaves;
   if (threadIdx.x < 64)
     {
-      const uint32_t *flag = p.s.sync + kSyncAttnFlag + 32 * ((int)blockIdx.x & 7);
+      // (through the scalar memory path: a poll does not queue behind the two
+      // weight items this wave and its neighbours have just requested)
+      const uint32_t *flag
+          = (const uint32_t *)m.flags + kAttnFlagGroup * kFlagGroupWords + 32 * ((int)blockIdx.x & 7);
       bool ok = false;
       const int limit = m.wait_polls > 0 ? m.wait_polls : kFuseSpinLimit;
       for (int spin = 0; spin < limit; ++spin)
         {
-          if (ld_coherent_u32 (flag) != 0u)
+          if (flags_equal_scalar (flag, 1, 1u))
             {
               ok = true;
               break;
@@ -912,7 +920,7 @@ launch_attn_wo_xch (const Params &p, const vkl_layer_weights &lw, int layer, int
 bool
 attn_wo_fused (const Params &p, const vkl_decode_model *m, int G)
 {
-  return !m->separate_attn_wo && (int)p.pos + 1 < attn_split_min (*m)
+  return m->flags && !m->separate_attn_wo && (int)p.pos + 1 < attn_split_min (*m)
          && G >= 4 * m->n_heads && m->dim <= 8192 && (m->dim % 8) == 0;
 }
 
@@ -1149,6 +1157,53 @@ vkl_decode_step (const vkl_decode_model *m, const uint32_t *tok, uint32_t pos,
   if (int e = timer_collect (s))
     return e;
   return vkl_launch_status ();
+}
+
+namespace
+{
+std::mutex g_flags_mu;
+std::vector<void *> g_flags_free[16]; // per device: areas handed back (never freed)
+std::vector<std::pair<void *, int> > g_flags_out; // areas in use and their device
+}
+
+extern "C" int
+vkl_decode_flags_acquire (void **flags)
+{
+  VKL_CHECK_ARG (flags != nullptr);
+  *flags = nullptr;
+  int dev = 0;
+  VKL_HIP (hipGetDevice (&dev));
+  VKL_CHECK_ARG (dev >= 0 && dev < 16);
+  std::lock_guard<std::mutex> lock (g_flags_mu);
+  void *q = nullptr;
+  if (!g_flags_free[dev].empty ())
+    q = g_flags_free[dev].back (), g_flags_free[dev].pop_back ();
+  else
+    VKL_HIP (hipExtMallocWithFlags (&q, kFlagBytes, hipDeviceMallocUncached));
+  const hipError_t e = hipMemset (q, 0, kFlagBytes);
+  if (e != hipSuccess)
+    {
+      g_flags_free[dev].push_back (q);
+      return (int)e;
+    }
+  g_flags_out.push_back ({ q, dev });
+  *flags = q;
+  return 0;
+}
+
+extern "C" void
+vkl_decode_flags_release (void *flags)
+{
+  if (!flags)
+    return;
+  std::lock_guard<std::mutex> lock (g_flags_mu);
+  for (size_t i = 0; i < g_flags_out.size (); ++i)
+    if (g_flags_out[i].first == flags)
+      {
+        g_flags_free[g_flags_out[i].second].push_back (flags);
+        g_flags_out.erase (g_flags_out.begin () + (long)i);
+        return;
+      }
 }
 
 extern "C" int

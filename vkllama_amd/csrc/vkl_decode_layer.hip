@@ -54,8 +54,9 @@ namespace
 // 128-byte line of its own
 constexpr int kLsLaunch = 0;              // launches completed so far
 constexpr int kLsCnt = 32;                // + (stage * 8 + slot) * 32
-constexpr int kLsFlag = 32 + 4 * 8 * 32;  // + (stage * 8 + slot) * 32
-constexpr int kLsTicket = kLsFlag + 4 * 8 * 32; // + slot * 32: workgroups of the XCD that have started
+constexpr int kLsTicket = kLsCnt + 4 * 8 * 32; // + slot * 32: workgroups of the XCD that have started
+// (the flags, (stage * 8 + slot) * 32 words into vkl_decode_model::flags, are
+// polled through the scalar memory path and live in memory no cache holds)
 static_assert ((kLsTicket + 8 * 32) * 4 <= kLayerSyncBytes, "layer-sync area too small");
 constexpr int kSyncErr = 1; // word of Scratch::sync: a wait gave up
 constexpr int kLayerSpinLimit = 1 << 14;
@@ -161,11 +162,9 @@ courier_fetch (bool poll, const uint32_t *flag, int nflags, uint32_t mark, int l
       bool ok = !poll;
       if (poll)
         {
-          const uint32_t *f = flag + 32 * (lane & (nflags - 1));
           for (int spin = 0; spin < limit; ++spin)
             {
-              const bool up = ld_coherent_u32 (f) == mark;
-              if (__builtin_amdgcn_ballot_w64 (!up) == 0)
+              if (flags_equal_scalar (flag, nflags, mark))
                 {
                   ok = true;
                   break;
@@ -210,12 +209,10 @@ wait_flags (const uint32_t *flag, int nflags, uint32_t mark, int limit, uint32_t
 {
   if (threadIdx.x < 64)
     {
-      const uint32_t *f = flag + 32 * ((int)threadIdx.x & (nflags - 1));
       bool ok = false;
       for (int spin = 0; spin < limit; ++spin)
         {
-          const bool up = ld_coherent_u32 (f) == mark;
-          if (__builtin_amdgcn_ballot_w64 (!up) == 0)
+          if (flags_equal_scalar (flag, nflags, mark))
             {
               ok = true;
               break;
@@ -262,7 +259,7 @@ row_from_lds (const uint16_t *xl, int K, XRegs &x)
 
 struct LayerCtx
 {
-  uint32_t *ls, *err, *word;
+  uint32_t *ls, *err, *word, *flags;
   uint32_t mark;
   int limit, n_slot, slot, idx, nh, wg, G, layer;
   bool silent;
@@ -277,7 +274,7 @@ cnt_of (const LayerCtx &c, int stage, int k)
 __device__ __forceinline__ uint32_t *
 flag_of (const LayerCtx &c, int stage, int k)
 {
-  return c.ls + kLsFlag + (stage * 8 + k) * 32;
+  return c.flags + (stage * 8 + k) * 32;
 }
 
 #ifdef VKL_TRACE
@@ -496,7 +493,7 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
     GV2::run (ps, A, B, xl, e, red);
     VKL_TL (2)
     arrive (ls + kLsCnt + (ST_KQV * 8 + slot) * 32, (uint32_t)n_slot,
-            ls + kLsFlag + (ST_KQV * 8 + slot) * 32, 1, mark, false);
+            (uint32_t *)m.flags + (ST_KQV * 8 + slot) * 32, 1, mark, false);
     VKL_TL (3)
   }
 #ifdef VKL_TRACE
@@ -506,7 +503,7 @@ decode_layer_kernel (const Params p, const vkl_layer_weights lw, int layer, int 
       p.trace[((size_t)layer * 1024 + wg) * 16 + 14] = (unsigned)idx | (unsigned)slot << 16;
     }
 #endif
-  const LayerCtx c = { ls, err, word, mark, limit, n_slot, slot, idx, nh, wg, G, layer, silent };
+  const LayerCtx c = { ls, err, word, (uint32_t *)m.flags, mark, limit, n_slot, slot, idx, nh, wg, G, layer, silent };
   // the courier's path is a copy of the workers' (the branch is wave-uniform):
   // in one copy, with the courier's weight requests under a condition, the
   // item buffers of the two roles collide and spill
@@ -572,7 +569,7 @@ layer_launch_supported (const vkl_decode_model &m, int G)
 {
   // rows of up to two (dim) and four (ffn) chunks of 4096; every slot needs
   // workgroups beside the heads; two workgroups per compute unit must fit
-  return m.dim <= 8192 && m.ffn <= 16384 && (m.dim % 8) == 0 && (m.ffn % 8) == 0
+  return m.flags != nullptr && m.dim <= 8192 && m.ffn <= 16384 && (m.dim % 8) == 0 && (m.ffn % 8) == 0
          && G >= m.n_heads + 8 && (G % 8) == 0
          && 2 * (lds_bytes_needed (m.dim, m.ffn, m.maxlen, m.head_dim) + 32) <= 160 * 1024;
 }

@@ -527,6 +527,45 @@ final_argmax (const Params &p, int G, uint8_t *lds)
   return bi[kDecWaves];
 }
 
+// Flags of vkl_decode_model::flags: five groups of eight (one per XCD), every
+// flag on a 128-byte line of its own; groups 0..3 are the stages of the layer
+// launch, group 4 belongs to the attention + Wo launch.
+constexpr int kFlagGroupWords = 8 * 32;
+constexpr int kFlagGroups = 5;
+constexpr size_t kFlagBytes = (size_t)kFlagGroups * kFlagGroupWords * 4;
+
+// One look at `nflags` flags (1 or 8, 32 words apart) through the scalar
+// memory path (reads only; glc: past the scalar cache).  True: all equal `want`.
+__device__ __forceinline__ bool
+flags_equal_scalar (const uint32_t *flag, int nflags, uint32_t want)
+{
+  const uint64_t a = (uint64_t)flag;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane ((int)(uint32_t)a);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane ((int)(uint32_t)(a >> 32));
+  const uint64_t base = ((uint64_t)hi << 32) | lo;
+  if (nflags == 1)
+    {
+      uint32_t v;
+      asm volatile("s_load_dword %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(base) : "memory");
+      return v == want;
+    }
+  uint32_t v0, v1, v2, v3, v4, v5, v6, v7;
+  asm volatile("s_load_dword %0, %8, 0x0 glc\n\t"
+               "s_load_dword %1, %8, 0x80 glc\n\t"
+               "s_load_dword %2, %8, 0x100 glc\n\t"
+               "s_load_dword %3, %8, 0x180 glc\n\t"
+               "s_load_dword %4, %8, 0x200 glc\n\t"
+               "s_load_dword %5, %8, 0x280 glc\n\t"
+               "s_load_dword %6, %8, 0x300 glc\n\t"
+               "s_load_dword %7, %8, 0x380 glc\n\t"
+               "s_waitcnt lgkmcnt(0)"
+               : "=&s"(v0), "=&s"(v1), "=&s"(v2), "=&s"(v3), "=&s"(v4), "=&s"(v5), "=&s"(v6), "=&s"(v7)
+               : "s"(base)
+               : "memory");
+  return v0 == want && v1 == want && v2 == want && v3 == want && v4 == want && v5 == want
+         && v6 == want && v7 == want;
+}
+
 // One layer of the step as a single launch (vkl_decode_layer.hip): K/Q/V,
 // attention with one workgroup per head, Wo, up/gate, down.  G workgroups that
 // must all be resident at once.

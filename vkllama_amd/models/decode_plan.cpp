@@ -25,7 +25,11 @@ DecodePlan::DecodePlan ()
   memset (&desc_, 0, sizeof (desc_));
 }
 
-DecodePlan::~DecodePlan () {}
+DecodePlan::~DecodePlan ()
+{
+  // (back to the library's pool: memory of that kind is never freed)
+  vkl_decode_flags_release (desc_.flags);
+}
 
 absl::Status
 DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
@@ -135,6 +139,7 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
       "clearing decode scratch",
       vkl_memset (scratch_.data (), 0, sbytes, gpu->stream ())));
   desc_.scratch = scratch_.data ();
+  VKLLAMA_STATUS_OK (hip_status ("flags of the decode launches", vkl_decode_flags_acquire (&desc_.flags)));
   usable_ = true;
   return absl::OkStatus ();
 }
