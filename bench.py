@@ -47,7 +47,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE, calibrated against a copy kernel), keyed by (workload, phase);
 # filled in from the counter runs whose summaries are kept under profiles/
 TRAFFIC = {("llama2-7b-q8_0", "upgate"): (96197201, "profiles/decode_phase_kernels_llama2-7b-q8_0_hbm_traffic.txt"),
-           ("llama2-7b-q8_0", "layer"): (218655437, "profiles/decode_layer_kernel_llama2-7b-q8_0_hbm_traffic.txt")}
+           ("llama2-7b-q8_0", "layer"): (218700083, "profiles/decode_layer_kernel_llama2-7b-q8_0_hbm_traffic.txt")}
 
 
 def cpu_baseline(cfg, weights, n_tokens, gpu_model=None, n_parity=16):
