@@ -139,7 +139,9 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
       "clearing decode scratch",
       vkl_memset (scratch_.data (), 0, sbytes, gpu->stream ())));
   desc_.scratch = scratch_.data ();
-  VKLLAMA_STATUS_OK (hip_status ("flags of the decode launches", vkl_decode_flags_acquire (&desc_.flags)));
+  // (without such memory no launch waits: the step runs its launches per phase)
+  if (vkl_decode_flags_acquire (&desc_.flags) != 0)
+    desc_.flags = nullptr;
   usable_ = true;
   return absl::OkStatus ();
 }
