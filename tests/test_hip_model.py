@@ -218,6 +218,35 @@ def test_fp16_weights_model(fused):
     m.close()
 
 
+def test_decode_flag_areas_are_pooled(dev):
+    """vkl_decode_flags_acquire / release: the flags that workgroups poll inside
+    a launch live in device memory that no cache holds, which must never be
+    freed; the library hands areas out of a pool, zeroed, and takes them back.
+    A model holds one while it lives."""
+    import ctypes as C
+    from vkllama_amd import capi
+    raw = C.CDLL(capi.HIP_LIB_PATH)
+    raw.vkl_decode_flags_acquire.argtypes = [C.POINTER(C.c_void_p)]
+    raw.vkl_decode_flags_acquire.restype = C.c_int
+    raw.vkl_decode_flags_release.argtypes = [C.c_void_p]
+    raw.vkl_decode_flags_release.restype = None
+    a, b = C.c_void_p(), C.c_void_p()
+    assert raw.vkl_decode_flags_acquire(C.byref(a)) == 0 and a.value
+    assert raw.vkl_decode_flags_acquire(C.byref(b)) == 0 and b.value and b.value != a.value
+    raw.vkl_decode_flags_release(a)
+    cfg = dict(SMALL, n_layers=1)
+    m = M.Llama2(cfg, M.synth_weights(cfg, seed=2))      # takes the area just handed back
+    c = C.c_void_p()
+    assert raw.vkl_decode_flags_acquire(C.byref(c)) == 0 and c.value not in (a.value, b.value)
+    m.close()
+    d = C.c_void_p()
+    assert raw.vkl_decode_flags_acquire(C.byref(d)) == 0 and d.value == a.value   # the model's, back in the pool
+    for q in (b, c, d):
+        raw.vkl_decode_flags_release(q)
+    raw.vkl_decode_flags_release(None)                    # a no-op
+    assert raw.vkl_decode_flags_acquire(None) != 0
+
+
 def test_operator_attention_option(small):
     """Option "operator_attention": the attention of a prompt pass as the
     reference's three operators (scores, masked softmax with probabilities
