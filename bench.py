@@ -174,8 +174,9 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="llama2-7b-q8_0", choices=sorted(WORKLOADS) + ["matmul-q8_0-4096"])
-    ap.add_argument("--decode-mode", type=int, default=1, choices=(0, 1),
-                    help="1: one launch per layer (contexts below the split-attention length), 0: one launch per phase")
+    ap.add_argument("--decode-mode", type=int, default=-1, choices=(-1, 0, 1),
+                    help="1: one launch per layer (contexts below the split-attention length), 0: one launch per phase, "
+                         "-1: the library's default for the model's shape")
     ap.add_argument("--decode-graph", type=int, default=1, choices=(0, 1),
                     help="1: the decode loop is replayed from a captured HIP graph; 0: the same launches step by step "
                          "(for runs under a kernel tracer, which does not survive graph launches here)")
@@ -209,7 +210,8 @@ def main():
 
     t0 = time.perf_counter()
     m = M.Llama2(cfg, weights)
-    m.set_option("decode_mode", args.decode_mode)
+    if args.decode_mode >= 0:
+        m.set_option("decode_mode", args.decode_mode)
     m.set_option("decode_graph", args.decode_graph)
     t_load = time.perf_counter() - t0
 

@@ -80,6 +80,16 @@ typedef struct
 int vkl_decode_flags_acquire (void **flags);
 void vkl_decode_flags_release (void *flags);
 
+/* The launch form (the `mode` of vkl_decode_step and vkl_decode_loop) that
+ * measured faster for this model's shape on the MI355X: 1, one launch per
+ * layer, for rows of at most 4096 (dim) and 12288 (ffn) values when the model
+ * has its flag area (7B shape: 8 % faster with Q8_0 weights, 3 % with FP16);
+ * 0, one launch per phase, for wider rows (13B shape: the layer launch keeps
+ * twice the row in registers, spills, and runs 7 % slower) and without flags.
+ * Either value may be passed for any model that the form supports.
+ * No counterpart in the reference. */
+int vkl_decode_default_mode (const vkl_decode_model *m);
+
 /* bytes of device scratch a model of these dimensions needs */
 size_t vkl_decode_scratch_bytes (const vkl_decode_model *m);
 

@@ -72,7 +72,8 @@ int vkl_model_generate_sampled (vkl_model *m, const uint32_t *prompt_h,
                                 uint32_t *out_ids_h, double *prefill_ms,
                                 double *decode_ms);
 /* options, all per model: "fused_decode" (fused one-token decode on/off),
- * "decode_mode" (0 = one launch per phase, 1 = one launch per layer),
+ * "decode_mode" (0 = one launch per phase, 1 = one launch per layer; the
+ * default is what vkl_decode_default_mode says for the model's shape),
  * "decode_graph" (replay of the greedy loop from a HIP graph on/off),
  * "attn_split_min" (the context length from which attention is split over
  * several workgroups per head), "fuse_attn_wo" (mode 0: attention and the Wo

@@ -9,6 +9,7 @@
 //   test_host_classes --cpu   host-only checks (no device is touched)
 //   test_host_classes         everything (needs a GPU)
 // Exit status 0 when every check passed.
+#include "vkl_decode.h"
 #include "src/core/command.h"
 #include "src/core/float.h"
 #include "src/core/gpu_device.h"
@@ -225,6 +226,24 @@ test_cpu_float_and_quants ()
   y[3] = -2.54f, y[4] = 0.01f; // 0.01 * 127 / 2.54 = 0.5 -> 1
   CHECK (qint8_0_quantize_row (y.data (), raw.data (), 32).ok ());
   CHECK (raw[2 + 3] == -127 && raw[2 + 4] == 1 && raw[2 + 5] == 0);
+}
+
+// the launch form a model's decode steps take when nobody chooses one
+void
+test_cpu_default_decode_mode ()
+{
+  vkl_decode_model d;
+  memset (&d, 0, sizeof (d));
+  int area = 0;
+  d.dim = 4096, d.ffn = 11008, d.flags = &area;
+  CHECK (vkl_decode_default_mode (&d) == 1); // 7B rows: one launch per layer
+  d.flags = nullptr;
+  CHECK (vkl_decode_default_mode (&d) == 0); // nothing to wait on: launches per phase
+  d.flags = &area, d.dim = 5120, d.ffn = 13824;
+  CHECK (vkl_decode_default_mode (&d) == 0); // 13B rows measured slower in one launch
+  d.dim = 256, d.ffn = 704;
+  CHECK (vkl_decode_default_mode (&d) == 1);
+  CHECK (vkl_decode_default_mode (nullptr) == 0);
 }
 
 void
@@ -930,6 +949,7 @@ main (int argc, char **argv)
   const bool cpu_only = argc > 1 && !strcmp (argv[1], "--cpu");
   test_cpu_float_and_quants ();
   test_cpu_tensor_shapes ();
+  test_cpu_default_decode_mode ();
   if (!cpu_only)
     run_gpu ();
   printf ("%s: %d checks, %d failed\n", cpu_only ? "host-only" : "all", g_checks,

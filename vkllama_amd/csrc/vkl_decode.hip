@@ -1191,6 +1191,15 @@ vkl_decode_flags_acquire (void **flags)
   return 0;
 }
 
+extern "C" int
+vkl_decode_default_mode (const vkl_decode_model *m)
+{
+  // (measured at short contexts, greedy loop replayed from a graph, 8-10
+  // layers of each shape: 7B Q8_0 53.2 against 57.4 us per layer, 7B FP16
+  // 80.6 against 83.4, 13B Q8_0 85.0 against 79.5)
+  return m && m->flags && m->dim <= 4096 && m->ffn <= 12288 ? 1 : 0;
+}
+
 extern "C" void
 vkl_decode_flags_release (void *flags)
 {

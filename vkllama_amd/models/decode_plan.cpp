@@ -142,6 +142,8 @@ DecodePlan::build (Model &model, GPUDevice *gpu, InputLayer *in,
   // (without such memory no launch waits: the step runs its launches per phase)
   if (vkl_decode_flags_acquire (&desc_.flags) != 0)
     desc_.flags = nullptr;
+  // (the form that measured faster for this shape; set_mode overrides it)
+  mode_ = vkl_decode_default_mode (&desc_);
   usable_ = true;
   return absl::OkStatus ();
 }
